@@ -1,0 +1,163 @@
+/*
+ * pf8.h -- C ABI of libpf8.so: MI355X (gfx950) kernels for the PaddleFormers FP8 block-quant /
+ * block-scaled GEMM path.
+ *
+ * Every entry point replaces one third-party operator the reference resolves at call time
+ * (paddle.incubate.nn.functional.* and paddlefleet_ops.deep_gemm.*); the comment on each
+ * declaration cites the reference call site (paths relative to the PaddleFormers checkout).
+ *
+ * Conventions
+ *   - plain pointers to DEVICE memory and sizes; no framework types.  bf16 = uint16_t bit pattern,
+ *     e4m3 = uint8_t OCP float8_e4m3fn code, scales = float (decode scale: x ~= q * s).
+ *   - every function returns 0 on success or a negative PF8_E* code; pf8_last_error() gives the
+ *     thread-local message.  Nothing throws, nothing allocates device memory, nothing synchronises.
+ *   - `stream` is a hipStream_t (NULL = the null stream).  Launches are asynchronous.
+ *   - zero-sized problems are legal and return 0 without launching (the reference short-circuits
+ *     them: transformers/fp8_utils.py:185,202,308,945,998,1208,1256).
+ *   - scale_layout: 0 = row-major [rows, K/128] (output_scale_transpose=False),
+ *                   1 = [K/128, rows]          (output_scale_transpose=True, the layout the GEMMs
+ *                       consume as `.T`, transformers/fp8_utils.py:278,941).
+ *   - pow2: 0 = s = amax/448 (cli/train/deepseek_v3_pretrain/kernel.py:44);
+ *           1 = s rounded up to a power of two (utils/upcast_downcast_triton.py:71-85).
+ *     An all-zero tile gets s = 1 and zero bytes.
+ *   - all base pointers must be 16-byte aligned; K (the quantised axis) must be a multiple of 128.
+ */
+#ifndef PF8_H
+#define PF8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PF8_OK 0
+#define PF8_EINVAL (-1)    /* bad shape, alignment, flag or null pointer */
+#define PF8_ELAUNCH (-2)   /* HIP reported an error at launch */
+#define PF8_ENODEV (-3)    /* no gfx950 device / wrong architecture */
+
+typedef void* pf8_stream_t; /* hipStream_t */
+
+int pf8_version(void);
+const char* pf8_last_error(void);
+
+/* deep_gemm.set_num_sms(get_sm_num()) -- transformers/fp8_utils.py:42,54-55,277: caps the number of
+ * compute units the GEMM grids are sized for (0 = all).  Returns the previous value. */
+int pf8_set_num_cus(int n);
+int pf8_get_num_cus(void);
+
+/* fp8_quant_blockwise(x, quant_method="1x128", input_transpose=False, output_scale_transpose=...)
+ * transformers/fp8_utils.py:262-268, 938-941; cli/train/deepseek_v3_pretrain/kernel.py:29-70.
+ * x bf16 [M,K] with row stride ldx (elements) -> q [M,K], s per scale_layout. */
+int pf8_quant_1x128(const uint16_t* x, int64_t M, int64_t K, int64_t ldx, uint8_t* q, float* s,
+                    int scale_layout, int pow2, pf8_stream_t stream);
+
+/* fp8_quant_blockwise(w, quant_method="128x128", output_scale_transpose=False, input_transpose=...,
+ * return_transpose_only=...) -- transformers/fp8_utils.py:105-131, 628-665.
+ * w bf16 [R,C] -> q [R,C], s [R/128,C/128] and/or q_t [C,R], s_t [C/128,R/128]; either pair may be
+ * NULL (return_transpose_only=True passes q = s = NULL). */
+int pf8_quant_128x128(const uint16_t* w, int64_t R, int64_t C, uint8_t* q, float* s, uint8_t* q_t,
+                      float* s_t, int pow2, pf8_stream_t stream);
+
+/* fp8_quant_blockwise(x, quant_method="1x128", input_transpose=True[, return_transpose_only=True])
+ * transformers/fp8_utils.py:155-174, 380-382, 585-587, 725-727: one pass that emits the row-scaled
+ * copy q [M,K] (+ s) and the column-scaled transposed copy q_t [K,M] (+ s_t: layout 1 ->
+ * [M/128,K], layout 0 -> [K,M/128]).  M and K multiples of 128.  q = s = NULL skips the row copy. */
+int pf8_quant_transpose(const uint16_t* x, int64_t M, int64_t K, uint8_t* q, float* s, uint8_t* q_t,
+                        float* s_t, int scale_layout, int pow2, pf8_stream_t stream);
+
+/* fused_stack_transpose_quant(weight_list, transpose) -- transformers/fp8_utils.py:91-102;
+ * un-fused definition ernie token_dispatcher/fp8_utils.py:276-287.  w_list is a HOST array of E
+ * device pointers to bf16 [R,C] weights.  transpose=0: q [E*R, C], s [E*R/128, C/128];
+ * transpose=1: q [E*C, R], s [E*C/128, R/128]. */
+int pf8_stack_transpose_quant(const uint16_t* const* w_list, int E, int64_t R, int64_t C,
+                              int transpose, uint8_t* q, float* s, int pow2, pf8_stream_t stream);
+
+/* fused_weighted_swiglu_act_quant(o1, probs, using_pow2_scaling) -- transformers/fp8_utils.py:981-987;
+ * un-fused definition ernie token_dispatcher/fp8_utils.py:996-1004.  o1 bf16 [M,2I] (gate first),
+ * probs fp32 [M] or NULL -> q [M,I], s per scale_layout.  o2 (bf16 [M,I]) optionally receives the
+ * pre-quant activations (NULL to skip). */
+int pf8_swiglu_weighted_quant(const uint16_t* o1, const float* probs, int64_t M, int64_t I,
+                              uint8_t* q, float* s, uint16_t* o2, int scale_layout, int pow2,
+                              pf8_stream_t stream);
+
+/* fused_transpose_split_quant(x, scale, tokens_per_expert, pow_2_scales) --
+ * transformers/fp8_utils.py:1096-1100; un-fused definition ernie token_dispatcher/fp8_utils.py:1199-1210.
+ * x: bf16 [Mtot,K] (x_is_fp8=0) or e4m3 [Mtot,K] with fp32 scales xs (x_is_fp8=1; xs_layout 0 =
+ * [Mtot,K/128] row-major, 1 = [K/128,Mtot] -- the cached input_scale of the MoE node is the latter).
+ * rows_per_expert: HOST array of E counts, each a multiple of 128, summing to Mtot.
+ * Outputs are packed: expert e's q_t [K, M_e] starts at q_t + K*off_e and its s_t [M_e/128, K] at
+ * s_t + (off_e/128)*K, off_e = rows of the experts before e. */
+int pf8_transpose_split_quant(const void* x, const float* xs, int x_is_fp8, int xs_layout,
+                              const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q_t, float* s_t,
+                              int pow2, pf8_stream_t stream);
+
+/* fused_act_dequant(q, s) -- transformers/fp8_utils.py:136-138, 779.  1x128 dequant to bf16. */
+int pf8_act_dequant(const uint8_t* q, const float* s, int scale_layout, int64_t M, int64_t K,
+                    uint16_t* out, pf8_stream_t stream);
+
+/* weight_dequant(x, s) -- cli/train/deepseek_v3_pretrain/kernel.py:73-118;
+ * quantization/checkpoint_dequant.py:148-174,277-292.  128x128 dequant to bf16; R and C arbitrary
+ * (s is [ceil(R/128), ceil(C/128)], trailing partial blocks cropped). */
+int pf8_weight_dequant(const uint8_t* q, const float* s, int64_t R, int64_t C, uint16_t* out,
+                       pf8_stream_t stream);
+
+/* fused_swiglu_weighted_bwd(o1, do2_s, probs) -- transformers/fp8_utils.py:1049-1052; un-fused
+ * definition ernie token_dispatcher/fp8_utils.py:1088-1092.  -> do1 bf16 [M,2I], probs_grad fp32 [M],
+ * o2_s bf16 [M,I]. */
+int pf8_swiglu_weighted_bwd(const uint16_t* o1, const uint16_t* do2_s, const float* probs, int64_t M,
+                            int64_t I, uint16_t* do1, float* probs_grad, uint16_t* o2_s,
+                            pf8_stream_t stream);
+
+/* deep_gemm.fp8_gemm_nt((a, sa), (b, sb), out) -- transformers/fp8_utils.py:278, 368;
+ * cli/train/deepseek_v3_pretrain/kernel.py:129-220.  a e4m3 [M,K], sa per sa_layout, b e4m3 [N,K],
+ * sb fp32 [ceil(N/128), K/128] -> out bf16 [M,N] (row stride ldo elements). */
+int pf8_gemm_nt(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b, const float* sb,
+                int64_t M, int64_t N, int64_t K, uint16_t* out, int64_t ldo, pf8_stream_t stream);
+
+/* fp8_gemm_blockwise(..., is_a_1d_scaled=True, is_b_1d_scaled=True) / deep_gemm.fp8_gemm_nt(...,
+ * recipe=(1,1,128)) -- transformers/fp8_utils.py:176-221 (kitchen_gemm).  Weight-gradient GEMM:
+ * out[Kin,N] (+)= a_t[Kin,M] . b_t[N,M]^T, a_t/b_t e4m3, sa_t fp32 [M/128,Kin], sb_t fp32 [M/128,N],
+ * out fp32, accumulate != 0 adds to the existing contents.  M multiple of 128. */
+int pf8_gemm_nt_1d1d_f32(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t,
+                         int64_t Kin, int64_t N, int64_t M, float* out, int accumulate,
+                         pf8_stream_t stream);
+
+/* deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa), (b, sb), out, m_indices) --
+ * transformers/fp8_utils.py:906-911, 949-954, 1002-1007, 1042-1047, 1087-1092.  a [Mtot,K] rows sorted
+ * by expert, every expert segment a multiple of 128 rows; b [E,N,K]; sb [E,ceil(N/128),K/128];
+ * m_indices DEVICE int32 [Mtot] (expert of each row; negative = skip the 128-row tile).
+ * Mtot multiple of 128. */
+int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b,
+                                   const float* sb, int E, int64_t Mtot, int64_t N, int64_t K,
+                                   const int32_t* m_indices, uint16_t* out, pf8_stream_t stream);
+
+/* deep_gemm.m_grouped_fp8_gemm_nt_masked((a, sa), (b, sb), out, masked_m, expected_m) --
+ * ernie token_dispatcher/fp8_utils.py:227-233.  a [E,Mmax,K], sa [E,Mmax,K/128] row-major,
+ * b [E,N,K], sb [E,ceil(N/128),K/128], masked_m DEVICE int32 [E] valid rows -> out [E,Mmax,N];
+ * rows >= masked_m[e] are not written. */
+int pf8_grouped_gemm_nt_masked(const uint8_t* a, const float* sa, const uint8_t* b, const float* sb,
+                               int E, int64_t Mmax, int64_t N, int64_t K, const int32_t* masked_m,
+                               int expected_m, uint16_t* out, pf8_stream_t stream);
+
+/* Per-expert weight-gradient loop -- transformers/fp8_utils.py:1102-1134 (bwd_down_weight),
+ * 1136-1189 (bwd_gate_up_weight): for each expert e with rows_per_expert[e] > 0,
+ * out[e] [Kin,N] (+)= a_t[e] . b_t[e]^T as in pf8_gemm_nt_1d1d_f32, in ONE launch.  a_t/sa_t and
+ * b_t/sb_t use the packed layout written by pf8_transpose_split_quant; out is fp32 [E,Kin,N].
+ * rows_per_expert is a HOST array (E <= 256). */
+int pf8_grouped_wgrad(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t,
+                      const int64_t* rows_per_expert, int E, int64_t Kin, int64_t N, float* out,
+                      int accumulate, pf8_stream_t stream);
+
+/* Self-test hook used by the GPU tests: converts n floats to e4m3 with the same device routine the
+ * quantizers use (hardware OCP convert), so the codec can be swept exhaustively. */
+int pf8_debug_encode(const float* v, int64_t n, uint8_t* out, pf8_stream_t stream);
+/* Self-test hook: q[i] = e4m3(x[i] / s[i]) through the quantizers' fast-division path. */
+int pf8_debug_div_encode(const float* x, const float* s, int64_t n, uint8_t* out, pf8_stream_t stream);
+/* Self-test hook: out[i] = silu(x[i]) with the device restatement of the oracle's expf. */
+int pf8_debug_silu(const float* x, int64_t n, float* out, pf8_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PF8_H */

@@ -1,0 +1,333 @@
+"""ctypes front end of the CPU oracle (libpf8_oracle.so) on numpy arrays.
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, the smoke check and the CPU-baseline leg of the
+benchmark.  The product package never imports it.
+
+bf16 tensors are numpy uint16 bit patterns, e4m3 tensors are numpy uint8 codes, scales float32.
+Each wrapper names the C function it calls; the reference citations live in pf8_oracle.c.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libpf8_oracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (make -C oracle)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE] + (["-B"] if force else []), stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.pf8o_e4m3_decode.restype = C.c_float
+        _lib.pf8o_e4m3_decode.argtypes = [C.c_uint8]
+        _lib.pf8o_e4m3_encode.restype = C.c_uint8
+        _lib.pf8o_e4m3_encode.argtypes = [C.c_float]
+        _lib.pf8o_bf16_to_f32.restype = C.c_float
+        _lib.pf8o_bf16_to_f32.argtypes = [C.c_uint16]
+        _lib.pf8o_f32_to_bf16.restype = C.c_uint16
+        _lib.pf8o_f32_to_bf16.argtypes = [C.c_float]
+        _lib.pf8o_expf.restype = C.c_float
+        _lib.pf8o_expf.argtypes = [C.c_float]
+        _lib.pf8o_silu.restype = C.c_float
+        _lib.pf8o_silu.argtypes = [C.c_float]
+        _lib.pf8o_scale_from_amax.restype = C.c_float
+        _lib.pf8o_scale_from_amax.argtypes = [C.c_float, C.c_int]
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dt):
+    a = np.ascontiguousarray(a)
+    assert a.dtype == dt, (a.dtype, dt)
+    return a
+
+
+I64 = C.c_int64
+
+# ---------------------------------------------------------------------------------------------
+# numpy-side helpers (independent of the C code; used to cross-check it)
+# ---------------------------------------------------------------------------------------------
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit patterns, round-to-nearest-even (numpy restatement)."""
+    b = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = (b & 0x7FFFFFFF) > 0x7F800000
+    r = (b + 0x7FFF + ((b >> 16) & 1)) >> 16
+    r = np.where(nan, (b >> 16) | 0x40, r)
+    return r.astype(np.uint16)
+
+
+def bf16_bits_to_f32(h: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(h, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def e4m3_table() -> np.ndarray:
+    """The 256-entry decode table from the closed form (float64)."""
+    t = np.empty(256, dtype=np.float64)
+    for c in range(256):
+        e, m = (c >> 3) & 0xF, c & 7
+        if e == 0xF and m == 7:
+            v = np.nan
+        elif e == 0:
+            v = m * 2.0**-9
+        else:
+            v = (1 + m / 8.0) * 2.0 ** (e - 7)
+        t[c] = -v if c & 0x80 else v
+    return t
+
+
+def e4m3_decode_np(q: np.ndarray) -> np.ndarray:
+    return e4m3_table().astype(np.float32)[np.ascontiguousarray(q, dtype=np.uint8)]
+
+
+# ---------------------------------------------------------------------------------------------
+# scalar entry points
+# ---------------------------------------------------------------------------------------------
+
+
+def e4m3_decode(c: int) -> float:
+    return lib().pf8o_e4m3_decode(c)
+
+
+def e4m3_encode(v: float) -> int:
+    return lib().pf8o_e4m3_encode(float(v))
+
+
+def expf(x: float) -> float:
+    return lib().pf8o_expf(float(x))
+
+
+def silu(x: float) -> float:
+    return lib().pf8o_silu(float(x))
+
+
+def scale_from_amax(amax: float, pow2: bool = False) -> float:
+    return lib().pf8o_scale_from_amax(float(amax), int(pow2))
+
+
+def _array_fn(name, v, out_dtype):
+    flat = np.ascontiguousarray(v, dtype=np.float32).ravel()
+    out = np.empty(flat.size, out_dtype)
+    getattr(lib(), name)(_p(flat), I64(flat.size), _p(out))
+    return out.reshape(np.shape(v))
+
+
+def e4m3_encode_array(v):
+    return _array_fn("pf8o_e4m3_encode_array", v, np.uint8)
+
+
+def expf_array(v):
+    return _array_fn("pf8o_expf_array", v, np.float32)
+
+
+def silu_array(v):
+    return _array_fn("pf8o_silu_array", v, np.float32)
+
+
+def f32_to_bf16_array(v):
+    return _array_fn("pf8o_f32_to_bf16_array", v, np.uint16)
+
+
+def div_encode_array(x, s):
+    """e4m3_encode(x / s) element-wise with IEEE fp32 division."""
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    s = np.ascontiguousarray(s, dtype=np.float32).ravel()
+    out = np.empty(x.size, np.uint8)
+    lib().pf8o_div_encode_array(_p(x), _p(s), I64(x.size), _p(out))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# tensor entry points
+# ---------------------------------------------------------------------------------------------
+
+
+def quant_1x128(x, scale_layout=0, pow2=False):
+    """pf8o_quant_1x128: x uint16[M,K] -> (q uint8[M,K], s float32 [M,K/128] or [K/128,M])."""
+    x = _c(x, np.uint16)
+    M, K = x.shape
+    assert K % 128 == 0
+    q = np.empty((M, K), np.uint8)
+    s = np.empty((M, K // 128) if scale_layout == 0 else (K // 128, M), np.float32)
+    lib().pf8o_quant_1x128(_p(x), I64(M), I64(K), I64(K), _p(q), _p(s), int(scale_layout), int(pow2))
+    return q, s
+
+
+def quant_128x128(w, want=(True, False), pow2=False):
+    """pf8o_quant_128x128: returns (q, s, qt, st); entries not wanted are None."""
+    w = _c(w, np.uint16)
+    R, Cc = w.shape
+    assert R % 128 == 0 and Cc % 128 == 0
+    q = s = qt = st = None
+    if want[0]:
+        q, s = np.empty((R, Cc), np.uint8), np.empty((R // 128, Cc // 128), np.float32)
+    if want[1]:
+        qt, st = np.empty((Cc, R), np.uint8), np.empty((Cc // 128, R // 128), np.float32)
+    lib().pf8o_quant_128x128(_p(w), I64(R), I64(Cc), _p(q), _p(s), _p(qt), _p(st), int(pow2))
+    return q, s, qt, st
+
+
+def quant_transpose(x, scale_layout=1, pow2=False, want_row=True):
+    """pf8o_quant_transpose: (q[M,K], s, qt[K,M], st)."""
+    x = _c(x, np.uint16)
+    M, K = x.shape
+    assert M % 128 == 0 and K % 128 == 0
+    q = s = None
+    if want_row:
+        q = np.empty((M, K), np.uint8)
+        s = np.empty((K // 128, M) if scale_layout else (M, K // 128), np.float32)
+    qt = np.empty((K, M), np.uint8)
+    st = np.empty((M // 128, K) if scale_layout else (K, M // 128), np.float32)
+    lib().pf8o_quant_transpose(_p(x), I64(M), I64(K), _p(q), _p(s), _p(qt), _p(st), int(scale_layout), int(pow2))
+    return q, s, qt, st
+
+
+def stack_transpose_quant(w_list, transpose=False, pow2=False):
+    ws = [_c(w, np.uint16) for w in w_list]
+    E = len(ws)
+    R, Cc = ws[0].shape
+    ptrs = (C.c_void_p * E)(*[w.ctypes.data for w in ws])
+    if transpose:
+        q, s = np.empty((E * Cc, R), np.uint8), np.empty((E * Cc // 128, R // 128), np.float32)
+    else:
+        q, s = np.empty((E * R, Cc), np.uint8), np.empty((E * R // 128, Cc // 128), np.float32)
+    lib().pf8o_stack_transpose_quant(ptrs, int(E), I64(R), I64(Cc), int(transpose), _p(q), _p(s), int(pow2))
+    return q, s
+
+
+def swiglu_weighted_quant(o1, probs=None, scale_layout=0, pow2=False, return_o2=False):
+    o1 = _c(o1, np.uint16)
+    M, I2 = o1.shape
+    I = I2 // 2
+    assert I % 128 == 0
+    if probs is not None:
+        probs = _c(probs, np.float32)
+        assert probs.shape == (M,)
+    q = np.empty((M, I), np.uint8)
+    s = np.empty((M, I // 128) if scale_layout == 0 else (I // 128, M), np.float32)
+    o2 = np.empty((M, I), np.uint16)
+    lib().pf8o_swiglu_weighted_quant(_p(o1), _p(probs), I64(M), I64(I), _p(q), _p(s), int(scale_layout), int(pow2), _p(o2))
+    return (q, s, o2) if return_o2 else (q, s)
+
+
+def act_dequant(q, s, scale_layout=0):
+    q = _c(q, np.uint8)
+    s = _c(s, np.float32)
+    M, K = q.shape
+    out = np.empty((M, K), np.uint16)
+    lib().pf8o_act_dequant(_p(q), _p(s), int(scale_layout), I64(M), I64(K), _p(out))
+    return out
+
+
+def weight_dequant(q, s):
+    q = _c(q, np.uint8)
+    s = _c(s, np.float32)
+    R, Cc = q.shape
+    assert s.shape == ((R + 127) // 128, (Cc + 127) // 128)
+    out = np.empty((R, Cc), np.uint16)
+    lib().pf8o_weight_dequant(_p(q), _p(s), I64(R), I64(Cc), _p(out))
+    return out
+
+
+def transpose_split_quant(x, xs, rows, pow2=False, xs_layout=0):
+    """pf8o_transpose_split_quant -> (list of qt[e] [K,M_e], list of st[e] [M_e/128,K])."""
+    is_fp8 = x.dtype == np.uint8
+    x = np.ascontiguousarray(x)
+    Mtot, K = x.shape
+    rows = np.asarray(rows, dtype=np.int64)
+    assert rows.sum() == Mtot and (rows % 128 == 0).all()
+    if is_fp8:
+        xs = _c(xs, np.float32)
+        assert xs.shape == ((Mtot, K // 128) if xs_layout == 0 else (K // 128, Mtot))
+    qt = np.empty(K * Mtot, np.uint8)
+    st = np.empty((Mtot // 128) * K, np.float32)
+    lib().pf8o_transpose_split_quant(_p(x), _p(xs) if is_fp8 else None, int(is_fp8), int(xs_layout), _p(rows), int(len(rows)), I64(K),
+                                     _p(qt), _p(st), int(pow2))
+    qs, ss, off = [], [], 0
+    for r in rows:
+        r = int(r)
+        qs.append(qt[off * K:(off + r) * K].reshape(K, r))
+        ss.append(st[(off // 128) * K:((off + r) // 128) * K].reshape(r // 128, K))
+        off += r
+    return qs, ss
+
+
+def swiglu_weighted_bwd(o1, do2_s, probs):
+    o1, do2_s, probs = _c(o1, np.uint16), _c(do2_s, np.uint16), _c(probs, np.float32)
+    M, I2 = o1.shape
+    I = I2 // 2
+    do1 = np.empty((M, I2), np.uint16)
+    pg = np.empty((M,), np.float32)
+    o2s = np.empty((M, I), np.uint16)
+    lib().pf8o_swiglu_weighted_bwd(_p(o1), _p(do2_s), _p(probs), I64(M), I64(I), _p(do1), _p(pg), _p(o2s))
+    return do1, pg, o2s
+
+
+def gemm_nt(a, sa, b, sb, sa_layout=0, dequant_ref=False):
+    """pf8o_gemm_nt (block-scaled accumulation) or pf8o_gemm_nt_dequant_ref -> bf16 bits [M,N]."""
+    a, b, sa, sb = _c(a, np.uint8), _c(b, np.uint8), _c(sa, np.float32), _c(sb, np.float32)
+    M, K = a.shape
+    N = b.shape[0]
+    assert b.shape[1] == K and K % 128 == 0
+    assert sa.shape == ((M, K // 128) if sa_layout == 0 else (K // 128, M))
+    assert sb.shape == ((N + 127) // 128, K // 128)
+    out = np.empty((M, N), np.uint16)
+    fn = lib().pf8o_gemm_nt_dequant_ref if dequant_ref else lib().pf8o_gemm_nt
+    fn(_p(a), _p(sa), int(sa_layout), _p(b), _p(sb), I64(M), I64(N), I64(K), _p(out))
+    return out
+
+
+def gemm_nt_1d1d_f32(a_t, sa_t, b_t, sb_t, out=None):
+    a_t, b_t, sa_t, sb_t = _c(a_t, np.uint8), _c(b_t, np.uint8), _c(sa_t, np.float32), _c(sb_t, np.float32)
+    Kin, M = a_t.shape
+    N = b_t.shape[0]
+    assert b_t.shape[1] == M and M % 128 == 0
+    assert sa_t.shape == (M // 128, Kin) and sb_t.shape == (M // 128, N)
+    acc = out is not None
+    if out is None:
+        out = np.empty((Kin, N), np.float32)
+    else:
+        out = _c(out, np.float32).copy()
+    lib().pf8o_gemm_nt_1d1d_f32(_p(a_t), _p(sa_t), _p(b_t), _p(sb_t), I64(Kin), I64(N), I64(M), _p(out), int(acc))
+    return out
+
+
+def grouped_gemm_nt_contiguous(a, sa, b, sb, m_indices, sa_layout=0, out=None):
+    a, b, sa, sb = _c(a, np.uint8), _c(b, np.uint8), _c(sa, np.float32), _c(sb, np.float32)
+    m_indices = _c(m_indices, np.int32)
+    Mtot, K = a.shape
+    E, N, _ = b.shape
+    assert sb.shape == (E, (N + 127) // 128, K // 128)
+    out = np.zeros((Mtot, N), np.uint16) if out is None else out
+    lib().pf8o_grouped_gemm_nt_contiguous(_p(a), _p(sa), int(sa_layout), _p(b), _p(sb), int(E), I64(Mtot), I64(N), I64(K),
+                                          _p(m_indices), _p(out))
+    return out
+
+
+def grouped_gemm_nt_masked(a, sa, b, sb, masked_m, out=None):
+    a, b, sa, sb = _c(a, np.uint8), _c(b, np.uint8), _c(sa, np.float32), _c(sb, np.float32)
+    masked_m = _c(masked_m, np.int32)
+    E, Mmax, K = a.shape
+    N = b.shape[1]
+    out = np.zeros((E, Mmax, N), np.uint16) if out is None else out
+    lib().pf8o_grouped_gemm_nt_masked(_p(a), _p(sa), _p(b), _p(sb), int(E), I64(Mmax), I64(N), I64(K), _p(masked_m), _p(out))
+    return out

@@ -1,0 +1,187 @@
+// pf8_device.h -- device-side scalar helpers shared by the gfx950 kernels: bf16 unpack/round,
+// OCP e4m3 packing through the hardware converter, the 16-lane (one DPP row = one 1x128 tile)
+// amax reduction, the scale rule and the tile quantizer with its fast exact-division path.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pf8 {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// a dword holds two bf16: element 0 in the low half
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xFFFF0000u); }
+
+// two fp32 -> packed bf16 pair, round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+// one fp32 -> bf16 -> fp32 (the value a bf16 tensor would hold)
+__device__ __forceinline__ float round_bf16(float f) { return bf16_lo(pack_bf16(f, 0.0f)); }
+
+// unsigned max with the other operand fetched from a lane `ror` positions away inside the 16-lane
+// DPP row; magnitudes of non-NaN floats order like their bit patterns, so amax runs on integers
+// (no NaN-canonicalisation instructions in the way).
+template <int ROR>
+__device__ __forceinline__ uint32_t row_max_step(uint32_t v) {
+    uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x120 + ROR, 0xF, 0xF, false);
+    return v > o ? v : o;
+}
+// all 16 lanes of a DPP row end with the row maximum
+__device__ __forceinline__ uint32_t row16_max(uint32_t v) {
+    v = row_max_step<8>(v);
+    v = row_max_step<4>(v);
+    v = row_max_step<2>(v);
+    v = row_max_step<1>(v);
+    return v;
+}
+
+// 16-byte / 8-byte global accesses.  PF8_STREAMING=1 marks them non-temporal (streamed once).
+#ifndef PF8_STREAMING
+#define PF8_STREAMING 0
+#endif
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 ld16(const void* p) {
+#if PF8_STREAMING
+    u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+#else
+    u32x4 v = *reinterpret_cast<const u32x4*>(p);
+#endif
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st16(void* p, uint4 o) {
+    u32x4 v = {o.x, o.y, o.z, o.w};
+#if PF8_STREAMING
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+#else
+    *reinterpret_cast<u32x4*>(p) = v;
+#endif
+}
+__device__ __forceinline__ void st8(void* p, uint2 o) {
+    u32x2 v = {o.x, o.y};
+#if PF8_STREAMING
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+#else
+    *reinterpret_cast<u32x2*>(p) = v;
+#endif
+}
+
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+// element-wise max of the two 16-bit halves (v_pk_max_u16)
+__device__ __forceinline__ uint32_t pkmax_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
+
+// |.| bit patterns of the 8 bf16 in a 16-byte chunk, reduced to one fp32-positioned pattern
+__device__ __forceinline__ uint32_t amax_bits8(uint4 w) {
+    uint32_t m = pkmax_u16(pkmax_u16(w.x & 0x7FFF7FFFu, w.y & 0x7FFF7FFFu),
+                           pkmax_u16(w.z & 0x7FFF7FFFu, w.w & 0x7FFF7FFFu));
+    return umax(m << 16, m & 0xFFFF0000u);
+}
+
+struct TileScale {
+    float s;     // decode scale stored next to the bytes
+    float r;     // approximate reciprocal used by the fast path
+    bool slow;   // tile must take the IEEE division path (scale too small for a finite reciprocal)
+};
+
+// s = amax/448 (IEEE divide), amax == 0 -> 1; pow2: decode scale rounded up to a power of two.
+__device__ __forceinline__ TileScale make_scale(uint32_t amax_bits, bool pow2) {
+    TileScale t;
+    float amax = u2f(amax_bits);
+    float s = amax / 448.0f;
+    if (pow2) s = u2f((f2u(s) + 0x007FFFFFu) & 0x7F800000u);
+    if (amax_bits == 0u) s = 1.0f;
+    t.s = s;
+    t.r = __builtin_amdgcn_rcpf(s);
+    t.slow = !(s >= 1.0e-30f);
+    return t;
+}
+
+// two fp32 -> two e4m3 codes in the low / high half of a dword (hardware OCP convert, RNE)
+__device__ __forceinline__ uint32_t cvt_e4m3_lo(float a, float b, uint32_t old) {
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, false);
+}
+__device__ __forceinline__ uint32_t cvt_e4m3_hi(float a, float b, uint32_t old) {
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, true);
+}
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
+    return cvt_e4m3_hi(c, d, cvt_e4m3_lo(a, b, 0u));
+}
+
+// Quantise 8 values of one tile: bytes == e4m3_rne(v / s) with v / s the correctly rounded fp32
+// quotient.  Fast path: y = v * rcp(s) is within 4 ulp of that quotient; the e4m3 code can differ
+// only if a rounding boundary of the 3-bit mantissa grid (fp32 mantissa low 19 bits == 0, which
+// also covers the coarser subnormal grid) lies within that distance, so any element that close to a
+// boundary sends the lane through the exact division instead.
+__device__ __forceinline__ uint2 quant8(const float (&v)[8], const TileScale& t) {
+    float y[8];
+    bool redo = t.slow;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        y[i] = v[i] * t.r;
+        redo |= (((f2u(y[i]) + 8u) & 0x7FFFFu) <= 16u);
+    }
+    if (__builtin_expect(redo, 0)) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = v[i] / t.s;
+    }
+    uint2 o;
+    o.x = pack4_e4m3(y[0], y[1], y[2], y[3]);
+    o.y = pack4_e4m3(y[4], y[5], y[6], y[7]);
+    return o;
+}
+
+__device__ __forceinline__ void unpack8(uint4 w, float (&v)[8]) {
+    v[0] = bf16_lo(w.x); v[1] = bf16_hi(w.x);
+    v[2] = bf16_lo(w.y); v[3] = bf16_hi(w.y);
+    v[4] = bf16_lo(w.z); v[5] = bf16_hi(w.z);
+    v[6] = bf16_lo(w.w); v[7] = bf16_hi(w.w);
+}
+
+// e4m3 code -> fp32 (exact).  Subnormals and the NaN code handled explicitly.
+__device__ __forceinline__ float e4m3_to_f32(uint32_t c) {
+    uint32_t mag = c & 0x7Fu;
+    uint32_t sign = (c & 0x80u) << 24;
+    float v;
+    if (mag >= 8u) v = u2f((mag << 20) + 0x3C000000u);          // (e - 7 + 127) << 23 | m << 20
+    else v = (float)mag * 0.001953125f;                        // m * 2^-9
+    if (mag == 0x7Fu) v = u2f(0x7FC00000u);
+    return u2f(f2u(v) | sign);
+}
+
+// expf restated operation for operation from the CPU checker: clamp, Cody-Waite reduction with two
+// fused steps, degree-5 Horner polynomial with fused multiply-adds, exact power-of-two scaling.
+__device__ __forceinline__ float expf_fixed(float x) {
+    x = __builtin_fminf(__builtin_fmaxf(x, -87.0f), 88.5f);
+    float n = __builtin_rintf(x * 1.44269504088896341f);
+    float r = __builtin_fmaf(n, -0.693359375f, x);
+    r = __builtin_fmaf(n, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+    p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+    p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+    p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+    p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+    float r2 = r * r;
+    float y = __builtin_fmaf(p, r2, r);
+    y = y + 1.0f;
+    return __builtin_ldexpf(y, (int)n);
+}
+
+// silu(g) = g / (1 + exp(-g)), IEEE division
+__device__ __forceinline__ float silu_exact(float g) { return g / (1.0f + expf_fixed(-g)); }
+
+}  // namespace pf8

@@ -1,0 +1,670 @@
+// pf8_quant.hip -- bandwidth-bound block quantizers for gfx950 and their C entry points.
+//
+// Data layout in HBM: activations bf16 row-major [rows, K]; e4m3 bytes in the same shape; scales
+// fp32 either [rows, K/128] or [K/128, rows].  One 1x128 tile = 256 B of bf16 = 16 lanes x 16 B, i.e.
+// exactly one DPP row of a 64-wide wavefront, so the tile amax is four DPP max steps and never
+// touches LDS.  2-D work (128x128 weight tiles, the fused row+column quantizer, the per-expert
+// transposing quantizer) stages one 128x128 tile per 256-thread workgroup in registers (8x8
+// elements per thread) and uses LDS only to turn the column-scaled bytes into 16-byte coalesced
+// rows of the transposed output.
+#include "pf8_device.h"
+#include "pf8_host.h"
+
+namespace pf8 {
+
+// ---------------------------------------------------------------------------------------------
+// 1x128 quantizer: one wavefront per row, four tiles per load instruction
+// ---------------------------------------------------------------------------------------------
+
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict__ x, int64_t M, int KB, int64_t ldx,
+                                                     uint8_t* __restrict__ q, float* __restrict__ s, int pow2) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, l = lane & 15;
+    const int64_t r = (int64_t)blockIdx.x * 4 + wave;
+    if (r >= M) return;
+    const uint4* xr = reinterpret_cast<const uint4*>(x + r * ldx);
+    uint2* qr = reinterpret_cast<uint2*>(q + r * (int64_t)KB * 128);
+    constexpr int U = 4;   // tiles in flight per 16-lane group
+    for (int kb0 = 0; kb0 < KB; kb0 += 4 * U) {
+        uint4 w[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int kb = kb0 + 4 * u + g;
+            w[u] = make_uint4(0, 0, 0, 0);
+            if (kb < KB) w[u] = ld16(xr + kb * 16 + l);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int kb = kb0 + 4 * u + g;
+            if (kb < KB) {
+                TileScale t = make_scale(row16_max(amax_bits8(w[u])), pow2 != 0);
+                float v[8];
+                unpack8(w[u], v);
+                uint2 o = quant8(v, t);
+                st8(qr + kb * 16 + l, o);
+                if (l == 0) {
+                    if (LAYOUT == 0) s[r * KB + kb] = t.s;
+                    else s[(int64_t)kb * M + r] = t.s;
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fused SwiGLU (+probs) + 1x128 quantizer: one wavefront per row
+// ---------------------------------------------------------------------------------------------
+
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void k_swiglu_quant(const uint16_t* __restrict__ o1, const float* __restrict__ probs,
+                                                      int64_t M, int IB, uint8_t* __restrict__ q, float* __restrict__ s,
+                                                      uint16_t* __restrict__ o2, int pow2) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, l = lane & 15;
+    const int64_t r = (int64_t)blockIdx.x * 4 + wave;
+    if (r >= M) return;
+    const int64_t I = (int64_t)IB * 128;
+    const uint4* gr = reinterpret_cast<const uint4*>(o1 + r * 2 * I);
+    const uint4* ur = reinterpret_cast<const uint4*>(o1 + r * 2 * I + I);
+    uint2* qr = reinterpret_cast<uint2*>(q + r * I);
+    const bool has_p = probs != nullptr;
+    const float p = has_p ? probs[r] : 1.0f;
+    for (int kb0 = 0; kb0 < IB; kb0 += 8) {
+        uint4 wg[2], wu[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            int kb = kb0 + 4 * u + g;
+            wg[u] = make_uint4(0, 0, 0, 0);
+            wu[u] = make_uint4(0, 0, 0, 0);
+            if (kb < IB) {
+                wg[u] = ld16(gr + kb * 16 + l);
+                wu[u] = ld16(ur + kb * 16 + l);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            int kb = kb0 + 4 * u + g;
+            if (kb < IB) {
+                float gv[8], uv[8], v[8];
+                unpack8(wg[u], gv);
+                unpack8(wu[u], uv);
+                uint32_t am = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    float y = round_bf16(silu_exact(gv[i]) * uv[i]);
+                    if (has_p) y = round_bf16(y * p);
+                    v[i] = y;
+                    am = umax(am, f2u(y) & 0x7FFFFFFFu);
+                }
+                if (o2) {
+                    uint4 ob;
+                    ob.x = (f2u(v[0]) >> 16) | (f2u(v[1]) & 0xFFFF0000u);
+                    ob.y = (f2u(v[2]) >> 16) | (f2u(v[3]) & 0xFFFF0000u);
+                    ob.z = (f2u(v[4]) >> 16) | (f2u(v[5]) & 0xFFFF0000u);
+                    ob.w = (f2u(v[6]) >> 16) | (f2u(v[7]) & 0xFFFF0000u);
+                    reinterpret_cast<uint4*>(o2 + r * I)[kb * 16 + l] = ob;
+                }
+                TileScale t = make_scale(row16_max(am), pow2 != 0);
+                uint2 o = quant8(v, t);
+                st8(qr + kb * 16 + l, o);
+                if (l == 0) {
+                    if (LAYOUT == 0) s[r * IB + kb] = t.s;
+                    else s[(int64_t)kb * M + r] = t.s;
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// SwiGLU backward with probs: one wavefront per row
+// ---------------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void k_swiglu_bwd(const uint16_t* __restrict__ o1, const uint16_t* __restrict__ do2_s,
+                                                    const float* __restrict__ probs, int64_t M, int64_t I,
+                                                    uint16_t* __restrict__ do1, float* __restrict__ probs_grad,
+                                                    uint16_t* __restrict__ o2_s) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + wave;
+    if (r >= M) return;
+    const float p = probs[r];
+    const uint4* gr = reinterpret_cast<const uint4*>(o1 + r * 2 * I);
+    const uint4* ur = reinterpret_cast<const uint4*>(o1 + r * 2 * I + I);
+    const uint4* dr = reinterpret_cast<const uint4*>(do2_s + r * I);
+    uint4* dgr = reinterpret_cast<uint4*>(do1 + r * 2 * I);
+    uint4* dur = reinterpret_cast<uint4*>(do1 + r * 2 * I + I);
+    uint4* osr = reinterpret_cast<uint4*>(o2_s + r * I);
+    const int chunks = (int)(I / 8);
+    float pg = 0.0f;
+    for (int c = lane; c < chunks; c += 64) {
+        uint4 wg = gr[c], wu = ur[c], wd = dr[c];
+        float gv[8], uv[8], dv[8], dg[8], du[8], os[8];
+        unpack8(wg, gv);
+        unpack8(wu, uv);
+        unpack8(wd, dv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float e = expf_fixed(-gv[i]);
+            float den = 1.0f + e;
+            float sl = gv[i] / den;
+            float o2f = round_bf16(sl * uv[i]);
+            os[i] = o2f * p;
+            float do2 = round_bf16(dv[i] * p);
+            pg += dv[i] * o2f;
+            float sig = 1.0f / den;
+            float t1 = 1.0f - sig;
+            float t2 = gv[i] * t1;
+            float t3 = 1.0f + t2;
+            float t4 = sig * t3;
+            float t5 = do2 * uv[i];
+            dg[i] = t5 * t4;
+            du[i] = do2 * sl;
+        }
+        uint4 a, b, o;
+        a.x = pack_bf16(dg[0], dg[1]); a.y = pack_bf16(dg[2], dg[3]); a.z = pack_bf16(dg[4], dg[5]); a.w = pack_bf16(dg[6], dg[7]);
+        b.x = pack_bf16(du[0], du[1]); b.y = pack_bf16(du[2], du[3]); b.z = pack_bf16(du[4], du[5]); b.w = pack_bf16(du[6], du[7]);
+        o.x = pack_bf16(os[0], os[1]); o.y = pack_bf16(os[2], os[3]); o.z = pack_bf16(os[4], os[5]); o.w = pack_bf16(os[6], os[7]);
+        dgr[c] = a;
+        dur[c] = b;
+        osr[c] = o;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) pg += __shfl_xor(pg, off);
+    if (lane == 0) probs_grad[r] = pg;
+}
+
+// ---------------------------------------------------------------------------------------------
+// 128x128-tile kernels: 256 threads, thread (g = tid/16, l = tid%16) owns rows 8g..8g+7 and
+// columns 8l..8l+7 of the tile
+// ---------------------------------------------------------------------------------------------
+
+constexpr int LDT = 33;   // dwords per row of the transposed byte tile in LDS (128 B + 4 B pad)
+
+// write one thread's column-major bytes (column 8l+j, rows 8g..8g+7) into the LDS tile
+__device__ __forceinline__ void lds_put_col(uint32_t* lds_t, int l, int g, int j, uint2 bytes) {
+    uint32_t* p = lds_t + (8 * l + j) * LDT + 2 * g;
+    p[0] = bytes.x;
+    p[1] = bytes.y;
+}
+// after a barrier: thread reads 16 bytes of transposed row c = (tid>>3) + 32*i
+__device__ __forceinline__ uint4 lds_get_row(const uint32_t* lds_t, int c, int seg) {
+    const uint32_t* p = lds_t + c * LDT + 4 * seg;
+    return make_uint4(p[0], p[1], p[2], p[3]);
+}
+
+struct TileSrc {
+    const uint16_t* x;     // bf16 source (or nullptr when the source is e4m3)
+    const uint8_t* xq;     // e4m3 source
+    const float* xs;       // scales of the e4m3 source: [rows, K/128] (xs_layout 0) or [K/128, rows] (1)
+    int64_t ld;            // row stride in elements
+    int64_t rows;          // total rows (for xs_layout 1)
+    int xs_layout;
+};
+
+// load this thread's 8x8 patch as fp32 values; amax bit patterns per row chunk go to rmax[i]
+__device__ __forceinline__ void load_patch(const TileSrc& src, int64_t row0, int64_t col0, int g, int l, float (&v)[8][8]) {
+    if (src.x) {
+        uint4 w[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            w[i] = ld16(src.x + (row0 + 8 * g + i) * src.ld + col0 + 8 * l);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) unpack8(w[i], v[i]);
+    } else {
+        uint2 w[8];
+        float sc[8];
+        const int64_t KB = src.ld / 128;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int64_t r = row0 + 8 * g + i;
+            w[i] = *reinterpret_cast<const uint2*>(src.xq + r * src.ld + col0 + 8 * l);
+            sc[i] = src.xs_layout == 0 ? src.xs[r * KB + col0 / 128] : src.xs[(col0 / 128) * src.rows + r];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[i][j] = round_bf16(e4m3_to_f32((w[i].x >> (8 * j)) & 0xFFu) * sc[i]);
+                v[i][4 + j] = round_bf16(e4m3_to_f32((w[i].y >> (8 * j)) & 0xFFu) * sc[i]);
+            }
+        }
+    }
+}
+
+// reduce a per-thread value over the whole 256-thread workgroup (max of unsigned)
+__device__ __forceinline__ uint32_t block_max(uint32_t v, uint32_t* lds4) {
+    v = row16_max(v);
+    v = umax(v, (uint32_t)__shfl_xor((int)v, 16));
+    v = umax(v, (uint32_t)__shfl_xor((int)v, 32));
+    if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = umax(umax(lds4[0], lds4[1]), umax(lds4[2], lds4[3]));
+    return v;
+}
+
+struct StackArgs {
+    const uint16_t* w[256];
+};
+
+// 128x128 block-scaled quantizer.  Source tile (tr, tc) of expert e; writes q (same orientation)
+// and/or qt (transposed).  STACK: sources come from a pointer table, outputs are stacked per expert.
+template <bool STACK>
+__global__ __launch_bounds__(256) void k_quant_128x128(const uint16_t* __restrict__ w, StackArgs ptrs, int64_t R, int64_t C,
+                                                       uint8_t* __restrict__ q, float* __restrict__ s, uint8_t* __restrict__ qt,
+                                                       float* __restrict__ st, int pow2) {
+    __shared__ uint32_t lds_t[128 * LDT];
+    __shared__ uint32_t lds4[4];
+    const int tid = threadIdx.x, g = tid >> 4, l = tid & 15;
+    const int64_t CB = C / 128, RB = R / 128;
+    const int64_t tc = blockIdx.x, tr = blockIdx.y, e = blockIdx.z;
+    TileSrc src;
+    src.x = STACK ? ptrs.w[e] : w;
+    src.xq = nullptr; src.xs = nullptr; src.ld = C; src.rows = R; src.xs_layout = 0;
+    const int64_t row0 = tr * 128, col0 = tc * 128;
+    float v[8][8];
+    load_patch(src, row0, col0, g, l, v);
+    uint32_t am = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) am = umax(am, f2u(v[i][j]) & 0x7FFFFFFFu);
+    am = block_max(am, lds4);
+    TileScale t = make_scale(am, pow2 != 0);
+    const int64_t ebase = e * R * C;
+    if (q) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            uint2 o = quant8(v[i], t);
+            st8(q + ebase + (row0 + 8 * g + i) * C + col0 + 8 * l, o);
+        }
+        if (tid == 0) s[e * RB * CB + tr * CB + tc] = t.s;
+    }
+    if (qt) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float col[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) col[i] = v[i][j];
+            lds_put_col(lds_t, l, g, j, quant8(col, t));
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int c = (tid >> 3) + 32 * i, seg = tid & 7;
+            uint4 o = lds_get_row(lds_t, c, seg);
+            st16(qt + ebase + (col0 + c) * R + row0 + 16 * seg, o);
+        }
+        if (tid == 0) st[e * RB * CB + tc * RB + tr] = t.s;
+    }
+}
+
+struct SplitArgs {
+    int32_t tile_start[257];   // first 128-row tile of each expert (prefix sums), tile_start[E] = total
+    int32_t E;
+};
+
+// Row-scaled copy (optional) + column-scaled transposed copy of one 128x128 tile.
+//   SPLIT=false: q[M,K] + s, qt[K,M] + st                (fused quant+transpose)
+//   SPLIT=true : qt / st packed per expert               (transpose-split-quant), source bf16 or e4m3
+template <bool SPLIT, int LAYOUT>
+__global__ __launch_bounds__(256) void k_quant_rowcol(TileSrc src, int64_t M, int64_t K, uint8_t* __restrict__ q,
+                                                      float* __restrict__ s, uint8_t* __restrict__ qt, float* __restrict__ st,
+                                                      SplitArgs sp, int pow2) {
+    __shared__ uint32_t lds_t[128 * LDT];
+    __shared__ uint32_t lds_cm[4 * 64];
+    const int tid = threadIdx.x, g = tid >> 4, l = tid & 15, wave = tid >> 6, lane = tid & 63;
+    const int64_t tc = blockIdx.x, tr = blockIdx.y;
+    const int64_t row0 = tr * 128, col0 = tc * 128;
+    const int64_t KB = K / 128, MB = M / 128;
+    float v[8][8];
+    load_patch(src, row0, col0, g, l, v);
+
+    // column amax: this thread's 8 rows, then the 4 row groups of the wave, then the 4 waves via LDS
+    uint32_t cm[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m = umax(m, f2u(v[i][j]) & 0x7FFFFFFFu);
+        m = umax(m, (uint32_t)__shfl_xor((int)m, 16));
+        m = umax(m, (uint32_t)__shfl_xor((int)m, 32));
+        cm[j] = m;
+    }
+    if (lane < 16) {
+        // bf16-derived magnitudes have 16 significant bits: pack two per dword
+#pragma unroll
+        for (int j = 0; j < 4; ++j) lds_cm[wave * 64 + 4 * l + j] = (cm[2 * j] >> 16) | (cm[2 * j + 1] & 0xFFFF0000u);
+    }
+
+    // row-scaled copy while the column maxima settle
+    if (q) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) m = umax(m, f2u(v[i][j]) & 0x7FFFFFFFu);
+            TileScale t = make_scale(row16_max(m), pow2 != 0);
+            uint2 o = quant8(v[i], t);
+            const int64_t r = row0 + 8 * g + i;
+            st8(q + r * K + col0 + 8 * l, o);
+            if (l == i) {
+                if (LAYOUT == 0) s[r * KB + tc] = t.s;
+                else s[tc * M + r] = t.s;
+            }
+        }
+    }
+    __syncthreads();
+    uint32_t cmp[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t a = pkmax_u16(lds_cm[0 * 64 + 4 * l + j], lds_cm[1 * 64 + 4 * l + j]);
+        uint32_t b = pkmax_u16(lds_cm[2 * 64 + 4 * l + j], lds_cm[3 * 64 + 4 * l + j]);
+        cmp[j] = pkmax_u16(a, b);
+    }
+    float cs[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        uint32_t am = (j & 1) ? (cmp[j >> 1] & 0xFFFF0000u) : (cmp[j >> 1] << 16);
+        TileScale t = make_scale(am, pow2 != 0);
+        cs[j] = t.s;
+        float col[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) col[i] = v[i][j];
+        lds_put_col(lds_t, l, g, j, quant8(col, t));
+    }
+    __syncthreads();
+
+    // destination of the transposed tile
+    int64_t qt_base, st_row, ldq;
+    if (SPLIT) {
+        // expert of this row tile: linear scan of the prefix table (E <= 256, uniform per workgroup)
+        int e = 0;
+        while (e + 1 < sp.E && (int64_t)sp.tile_start[e + 1] <= tr) ++e;
+        const int64_t off = (int64_t)sp.tile_start[e] * 128;                       // rows before this expert
+        const int64_t Me = (int64_t)(sp.tile_start[e + 1] - sp.tile_start[e]) * 128;
+        qt_base = off * K + (row0 - off);      // + c*Me
+        ldq = Me;
+        st_row = tr;                           // scale rows are tile rows, globally numbered
+    } else {
+        qt_base = row0;
+        ldq = M;
+        st_row = tr;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int c = (tid >> 3) + 32 * i, seg = tid & 7;
+        uint4 o = lds_get_row(lds_t, c, seg);
+        st16(qt + qt_base + (col0 + c) * ldq + 16 * seg, o);
+    }
+    if (g == 0) {
+        if (LAYOUT == 1 || SPLIT) {
+            float4* p = reinterpret_cast<float4*>(st + st_row * K + col0 + 8 * l);
+            p[0] = make_float4(cs[0], cs[1], cs[2], cs[3]);
+            p[1] = make_float4(cs[4], cs[5], cs[6], cs[7]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) st[(col0 + 8 * l + j) * MB + tr] = cs[j];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dequantizers
+// ---------------------------------------------------------------------------------------------
+
+// 1x128 dequant: one thread per 8 bytes
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void k_act_dequant(const uint8_t* __restrict__ q, const float* __restrict__ s, int64_t M,
+                                                     int64_t K, uint16_t* __restrict__ out) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;   // 8-byte chunk index
+    const int64_t cpr = K / 8;
+    if (idx >= M * cpr) return;
+    const int64_t r = idx / cpr, c8 = idx % cpr;
+    const int64_t kb = c8 / 16, KB = K / 128;
+    const float sc = LAYOUT == 0 ? s[r * KB + kb] : s[kb * M + r];
+    uint2 w = *reinterpret_cast<const uint2*>(q + idx * 8);
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        f[j] = e4m3_to_f32((w.x >> (8 * j)) & 0xFFu) * sc;
+        f[4 + j] = e4m3_to_f32((w.y >> (8 * j)) & 0xFFu) * sc;
+    }
+    uint4 o;
+    o.x = pack_bf16(f[0], f[1]); o.y = pack_bf16(f[2], f[3]); o.z = pack_bf16(f[4], f[5]); o.w = pack_bf16(f[6], f[7]);
+    *reinterpret_cast<uint4*>(out + idx * 8) = o;
+}
+
+// 128x128 dequant, arbitrary R and C: one thread per element (checkpoint-load path, not hot)
+__global__ __launch_bounds__(256) void k_weight_dequant(const uint8_t* __restrict__ q, const float* __restrict__ s, int64_t R,
+                                                        int64_t C, uint16_t* __restrict__ out) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= R * C) return;
+    const int64_t r = idx / C, c = idx % C, CB = (C + 127) / 128;
+    float f = e4m3_to_f32(q[idx]) * s[(r / 128) * CB + c / 128];
+    out[idx] = (uint16_t)(pack_bf16(f, 0.0f) & 0xFFFFu);
+}
+
+// ---------------------------------------------------------------------------------------------
+// self-test kernels
+// ---------------------------------------------------------------------------------------------
+
+__global__ void k_debug_encode(const float* v, int64_t n, uint8_t* out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (uint8_t)(cvt_e4m3_lo(v[i], 0.0f, 0u) & 0xFFu);
+}
+__global__ void k_debug_div_encode(const float* x, const float* s, int64_t n, uint8_t* out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    TileScale t;
+    t.s = s[i];
+    t.r = __builtin_amdgcn_rcpf(t.s);
+    t.slow = !(t.s >= 1.0e-30f);
+    float v[8] = {x[i], 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    uint2 o = quant8(v, t);
+    out[i] = (uint8_t)(o.x & 0xFFu);
+}
+__global__ void k_debug_silu(const float* x, int64_t n, float* out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = silu_exact(x[i]);
+}
+
+}  // namespace pf8
+
+using namespace pf8;
+
+// ---------------------------------------------------------------------------------------------
+// C entry points
+// ---------------------------------------------------------------------------------------------
+
+#define PF8_REQUIRE(cond, msg) do { if (!(cond)) return pf8_fail(PF8_EINVAL, __func__, msg); } while (0)
+#define PF8_ALIGNED16(p) ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)
+
+extern "C" int pf8_quant_1x128(const uint16_t* x, int64_t M, int64_t K, int64_t ldx, uint8_t* q, float* s, int scale_layout,
+                               int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(M >= 0 && K >= 0, "negative shape");
+    PF8_REQUIRE(K % 128 == 0, "K must be a multiple of 128");
+    if (M == 0 || K == 0) return PF8_OK;
+    PF8_REQUIRE(x && q && s, "null pointer");
+    PF8_REQUIRE(ldx >= K && ldx % 8 == 0, "ldx must be >= K and a multiple of 8");
+    PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q) && (reinterpret_cast<uintptr_t>(s) & 3u) == 0, "pointers must be 16-byte aligned");
+    PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
+    PF8_REQUIRE(M <= (int64_t)4 * 0x7FFFFFFF && K / 128 <= 0x7FFFFF, "shape too large");
+    dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    if (scale_layout == 0) hipLaunchKernelGGL(k_quant_1x128<0>, grid, block, 0, st, x, M, (int)(K / 128), ldx, q, s, pow2);
+    else hipLaunchKernelGGL(k_quant_1x128<1>, grid, block, 0, st, x, M, (int)(K / 128), ldx, q, s, pow2);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_quant_128x128(const uint16_t* w, int64_t R, int64_t C, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
+                                 int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(R >= 0 && C >= 0, "negative shape");
+    PF8_REQUIRE(R % 128 == 0 && C % 128 == 0, "R and C must be multiples of 128");
+    if (R == 0 || C == 0) return PF8_OK;
+    PF8_REQUIRE(w, "null pointer");
+    PF8_REQUIRE((q != nullptr) == (s != nullptr) && (q_t != nullptr) == (s_t != nullptr), "q/s and q_t/s_t come in pairs");
+    PF8_REQUIRE(q || q_t, "no output requested");
+    PF8_REQUIRE(PF8_ALIGNED16(w) && PF8_ALIGNED16(q) && PF8_ALIGNED16(q_t), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(R / 128 <= 65535 && C / 128 <= 0x7FFFFFFF, "shape too large");
+    dim3 grid((unsigned)(C / 128), (unsigned)(R / 128), 1), block(256);
+    StackArgs none = {};
+    hipLaunchKernelGGL(k_quant_128x128<false>, grid, block, 0, (hipStream_t)stream, w, none, R, C, q, s, q_t, s_t, pow2);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_stack_transpose_quant(const uint16_t* const* w_list, int E, int64_t R, int64_t C, int transpose, uint8_t* q,
+                                         float* s, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(E >= 0 && R >= 0 && C >= 0, "negative shape");
+    PF8_REQUIRE(R % 128 == 0 && C % 128 == 0, "R and C must be multiples of 128");
+    if (E == 0 || R == 0 || C == 0) return PF8_OK;
+    PF8_REQUIRE(w_list && q && s, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(q), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(R / 128 <= 65535, "shape too large");
+    for (int e = 0; e < E; ++e) PF8_REQUIRE(w_list[e] && PF8_ALIGNED16(w_list[e]), "null or misaligned weight pointer");
+    const int64_t per_q = R * C, per_s = (R / 128) * (C / 128);
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        const int n = E - e0 < 256 ? E - e0 : 256;
+        StackArgs a = {};
+        for (int i = 0; i < n; ++i) a.w[i] = w_list[e0 + i];
+        dim3 grid((unsigned)(C / 128), (unsigned)(R / 128), (unsigned)n), block(256);
+        uint8_t* qe = q + (int64_t)e0 * per_q;
+        float* se = s + (int64_t)e0 * per_s;
+        if (transpose)
+            hipLaunchKernelGGL(k_quant_128x128<true>, grid, block, 0, (hipStream_t)stream, nullptr, a, R, C, (uint8_t*)nullptr,
+                               (float*)nullptr, qe, se, pow2);
+        else
+            hipLaunchKernelGGL(k_quant_128x128<true>, grid, block, 0, (hipStream_t)stream, nullptr, a, R, C, qe, se,
+                               (uint8_t*)nullptr, (float*)nullptr, pow2);
+        int rc = pf8_check_launch(__func__);
+        if (rc) return rc;
+    }
+    return PF8_OK;
+}
+
+extern "C" int pf8_quant_transpose(const uint16_t* x, int64_t M, int64_t K, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
+                                   int scale_layout, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(M >= 0 && K >= 0, "negative shape");
+    PF8_REQUIRE(M % 128 == 0 && K % 128 == 0, "M and K must be multiples of 128");
+    if (M == 0 || K == 0) return PF8_OK;
+    PF8_REQUIRE(x && q_t && s_t, "null pointer");
+    PF8_REQUIRE((q != nullptr) == (s != nullptr), "q and s come as a pair");
+    PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q) && PF8_ALIGNED16(q_t) && PF8_ALIGNED16(s_t), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
+    PF8_REQUIRE(M / 128 <= 65535, "M too large");
+    TileSrc src = {x, nullptr, nullptr, K, M, 0};
+    SplitArgs sp = {};
+    dim3 grid((unsigned)(K / 128), (unsigned)(M / 128)), block(256);
+    if (scale_layout == 0)
+        hipLaunchKernelGGL((k_quant_rowcol<false, 0>), grid, block, 0, (hipStream_t)stream, src, M, K, q, s, q_t, s_t, sp, pow2);
+    else
+        hipLaunchKernelGGL((k_quant_rowcol<false, 1>), grid, block, 0, (hipStream_t)stream, src, M, K, q, s, q_t, s_t, sp, pow2);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_transpose_split_quant(const void* x, const float* xs, int x_is_fp8, int xs_layout, const int64_t* rows_per_expert,
+                                         int E, int64_t K, uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(xs_layout == 0 || xs_layout == 1, "xs_layout must be 0 or 1");
+    PF8_REQUIRE(E >= 0 && K >= 0, "negative shape");
+    PF8_REQUIRE(K % 128 == 0, "K must be a multiple of 128");
+    PF8_REQUIRE(E <= 256, "at most 256 experts per call");
+    if (E == 0 || K == 0) return PF8_OK;
+    PF8_REQUIRE(rows_per_expert, "null pointer");
+    SplitArgs sp = {};
+    int64_t total = 0;
+    for (int e = 0; e < E; ++e) {
+        PF8_REQUIRE(rows_per_expert[e] >= 0 && rows_per_expert[e] % 128 == 0, "rows_per_expert entries must be non-negative multiples of 128");
+        sp.tile_start[e] = (int32_t)(total / 128);
+        total += rows_per_expert[e];
+    }
+    PF8_REQUIRE(total / 128 <= 65535, "too many rows");
+    sp.tile_start[E] = (int32_t)(total / 128);
+    sp.E = E;
+    if (total == 0) return PF8_OK;
+    PF8_REQUIRE(x && q_t && s_t, "null pointer");
+    PF8_REQUIRE(!x_is_fp8 || xs, "fp8 input needs its scales");
+    PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q_t) && PF8_ALIGNED16(s_t), "pointers must be 16-byte aligned");
+    TileSrc src;
+    src.x = x_is_fp8 ? nullptr : (const uint16_t*)x;
+    src.xq = x_is_fp8 ? (const uint8_t*)x : nullptr;
+    src.xs = xs;
+    src.ld = K;
+    src.rows = total;
+    src.xs_layout = xs_layout;
+    dim3 grid((unsigned)(K / 128), (unsigned)(total / 128)), block(256);
+    hipLaunchKernelGGL((k_quant_rowcol<true, 1>), grid, block, 0, (hipStream_t)stream, src, total, K, (uint8_t*)nullptr,
+                       (float*)nullptr, q_t, s_t, sp, pow2);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_swiglu_weighted_quant(const uint16_t* o1, const float* probs, int64_t M, int64_t I, uint8_t* q, float* s,
+                                         uint16_t* o2, int scale_layout, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(M >= 0 && I >= 0, "negative shape");
+    PF8_REQUIRE(I % 128 == 0, "I must be a multiple of 128");
+    if (M == 0 || I == 0) return PF8_OK;
+    PF8_REQUIRE(o1 && q && s, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(o1) && PF8_ALIGNED16(q) && PF8_ALIGNED16(o2), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
+    PF8_REQUIRE(M <= (int64_t)4 * 0x7FFFFFFF, "shape too large");
+    dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    if (scale_layout == 0)
+        hipLaunchKernelGGL(k_swiglu_quant<0>, grid, block, 0, (hipStream_t)stream, o1, probs, M, (int)(I / 128), q, s, o2, pow2);
+    else
+        hipLaunchKernelGGL(k_swiglu_quant<1>, grid, block, 0, (hipStream_t)stream, o1, probs, M, (int)(I / 128), q, s, o2, pow2);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_swiglu_weighted_bwd(const uint16_t* o1, const uint16_t* do2_s, const float* probs, int64_t M, int64_t I,
+                                       uint16_t* do1, float* probs_grad, uint16_t* o2_s, pf8_stream_t stream) {
+    PF8_REQUIRE(M >= 0 && I >= 0, "negative shape");
+    PF8_REQUIRE(I % 8 == 0, "I must be a multiple of 8");
+    if (M == 0) return PF8_OK;
+    PF8_REQUIRE(I > 0, "I must be positive");
+    PF8_REQUIRE(o1 && do2_s && probs && do1 && probs_grad && o2_s, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(o1) && PF8_ALIGNED16(do2_s) && PF8_ALIGNED16(do1) && PF8_ALIGNED16(o2_s), "pointers must be 16-byte aligned");
+    dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    hipLaunchKernelGGL(k_swiglu_bwd, grid, block, 0, (hipStream_t)stream, o1, do2_s, probs, M, I, do1, probs_grad, o2_s);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_act_dequant(const uint8_t* q, const float* s, int scale_layout, int64_t M, int64_t K, uint16_t* out,
+                               pf8_stream_t stream) {
+    PF8_REQUIRE(M >= 0 && K >= 0, "negative shape");
+    PF8_REQUIRE(K % 128 == 0, "K must be a multiple of 128");
+    if (M == 0 || K == 0) return PF8_OK;
+    PF8_REQUIRE(q && s && out, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(q) && PF8_ALIGNED16(out), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
+    const int64_t chunks = M * (K / 8);
+    dim3 grid((unsigned)((chunks + 255) / 256)), block(256);
+    if (scale_layout == 0) hipLaunchKernelGGL(k_act_dequant<0>, grid, block, 0, (hipStream_t)stream, q, s, M, K, out);
+    else hipLaunchKernelGGL(k_act_dequant<1>, grid, block, 0, (hipStream_t)stream, q, s, M, K, out);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_weight_dequant(const uint8_t* q, const float* s, int64_t R, int64_t C, uint16_t* out, pf8_stream_t stream) {
+    PF8_REQUIRE(R >= 0 && C >= 0, "negative shape");
+    if (R == 0 || C == 0) return PF8_OK;
+    PF8_REQUIRE(q && s && out, "null pointer");
+    const int64_t n = R * C;
+    dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    hipLaunchKernelGGL(k_weight_dequant, grid, block, 0, (hipStream_t)stream, q, s, R, C, out);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_debug_encode(const float* v, int64_t n, uint8_t* out, pf8_stream_t stream) {
+    if (n <= 0) return PF8_OK;
+    PF8_REQUIRE(v && out, "null pointer");
+    hipLaunchKernelGGL(k_debug_encode, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, v, n, out);
+    return pf8_check_launch(__func__);
+}
+extern "C" int pf8_debug_div_encode(const float* x, const float* s, int64_t n, uint8_t* out, pf8_stream_t stream) {
+    if (n <= 0) return PF8_OK;
+    PF8_REQUIRE(x && s && out, "null pointer");
+    hipLaunchKernelGGL(k_debug_div_encode, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, s, n, out);
+    return pf8_check_launch(__func__);
+}
+extern "C" int pf8_debug_silu(const float* x, int64_t n, float* out, pf8_stream_t stream) {
+    if (n <= 0) return PF8_OK;
+    PF8_REQUIRE(x && out, "null pointer");
+    hipLaunchKernelGGL(k_debug_silu, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, n, out);
+    return pf8_check_launch(__func__);
+}

@@ -1,0 +1,154 @@
+"""Drop-in for the `deep_gemm` module object the reference binds at import time
+(`from paddlefleet_ops import deep_gemm`, transformers/fp8_utils.py:34-44).
+
+Same function names and argument conventions: operands are `(fp8_tensor, scale_tensor)` pairs,
+the output tensor is allocated by the caller and written in place.  Everything runs through the
+MFMA kernels of libpf8 on the current stream.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from .functional import FP8, _dev, _p, _scale_layout_of, _stream
+
+
+def set_num_sms(num: int) -> None:
+    """deep_gemm.set_num_sms(get_sm_num()) -- transformers/fp8_utils.py:277.  Caps the compute
+    units the GEMM grids assume (0 = the whole device)."""
+    _lib.lib().pf8_set_num_cus(int(num))
+
+
+def get_num_sms() -> int:
+    return int(_lib.lib().pf8_get_num_cus())
+
+
+def _check_pair(pair, what) -> Tuple[torch.Tensor, torch.Tensor]:
+    if not (isinstance(pair, (tuple, list)) and len(pair) == 2):
+        raise ValueError(f"{what} must be a (tensor, scale) pair")
+    t, s = pair
+    _dev(t, what)
+    _dev(s, what + " scale")
+    if t.dtype != FP8:
+        raise ValueError(f"{what} must be float8_e4m3fn")
+    return t, s
+
+
+def fp8_gemm_nt(a, b, out: torch.Tensor, c: Optional[torch.Tensor] = None, recipe=None, compiled_dims: str = "nk"):
+    """out[M, N] = a[M, K] . b[N, K]^T with block scales, fp32 accumulation.
+
+    Default recipe (transformers/fp8_utils.py:278): a is 1x128-scaled with sa logically [M, K/128]
+    (any strides; the M-contiguous `.T` view of a [K/128, M] tensor is consumed without a copy),
+    b is 128x128-scaled with sb [ceil(N/128), K/128]; out is bf16.
+    recipe=(1, 1, 128) (transformers/fp8_utils.py:187-194): both operands 1x128-scaled along K with
+    scales logically [rows, K/128]; out is fp32 and `c is out` means accumulate.
+    """
+    (ta, sa), (tb, sb) = _check_pair(a, "a"), _check_pair(b, "b")
+    _dev(out, "out")
+    M, K = ta.shape
+    N, K2 = tb.shape
+    if K != K2 or K % 128 != 0:
+        raise ValueError("a and b must share a K that is a multiple of 128")
+    if tuple(out.shape) != (M, N):
+        raise ValueError(f"out must be [{M}, {N}]")
+    if M == 0 or N == 0:
+        return out
+    ta = ta if ta.is_contiguous() else ta.contiguous()
+    tb = tb if tb.is_contiguous() else tb.contiguous()
+    if recipe is not None and tuple(recipe) == (1, 1, 128):
+        if out.dtype != torch.float32 or not out.is_contiguous():
+            raise ValueError("the (1, 1, 128) recipe writes a contiguous float32 output")
+        if c is not None and c is not out and c.data_ptr() != out.data_ptr():
+            raise ValueError("c must be the output tensor (in-place accumulation)")
+        # scales arrive as [rows, K/128] views of [K/128, rows] storage; the kernel wants the latter
+        sa_k = sa.t() if sa.t().is_contiguous() else sa.t().contiguous()
+        sb_k = sb.t() if sb.t().is_contiguous() else sb.t().contiguous()
+        if tuple(sa_k.shape) != (K // 128, M) or tuple(sb_k.shape) != (K // 128, N):
+            raise ValueError("scales must be [rows, K/128]")
+        _lib.call("pf8_gemm_nt_1d1d_f32", _p(ta), _p(sa_k), _p(tb), _p(sb_k), M, N, K, _p(out), int(c is not None), _stream())
+        return out
+    if recipe is not None:
+        raise ValueError(f"unsupported recipe {recipe!r}")
+    if c is not None:
+        raise ValueError("accumulation needs recipe=(1, 1, 128)")
+    if out.dtype != torch.bfloat16 or out.stride(-1) != 1:
+        raise ValueError("out must be bfloat16 with a unit inner stride")
+    sa, lay = _scale_layout_of(sa, M, K // 128, "a scale")
+    if tuple(sb.shape) != ((N + 127) // 128, K // 128) or sb.dtype != torch.float32:
+        raise ValueError(f"b scale must be float32 [{(N + 127) // 128}, {K // 128}]")
+    sb = sb if sb.is_contiguous() else sb.contiguous()
+    _lib.call("pf8_gemm_nt", _p(ta), _p(sa), lay, _p(tb), _p(sb), M, N, K, _p(out), out.stride(0), _stream())
+    return out
+
+
+def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.Tensor):
+    """Grouped GEMM over rows sorted by expert: row m uses b[m_indices[m]].
+
+    transformers/fp8_utils.py:949-954: a [Mtot, K] + sa [Mtot, K/128] (any strides), b [E, N, K] +
+    sb [E, N/128, K/128], m_indices int32 [Mtot]; every expert segment is a multiple of 128 rows.
+    """
+    (ta, sa), (tb, sb) = _check_pair(a, "a"), _check_pair(b, "b")
+    _dev(out, "out")
+    _dev(m_indices, "m_indices")
+    Mtot, K = ta.shape
+    if tb.dim() != 3:
+        raise ValueError("b must be [E, N, K]")
+    E, N, K2 = tb.shape
+    if K != K2 or K % 128 != 0:
+        raise ValueError("a and b must share a K that is a multiple of 128")
+    if Mtot % 128 != 0:
+        raise ValueError("the row count must be a multiple of 128 (expert segments are padded to 128)")
+    if tuple(out.shape) != (Mtot, N) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous bfloat16 [{Mtot}, {N}] tensor")
+    if m_indices.dtype != torch.int32 or m_indices.numel() != Mtot:
+        raise ValueError("m_indices must be int32 with one entry per row")
+    if Mtot == 0 or N == 0:
+        return out
+    ta = ta if ta.is_contiguous() else ta.contiguous()
+    tb = tb if tb.is_contiguous() else tb.contiguous()
+    sa, lay = _scale_layout_of(sa, Mtot, K // 128, "a scale")
+    if tuple(sb.shape) != (E, (N + 127) // 128, K // 128) or sb.dtype != torch.float32:
+        raise ValueError(f"b scale must be float32 [{E}, {(N + 127) // 128}, {K // 128}]")
+    sb = sb if sb.is_contiguous() else sb.contiguous()
+    m_indices = m_indices if m_indices.is_contiguous() else m_indices.contiguous()
+    _lib.call("pf8_grouped_gemm_nt_contiguous", _p(ta), _p(sa), lay, _p(tb), _p(sb), E, Mtot, N, K, _p(m_indices), _p(out), _stream())
+    return out
+
+
+def m_grouped_fp8_gemm_nt_masked(a, b, out: torch.Tensor, masked_m: torch.Tensor, expected_m: int):
+    """Grouped GEMM with a fixed capacity per expert.
+
+    ernie token_dispatcher/fp8_utils.py:227-233: a [E, Mmax, K] + sa [E, Mmax, K/128], b [E, N, K] +
+    sb [E, N/128, K/128], masked_m int32 [E]; rows at or beyond masked_m[e] are not written.
+    """
+    (ta, sa), (tb, sb) = _check_pair(a, "a"), _check_pair(b, "b")
+    _dev(out, "out")
+    _dev(masked_m, "masked_m")
+    if ta.dim() != 3 or tb.dim() != 3:
+        raise ValueError("a must be [E, Mmax, K] and b [E, N, K]")
+    E, Mmax, K = ta.shape
+    E2, N, K2 = tb.shape
+    if E != E2 or K != K2 or K % 128 != 0:
+        raise ValueError("a and b must agree on E and on a K that is a multiple of 128")
+    if tuple(out.shape) != (E, Mmax, N) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous bfloat16 [{E}, {Mmax}, {N}] tensor")
+    if masked_m.dtype != torch.int32 or masked_m.numel() != E:
+        raise ValueError("masked_m must be int32 [E]")
+    if E == 0 or Mmax == 0 or N == 0:
+        return out
+    ta, tb = ta.contiguous(), tb.contiguous()
+    if tuple(sa.shape) != (E, Mmax, K // 128) or tuple(sb.shape) != (E, (N + 127) // 128, K // 128):
+        raise ValueError("scale shapes must be [E, Mmax, K/128] and [E, N/128, K/128]")
+    sa, sb = sa.contiguous(), sb.contiguous()
+    _lib.call("pf8_grouped_gemm_nt_masked", _p(ta), _p(sa), _p(tb), _p(sb), E, Mmax, N, K, _p(masked_m.contiguous()), int(expected_m),
+              _p(out), _stream())
+    return out
+
+
+# names the reference aliases when it falls back to paddle.incubate.fp8.deep_gemm (fp8_utils.py:42-44)
+gemm_fp8_fp8_bf16_nt = fp8_gemm_nt
+m_grouped_gemm_fp8_fp8_bf16_nt_contiguous = m_grouped_fp8_gemm_nt_contiguous
+m_grouped_gemm_fp8_fp8_bf16_nt_masked = m_grouped_fp8_gemm_nt_masked

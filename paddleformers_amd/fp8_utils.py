@@ -1,0 +1,548 @@
+"""Host-side mirror of paddleformers/transformers/fp8_utils.py for the FP8 hot path.
+
+Same class and function names, argument meaning and error behaviour as the reference module; the
+third-party operators it resolves at call time are replaced by `paddleformers_amd.functional`
+(paddle.incubate.nn.functional.*) and `paddleformers_amd.deep_gemm` (paddlefleet_ops.deep_gemm).
+Tensors are torch-ROCm tensors; weights are bf16 tensors (optionally carrying a float32
+`main_grad` attribute, which the weight-gradient GEMMs accumulate into).
+
+One deliberate difference: FP8GroupGemmMlpFunctionNode.backward writes dx into a fresh tensor.
+The reference passes `dx=out_grad` (transformers/fp8_utils.py:1297-1303), which overwrites the
+output gradient before the down-projection weight gradient reads it (:1306-1313).
+"""
+from __future__ import annotations
+
+from functools import partial
+from typing import List, Optional, Sequence
+
+import numpy
+import torch
+
+from . import deep_gemm
+from . import functional as F8
+
+__all__ = [
+    "FP8LinearFunctionBase",
+    "FP8GroupGemmMlpFunctionNode",
+    "FP8Mlp",
+    "WeightGradStore",
+    "weight_quant",
+    "fused_stack_quant",
+    "split_group_gemm",
+    "swiglu",
+    "get_sm_num",
+]
+
+
+def swiglu(x, y=None):
+    """silu(x) * y with x, y the two halves of the last axis when y is None (fp8_utils.py:23-29)."""
+    return F8.swiglu(x, y)
+
+
+def get_sm_num():
+    """fp8_utils.py:54-55 returns 112 (of an H800's 132 SMs) to leave room for communication
+    kernels; on one GPU without collectives the whole device is used (0 = no cap)."""
+    return 0
+
+
+class WeightGradStore:
+    """Minimal stand-in for paddle's zero-bubble WeightGradStore (fp8_utils.py:31, :314-327):
+    when enabled, weight-gradient closures are queued and run at flush()."""
+
+    enabled = False
+    _queue: List = []
+
+    @classmethod
+    def put(cls, fn):
+        cls._queue.append(fn)
+
+    @classmethod
+    def flush(cls):
+        q, cls._queue = cls._queue, []
+        for fn in q:
+            fn()
+
+    @classmethod
+    def clear(cls):
+        cls._queue = []
+
+
+def extract_first_if_tuple(x):
+    return x[0] if isinstance(x, tuple) else x
+
+
+def _get_fp8_weight_and_scale(weight, stacked=False, transpose=False):
+    """Cached quantised weights live as attributes on the bf16 tensor (fp8_utils.py:76-88)."""
+    if stacked:
+        if transpose:
+            return weight.fp8_weight_stacked_transpose, weight.fp8_scale_stacked_transpose
+        return weight.fp8_weight_stacked, weight.fp8_scale_stacked
+    if transpose:
+        return weight.fp8_weight_transpose, weight.fp8_scale_transpose
+    return weight.fp8_weight, weight.fp8_scale
+
+
+def fused_stack_quant(expert_weight_list, transpose=False):
+    """fp8_utils.py:91-102: use the per-step cache on expert 0's weight when present, else quantise."""
+    w0 = expert_weight_list[0]
+    if transpose and hasattr(w0, "fp8_weight_stacked_transpose"):
+        return _get_fp8_weight_and_scale(w0, stacked=True, transpose=True)
+    if not transpose and hasattr(w0, "fp8_weight_stacked"):
+        return _get_fp8_weight_and_scale(w0, stacked=True, transpose=False)
+    if hasattr(w0, "fp8_weight_stacked"):
+        # only the other orientation is cached: callers transpose it themselves (fp8_utils.py:925-927)
+        return _get_fp8_weight_and_scale(w0, stacked=True, transpose=False)
+    if hasattr(w0, "fp8_weight_stacked_transpose"):
+        return _get_fp8_weight_and_scale(w0, stacked=True, transpose=True)
+    return F8.fused_stack_transpose_quant(expert_weight_list, transpose=transpose)
+
+
+def weight_quant(weight, transpose=False):
+    """fp8_utils.py:105-131: 128x128 quantisation of one weight, cached copies first."""
+    if transpose:
+        if hasattr(weight, "fp8_weight_transpose"):
+            return weight.fp8_weight_transpose, weight.fp8_scale_transpose
+        if hasattr(weight, "fp8_weight"):
+            return weight.fp8_weight.T.contiguous(), weight.fp8_scale.T.contiguous()
+        return F8.fp8_quant_blockwise(weight, output_scale_transpose=False, quant_method="128x128", input_transpose=True,
+                                      return_transpose_only=True)
+    if hasattr(weight, "fp8_weight"):
+        return weight.fp8_weight, weight.fp8_scale
+    if hasattr(weight, "fp8_weight_transpose"):
+        return weight.fp8_weight_transpose.T.contiguous(), weight.fp8_scale_transpose.T.contiguous()
+    return F8.fp8_quant_blockwise(weight, output_scale_transpose=False, quant_method="128x128", input_transpose=False,
+                                  return_transpose_only=False)
+
+
+def cache_fp8_weight(weight, quant_transpose=None):
+    """fp8_utils.py:628-665: attach quantised copies to the weight for the coming step."""
+    if quant_transpose is None:
+        q, s, qt, st = F8.fp8_quant_blockwise(weight, output_scale_transpose=False, quant_method="128x128", input_transpose=True)
+        weight.fp8_weight, weight.fp8_scale = q, s
+        weight.fp8_weight_transpose, weight.fp8_scale_transpose = qt, st
+    elif quant_transpose is True:
+        qt, st = F8.fp8_quant_blockwise(weight, output_scale_transpose=False, quant_method="128x128", input_transpose=True,
+                                        return_transpose_only=True)
+        weight.fp8_weight_transpose, weight.fp8_scale_transpose = qt, st
+    elif quant_transpose is False:
+        q, s = F8.fp8_quant_blockwise(weight, output_scale_transpose=False, quant_method="128x128", input_transpose=False)
+        weight.fp8_weight, weight.fp8_scale = q, s
+    else:
+        raise ValueError("quant_transpose must be either True, False or None.")
+
+
+def split_group_gemm(x_fp8, x_scale, w_fp8, w_scale, tokens_per_expert, gemm_out):
+    """fp8_utils.py:853-870: the grouped GEMM as a loop of dense GEMMs, empty experts skipped."""
+    start_idx = 0
+    for i, token_num in enumerate(tokens_per_expert):
+        if token_num == 0:
+            continue
+        end_idx = start_idx + token_num
+        deep_gemm.fp8_gemm_nt(
+            (x_fp8[start_idx:end_idx], x_scale[start_idx:end_idx].contiguous()),
+            (w_fp8[i], w_scale[i]),
+            gemm_out[start_idx:end_idx],
+        )
+        start_idx = end_idx
+    return gemm_out
+
+
+class FP8LinearFunctionBase:
+    @staticmethod
+    def dequantize_fp8_to_fp32(fp8_tensor, scale):
+        """fp8_utils.py:136-138 (despite the name the reference returns bf16)."""
+        return F8.fused_act_dequant(fp8_tensor.reshape(-1, fp8_tensor.shape[-1]), scale.reshape(-1, scale.shape[-1])).reshape(fp8_tensor.shape)
+
+    @staticmethod
+    def padding(x, axis):
+        """fp8_utils.py:140-152: zero-pad `axis` up to the next multiple of 512."""
+        n = x.shape[axis]
+        if n % 512 != 0:
+            if (n + 128 - (n % 128)) % 512 != 0:
+                padding_size = 512
+            else:
+                padding_size = 128
+            pad_size = padding_size - (n % padding_size)
+            if axis == 0:
+                x = torch.cat([x, torch.zeros([pad_size, x.shape[-1]], dtype=x.dtype, device=x.device)], dim=0)
+            else:
+                x = torch.cat([x, torch.zeros([x.shape[0], pad_size], dtype=x.dtype, device=x.device)], dim=-1)
+        return x
+
+    @staticmethod
+    def padding_and_quant_input(tensor):
+        """fp8_utils.py:155-174: row-scaled copy of the input and column-scaled transposed copy of
+        the (zero-padded) input."""
+        if tensor.shape[0] % 512 != 0:
+            tensor_fp8, tensor_scale = F8.fp8_quant_blockwise(tensor, output_scale_transpose=True, quant_method="1x128",
+                                                              input_transpose=False)
+            tensor = FP8LinearFunctionBase.padding(tensor, 0)
+            tensor_t_fp8, tensor_t_scale = F8.fp8_quant_blockwise(tensor, output_scale_transpose=True, quant_method="1x128",
+                                                                  input_transpose=True, return_transpose_only=True)
+            return tensor_fp8, tensor_scale, tensor_t_fp8, tensor_t_scale
+        return F8.fp8_quant_blockwise(tensor, output_scale_transpose=True, quant_method="1x128", input_transpose=True)
+
+    @staticmethod
+    def kitchen_gemm(x_fp8, x_scale, w_fp8, w_scale, is_a_1d_scaled, is_b_1d_scaled, out=None, rtn_dtype=torch.bfloat16):
+        """fp8_utils.py:176-221: weight-gradient GEMM, accumulate when `out` is given; zero-sized
+        operands give zeros."""
+        if out is not None:
+            accumulate, out_dtype = True, out.dtype
+        else:
+            accumulate, out_dtype = False, rtn_dtype
+        if numpy.prod(x_fp8.shape) != 0 and numpy.prod(w_fp8.shape) != 0:
+            if out is None and out_dtype != torch.float32:
+                y = F8.fp8_gemm_blockwise(a=x_fp8, a_decode_scale=x_scale, b=w_fp8, b_decode_scale=w_scale, out_dtype=torch.float32,
+                                          out=None, accumulate=False, use_split_accumulator=True,
+                                          is_a_1d_scaled=is_a_1d_scaled, is_b_1d_scaled=is_b_1d_scaled)
+                return y.to(out_dtype)
+            return F8.fp8_gemm_blockwise(a=x_fp8, a_decode_scale=x_scale, b=w_fp8, b_decode_scale=w_scale, out_dtype=out_dtype,
+                                         out=out, accumulate=accumulate, use_split_accumulator=True,
+                                         is_a_1d_scaled=is_a_1d_scaled, is_b_1d_scaled=is_b_1d_scaled)
+        y = torch.zeros([x_fp8.shape[0], w_fp8.shape[0]], dtype=out_dtype, device=x_fp8.device)
+        if out is not None:
+            return out + y
+        return y
+
+    @staticmethod
+    def compute_fp8_linear(input, weight, weight_transpose=False, return_transpose_only=False, return_mode="output_only", *,
+                           out=None):
+        """fp8_utils.py:224-291: quantise the input (unless it already is a (fp8, scale) pair),
+        fetch or quantise the weight, run the NT GEMM.  return_mode selects the extra outputs."""
+        is_input_quantized = isinstance(input, (tuple, list)) and len(input) == 2
+        if is_input_quantized:
+            input_fp8, input_scale = input
+            if return_mode == "with_input_transpose_quant":
+                raise RuntimeError("Cannot return transposed quant if input is already quantized. Use raw input instead.")
+        else:
+            if return_mode == "with_input_transpose_quant":
+                input_fp8, input_scale, input_t_fp8, input_t_scale = FP8LinearFunctionBase.padding_and_quant_input(input)
+            else:
+                input_fp8, input_scale = F8.fp8_quant_blockwise(input, output_scale_transpose=True, quant_method="1x128",
+                                                                input_transpose=False, return_transpose_only=False)
+        weight_fp8, weight_scale = weight_quant(weight, weight_transpose)
+        if out is None:
+            out = torch.empty([input_fp8.shape[0], weight_fp8.shape[0]], dtype=weight.dtype, device=weight.device)
+        deep_gemm.set_num_sms(get_sm_num())
+        deep_gemm.fp8_gemm_nt((input_fp8, input_scale.T), (weight_fp8, weight_scale), out)
+        if return_mode == "output_only":
+            return out
+        if return_mode == "with_input_quant":
+            return (out, input_fp8, input_scale)
+        if return_mode == "with_input_transpose_quant":
+            return (out, input_t_fp8, input_t_scale)
+        raise RuntimeError(
+            f"Unsupported return_mode: {return_mode}. "
+            "Supported modes: 'output_only', 'with_input_quant', 'with_input_transpose_quant'"
+        )
+
+    @staticmethod
+    def compute_expert_w_grad(input_t, input_t_scale, dout_t, dout_t_scale, is_a_1d_scaled=True, is_b_1d_scaled=True, weight=None,
+                              rtn_dtype=torch.bfloat16):
+        """fp8_utils.py:293-350: accumulate one expert's weight gradient into weight.main_grad
+        (or weight.grad), optionally deferred through WeightGradStore."""
+        if input_t is None or numpy.prod(input_t.shape) == 0:
+            return None
+        if hasattr(weight, "main_grad"):
+            if weight.main_grad is None:
+                weight.main_grad = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device)
+            if WeightGradStore.enabled:
+                WeightGradStore.put(partial(FP8LinearFunctionBase.kitchen_gemm, input_t, input_t_scale, dout_t, dout_t_scale,
+                                            is_a_1d_scaled, is_b_1d_scaled, weight.main_grad, rtn_dtype))
+                result = None
+            else:
+                result = FP8LinearFunctionBase.kitchen_gemm(input_t, input_t_scale, dout_t, dout_t_scale, is_a_1d_scaled,
+                                                            is_b_1d_scaled, weight.main_grad, rtn_dtype)
+        else:
+            if getattr(weight, "grad", None) is None:
+                weight.grad = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device)
+            result = FP8LinearFunctionBase.kitchen_gemm(input_t, input_t_scale, dout_t, dout_t_scale, is_a_1d_scaled, is_b_1d_scaled,
+                                                        weight.grad, rtn_dtype)
+        if hasattr(weight, "_apply_backward_hook"):
+            weight._apply_backward_hook()
+        return result
+
+    @staticmethod
+    def fp8_mlp_fwd(x, w1, w2):
+        """fp8_utils.py:448-467: o1 = x.w1, o2 = swiglu(o1), o3 = o2.w2 with FP8 GEMMs."""
+        x_orig_shape = x.shape
+        x = x.reshape([-1, x_orig_shape[-1]])
+        o1, x_fp8, x_scale = FP8LinearFunctionBase.compute_fp8_linear(x, w1, weight_transpose=True, return_transpose_only=True,
+                                                                      return_mode="with_input_quant")
+        o2 = swiglu(o1)
+        o3 = FP8LinearFunctionBase.compute_fp8_linear(o2, w2, weight_transpose=True, return_transpose_only=True)
+        if len(x_orig_shape) > 2:
+            o3 = o3.reshape([x_orig_shape[0], -1, o3.shape[-1]])
+        return o1, x_fp8, x_scale, o3
+
+
+class FP8Mlp(torch.nn.Module):
+    """fp8_utils.py:806-850: SwiGLU MLP with w1 [H, 2I] and w2 [I, H] in bf16, FP8 forward."""
+
+    def __init__(self, hidden_size, intermediate_size, device=None):
+        super().__init__()
+        self.w1 = torch.nn.Parameter(torch.empty(hidden_size, intermediate_size * 2, dtype=torch.bfloat16, device=device))
+        self.w2 = torch.nn.Parameter(torch.empty(intermediate_size, hidden_size, dtype=torch.bfloat16, device=device))
+
+    def fp8_quant_weight(self, quant_transpose=None):
+        cache_fp8_weight(self.w1, quant_transpose)
+        cache_fp8_weight(self.w2, quant_transpose)
+
+    @torch.no_grad()
+    def forward(self, x):
+        return FP8LinearFunctionBase.fp8_mlp_fwd(x, self.w1, self.w2)[3]
+
+
+class FP8GroupGemmMlpFunctionNode:
+    """The fused FP8 MoE expert MLP (fp8_utils.py:873-1321).
+
+    forward : up+gate grouped GEMM -> fused SwiGLU*probs + 1x128 requant -> down grouped GEMM
+    backward: (recompute o1) -> dgrad-down grouped GEMM -> SwiGLU backward -> wgrad1 -> dgrad-up
+              grouped GEMM -> wgrad2
+    `custom_map.experts` is a list of objects with bf16 tensors `w1` [H, 2I] and `w2` [I, H]
+    (None entries are skipped).  Rows of the input are sorted by expert, each expert's segment
+    zero-padded to a multiple of 128 rows; tokens_per_expert holds the padded counts.
+    """
+
+    def __init__(self, custom_map, recompute_fwd_gate_up=False, is_split_group_gemm=False,
+                 name="experts_group_gemm_contiguous_node"):
+        self.experts = custom_map.experts
+        self.recompute_fwd_gate_up = recompute_fwd_gate_up
+        self.is_split_group_gemm = is_split_group_gemm
+        self.name = name
+        self.m_indices = None
+        self.input = None
+        self.input_fp8 = None
+        self.input_scale = None
+        self.o1 = None
+        self.all_unzipped_grad = None
+        self.fwd_subbatch = None
+        self.bwd_subbatch = None
+
+    def reset_statue(self):
+        self.m_indices = None
+        self.fwd_subbatch = None
+        self.bwd_subbatch = None
+        self.clear_activation_tensors()
+
+    def clear_activation_tensors(self):
+        self.input = None
+        self.input_fp8 = None
+        self.input_scale = None
+        self.o1 = None
+        self.all_unzipped_grad = None
+
+    def gen_m_indices(self, tokens_per_expert):
+        """fp8_utils.py:906-911: expert id of every (padded) row, int32."""
+        dev = self.experts[0].w1.device if self.experts and self.experts[0] is not None else "cuda"
+        counts = torch.tensor([int(t) for t in tokens_per_expert], dtype=torch.int64)
+        return torch.repeat_interleave(torch.arange(len(tokens_per_expert), dtype=torch.int32), counts).to(dev)
+
+    @staticmethod
+    def _stacked(expert_w, transpose, num_expert):
+        q, s = fused_stack_quant(expert_w, transpose=transpose)
+        q = q.reshape([num_expert, -1, q.shape[-1]])
+        s = s.reshape([num_expert, -1, s.shape[-1]])
+        w0 = expert_w[0]
+        want, other = ("fp8_weight_stacked_transpose", "fp8_weight_stacked") if transpose else ("fp8_weight_stacked", "fp8_weight_stacked_transpose")
+        if hasattr(w0, other) and not hasattr(w0, want):
+            q = q.contiguous().transpose(1, 2).contiguous()
+            s = s.contiguous().transpose(1, 2).contiguous()
+        return q, s
+
+    def fwd_gate_up(self, x, expert_w1, num_expert, tokens_per_expert, m_indices=None):
+        """o1 [m_sum, 2I] = x [m_sum, H] . w1 (fp8_utils.py:913-959)."""
+        if not self.is_split_group_gemm and self.m_indices is None:
+            self.m_indices = self.gen_m_indices(tokens_per_expert)
+        w1_t_quant, w1_t_scale = self._stacked(expert_w1, True, num_expert)
+        if x is None:
+            x_fp8, x_scale = self.input_fp8, self.input_scale
+            assert x_fp8 is not None and x_scale is not None
+        elif isinstance(x, tuple):
+            x_fp8, x_scale = x
+            x_scale = x_scale.t().contiguous().t()
+        else:
+            x_fp8, x_scale = F8.fp8_quant_blockwise(x, output_scale_transpose=True, quant_method="1x128", input_transpose=False)
+            x_scale = x_scale.T
+        o1 = torch.empty([x_fp8.shape[0], w1_t_quant.shape[1]], dtype=expert_w1[0].dtype, device=x_fp8.device)
+        if numpy.prod(x_fp8.shape) != 0:
+            if self.is_split_group_gemm:
+                split_group_gemm(x_fp8, x_scale, w1_t_quant, w1_t_scale, tokens_per_expert, o1)
+            else:
+                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((x_fp8, x_scale), (w1_t_quant, w1_t_scale), o1,
+                                                           self.m_indices if m_indices is None else m_indices)
+        if m_indices is None:
+            self.input_fp8 = x_fp8
+            self.input_scale = x_scale
+        return o1
+
+    def fwd_swiglu(self, o1):
+        return swiglu(o1)
+
+    def fwd_down(self, o1, unzipped_probs, expert_w2, num_expert, tokens_per_expert, m_indices=None, o3=None, clear_o1=False):
+        """o3 [m_sum, H] = quant(swiglu(o1) * probs) . w2 (fp8_utils.py:965-1009)."""
+        w2_quant, w2_scale = self._stacked(expert_w2, True, num_expert)
+        unzipped_probs = unzipped_probs.squeeze(-1)
+        o2_fp8, o2_scale = F8.fused_weighted_swiglu_act_quant(o1, unzipped_probs, using_pow2_scaling=True)
+        o3_shape = [o2_fp8.shape[0], w2_quant.shape[1]]
+        if o3 is not None:
+            assert list(o3.shape) == o3_shape, "{} vs {}".format(list(o3.shape), o3_shape)
+        else:
+            o3 = torch.empty(o3_shape, dtype=o1.dtype, device=o1.device)
+        if numpy.prod(o2_fp8.shape) != 0:
+            if self.is_split_group_gemm:
+                split_group_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, tokens_per_expert, o3)
+            else:
+                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2_fp8, o2_scale), (w2_quant, w2_scale), o3,
+                                                           m_indices if self.fwd_subbatch else self.m_indices)
+        return o3
+
+    def bwd_dowm_input(self, expert_w2, unzipped_grad, o1, tokens_per_expert, m_indices=None, unzipped_probs=None):
+        """do2_s [m_sum, I] = do3 . w2^T, then the SwiGLU backward (fp8_utils.py:1011-1052)."""
+        bw_w2_quant, bw_w2_scale = self._stacked(expert_w2, False, len(expert_w2))
+        if isinstance(unzipped_grad, tuple):
+            unzipped_grad_fp8, unzipped_grad_scale = unzipped_grad
+            unzipped_grad_scale = unzipped_grad_scale.t().contiguous().t()
+        else:
+            unzipped_grad_fp8, unzipped_grad_scale = F8.fp8_quant_blockwise(unzipped_grad, output_scale_transpose=True,
+                                                                            quant_method="1x128", input_transpose=False)
+            unzipped_grad_scale = unzipped_grad_scale.T
+        do2_s = torch.empty([unzipped_grad_fp8.shape[0], bw_w2_quant.shape[1]], dtype=torch.bfloat16, device=o1.device)
+        if numpy.prod(unzipped_grad_fp8.shape) != 0:
+            if self.is_split_group_gemm:
+                split_group_gemm(unzipped_grad_fp8, unzipped_grad_scale, bw_w2_quant, bw_w2_scale, tokens_per_expert, do2_s)
+            else:
+                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((unzipped_grad_fp8, unzipped_grad_scale), (bw_w2_quant, bw_w2_scale),
+                                                           do2_s, m_indices if self.bwd_subbatch else self.m_indices)
+        do1, probs_grad, o2_s = F8.fused_swiglu_weighted_bwd(o1, do2_s, unzipped_probs)
+        return do1, o2_s, probs_grad
+
+    def bwd_gate_up_input(self, do1, expert_w1, tokens_per_expert, m_indices=None, dx=None):
+        """dx [m_sum, H] = do1 . w1^T (fp8_utils.py:1058-1094)."""
+        bw_w1_quant, bw_w1_scale = self._stacked(expert_w1, False, len(expert_w1))
+        do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, output_scale_transpose=True, quant_method="1x128", input_transpose=False)
+        do1_scale = do1_scale.T
+        dx_shape = [do1_fp8.shape[0], bw_w1_quant.shape[1]]
+        if dx is None or dx.dtype != do1.dtype:
+            dx = torch.empty(dx_shape, dtype=do1.dtype, device=do1.device)
+        else:
+            assert list(dx.shape) == dx_shape, f"{list(dx.shape)} vs {dx_shape}"
+        if numpy.prod(do1_fp8.shape) != 0:
+            if self.is_split_group_gemm:
+                split_group_gemm(do1_fp8, do1_scale, bw_w1_quant, bw_w1_scale, tokens_per_expert, dx)
+            else:
+                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((do1_fp8, do1_scale), (bw_w1_quant, bw_w1_scale), dx,
+                                                           m_indices if self.bwd_subbatch else self.m_indices)
+        return dx
+
+    def fused_transpose_split_quant(self, x, scale, tokens_per_expert, pow_2_scales):
+        return F8.fused_transpose_split_quant(x, scale, tokens_per_expert, pow_2_scales)
+
+    @staticmethod
+    def _expert_wgrads(a_t, sa_t, b_t, sb_t, expert_w):
+        """Per-expert loop of fp8_utils.py:1117-1129 / :1170-1182."""
+        with torch.no_grad():
+            for i in range(len(expert_w)):
+                FP8LinearFunctionBase.compute_expert_w_grad(a_t[i], sa_t[i], b_t[i], sb_t[i], True, True, expert_w[i], torch.float32)
+
+    def bwd_down_weight(self, do3, o2, expert_w2, tokens_per_expert):
+        """dw2[e] [I, H] += o2_e^T . do3_e (fp8_utils.py:1102-1134)."""
+        if isinstance(o2, tuple):
+            o2_t_fp8, o2_t_scale = o2
+        else:
+            o2_t_fp8, o2_t_scale = self.fused_transpose_split_quant(o2, None, tokens_per_expert, True)
+        if isinstance(do3, tuple):
+            do3_t_fp8, do3_t_scale = do3
+        else:
+            do3_t_fp8, do3_t_scale = self.fused_transpose_split_quant(do3, None, tokens_per_expert, True)
+        fn = partial(self._expert_wgrads, o2_t_fp8, o2_t_scale, do3_t_fp8, do3_t_scale, expert_w2)
+        if WeightGradStore.enabled:
+            WeightGradStore.put(fn)
+        else:
+            fn()
+
+    def bwd_gate_up_weight(self, do1, input_x, expert_w1, tokens_per_expert, input_fp8_slice=None, input_scale_slice=None,
+                           clear_input=False):
+        """dw1[e] [H, 2I] += x_e^T . do1_e (fp8_utils.py:1136-1189)."""
+        if input_x is None:
+            inp = (input_fp8_slice, input_scale_slice) if self.bwd_subbatch else (self.input_fp8, self.input_scale)
+            input_x_t_fp8, input_x_t_scale = self.fused_transpose_split_quant(inp[0], inp[1], tokens_per_expert, True)
+        else:
+            input_x_t_fp8, input_x_t_scale = self.fused_transpose_split_quant(input_x, None, tokens_per_expert, True)
+        if clear_input:
+            self.input_fp8 = None
+            self.input_scale = None
+            self.input = None
+        do1_t_fp8, do1_t_scale = self.fused_transpose_split_quant(do1, None, tokens_per_expert, True)
+        fn = partial(self._expert_wgrads, input_x_t_fp8, input_x_t_scale, do1_t_fp8, do1_t_scale, expert_w1)
+        if WeightGradStore.enabled:
+            WeightGradStore.put(fn)
+        else:
+            fn()
+
+    @torch.no_grad()
+    def forward(self, hs_out, unzipped_probs, tokens_per_expert, m_indices=None):
+        """fp8_utils.py:1191-1232.  hs_out: bf16 [m_sum, H], a (fp8, scale) pair, or None to reuse
+        the cached quantised input.  Zero rows -> zeros."""
+        if self.fwd_subbatch:
+            assert m_indices is not None
+        dtype = torch.bfloat16
+        if hs_out is None:
+            assert self.input_fp8 is not None
+            assert self.input_scale is not None
+            shape, dev = self.input_fp8.shape, self.input_fp8.device
+        elif isinstance(hs_out, tuple):
+            shape, dev = hs_out[0].shape, hs_out[0].device
+        else:
+            shape, dev = hs_out.shape, hs_out.device
+        if shape[0] == 0:
+            return torch.zeros(list(shape), dtype=dtype, device=dev)
+        expert_w1 = [x.w1 for x in self.experts if x is not None]
+        expert_w2 = [x.w2 for x in self.experts if x is not None]
+        num_expert = len(expert_w1)
+        o1 = self.fwd_gate_up(hs_out, expert_w1, num_expert, tokens_per_expert, m_indices)
+        if not self.recompute_fwd_gate_up:
+            self.o1 = o1
+            clear_o1 = False
+        else:
+            clear_o1 = True
+        return self.fwd_down(o1, unzipped_probs, expert_w2, num_expert, tokens_per_expert, clear_o1=clear_o1, m_indices=m_indices)
+
+    @torch.no_grad()
+    def backward(self, out_grad, unzipped_probs, tokens_per_expert, input_fp8_slice=None, input_scale_slice=None, m_indices=None,
+                 reset_status=False):
+        """fp8_utils.py:1234-1321.  Returns (dx, probs_grad); weight gradients are accumulated
+        into each expert weight's main_grad (or grad)."""
+        if self.bwd_subbatch:
+            assert m_indices is not None and input_fp8_slice is not None and input_scale_slice is not None and tokens_per_expert is not None
+        dtype = torch.bfloat16
+        g0 = extract_first_if_tuple(out_grad)
+        if g0.shape[0] == 0:
+            return torch.zeros_like(g0, dtype=dtype), torch.zeros_like(unzipped_probs)
+        expert_w1 = [x.w1 for x in self.experts if x is not None]
+        expert_w2 = [x.w2 for x in self.experts if x is not None]
+        if self.recompute_fwd_gate_up:
+            inp = None if not self.bwd_subbatch else (input_fp8_slice, input_scale_slice)
+            o1 = self.fwd_gate_up(inp, expert_w1, len(expert_w1), tokens_per_expert, m_indices=m_indices)
+        else:
+            o1 = self.o1
+        do1, o2_s, probs_grad = self.bwd_dowm_input(expert_w2, out_grad, o1, tokens_per_expert, unzipped_probs=unzipped_probs,
+                                                    m_indices=m_indices)
+        del o1
+        self.o1 = None
+        self.bwd_gate_up_weight(do1, None, expert_w1, tokens_per_expert, input_fp8_slice=input_fp8_slice,
+                                input_scale_slice=input_scale_slice, clear_input=reset_status)
+        if reset_status:
+            self.input_fp8 = None
+            self.input_scale = None
+            self.input = None
+        dx = self.bwd_gate_up_input(do1, expert_w1, tokens_per_expert, dx=None, m_indices=m_indices)
+        del do1
+        if isinstance(out_grad, tuple):
+            do3_fp8, do3_scale = self.fused_transpose_split_quant(out_grad[0], out_grad[1], tokens_per_expert, True)
+            self.bwd_down_weight((do3_fp8, do3_scale), o2_s, expert_w2, tokens_per_expert)
+        else:
+            self.bwd_down_weight(out_grad, o2_s, expert_w2, tokens_per_expert)
+        if reset_status:
+            self.reset_statue()
+        return dx, probs_grad

@@ -1,0 +1,421 @@
+"""Drop-in replacements for the `paddle.incubate.nn.functional` FP8 operators the reference calls.
+
+Same names, keyword arguments, output shapes and scale conventions as the call sites in
+paddleformers/transformers/fp8_utils.py; tensors are device tensors (torch-ROCm here: bf16 =
+torch.bfloat16, e4m3 = torch.float8_e4m3fn, scales fp32) and every function launches a libpf8
+kernel on the current stream.  There is no CPU path: a CPU tensor raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+
+FP8 = torch.float8_e4m3fn
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t: torch.Tensor, what: str) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{what} must be a tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{what} must live on the GPU: libpf8 has no CPU path")
+    return t
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _as2d(x: torch.Tensor) -> torch.Tensor:
+    return x.reshape(-1, x.shape[-1])
+
+
+def _scale_layout_of(s: torch.Tensor, rows: int, blocks: int, what: str) -> Tuple[torch.Tensor, int]:
+    """A logical [rows, blocks] scale tensor -> (tensor, layout flag) without copying when its
+    memory is either row-major (0) or blocks-major, i.e. a transposed view of [blocks, rows] (1)."""
+    if tuple(s.shape) != (rows, blocks):
+        raise ValueError(f"{what} must have shape [{rows}, {blocks}], got {list(s.shape)}")
+    if s.dtype != torch.float32:
+        raise ValueError(f"{what} must be float32")
+    if s.is_contiguous():
+        return s, 0
+    if s.stride() == (1, rows):
+        return s, 1
+    return s.contiguous(), 0
+
+
+# ---------------------------------------------------------------------------------------------
+# fp8_quant_blockwise
+# ---------------------------------------------------------------------------------------------
+
+
+def fp8_quant_blockwise(
+    x: torch.Tensor,
+    quant_method: str = "1x128",
+    input_transpose: bool = False,
+    output_scale_transpose: bool = False,
+    return_transpose_only: bool = False,
+    using_pow2_scale: bool = False,
+):
+    """Block-wise e4m3 quantization, scale = amax/448 per tile.
+
+    Mirrors the keyword use at transformers/fp8_utils.py:112-131 (128x128 weights) and
+    :158-173, :262-268 (1x128 activations).  Returns (q, s), (q, s, q_t, s_t) when
+    input_transpose, or (q_t, s_t) when also return_transpose_only.
+    Scale shapes: 1x128 -> [M, K/128], or [K/128, M] with output_scale_transpose (transposed copy:
+    [K, M/128] / [M/128, K]); 128x128 -> [R/128, C/128] (transposed copy [C/128, R/128]).
+    """
+    _dev(x, "x")
+    if x.dtype != torch.bfloat16:
+        raise ValueError("fp8_quant_blockwise expects a bfloat16 tensor")
+    if return_transpose_only and not input_transpose:
+        raise ValueError("return_transpose_only requires input_transpose=True")
+    x2 = _as2d(x)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    M, K = x2.shape
+    pow2 = int(bool(using_pow2_scale))
+    dev = x.device
+    if quant_method == "1x128":
+        if K % 128 != 0:
+            raise ValueError(f"last dimension must be divisible by 128, got {K}")
+        lay = 1 if output_scale_transpose else 0
+        if not input_transpose:
+            q = torch.empty((M, K), dtype=FP8, device=dev)
+            s = torch.empty((K // 128, M) if lay else (M, K // 128), dtype=torch.float32, device=dev)
+            _lib.call("pf8_quant_1x128", _p(x2), M, K, K, _p(q), _p(s), lay, pow2, _stream())
+            return q.reshape(x.shape), s
+        if M % 128 != 0:
+            raise ValueError(f"input_transpose=True needs the row count to be a multiple of 128, got {M}")
+        q = s = None
+        if not return_transpose_only:
+            q = torch.empty((M, K), dtype=FP8, device=dev)
+            s = torch.empty((K // 128, M) if lay else (M, K // 128), dtype=torch.float32, device=dev)
+        q_t = torch.empty((K, M), dtype=FP8, device=dev)
+        s_t = torch.empty((M // 128, K) if lay else (K, M // 128), dtype=torch.float32, device=dev)
+        _lib.call("pf8_quant_transpose", _p(x2), M, K, _p(q), _p(s), _p(q_t), _p(s_t), lay, pow2, _stream())
+        if return_transpose_only:
+            return q_t, s_t
+        return q, s, q_t, s_t
+    if quant_method == "128x128":
+        if M % 128 != 0 or K % 128 != 0:
+            raise ValueError(f"128x128 quantization needs both dimensions divisible by 128, got [{M}, {K}]")
+        if output_scale_transpose:
+            raise ValueError("128x128 quantization has no output_scale_transpose layout")
+        q = s = q_t = s_t = None
+        if not return_transpose_only:
+            q = torch.empty((M, K), dtype=FP8, device=dev)
+            s = torch.empty((M // 128, K // 128), dtype=torch.float32, device=dev)
+        if input_transpose:
+            q_t = torch.empty((K, M), dtype=FP8, device=dev)
+            s_t = torch.empty((K // 128, M // 128), dtype=torch.float32, device=dev)
+        _lib.call("pf8_quant_128x128", _p(x2), M, K, _p(q), _p(s), _p(q_t), _p(s_t), pow2, _stream())
+        if return_transpose_only:
+            return q_t, s_t
+        if input_transpose:
+            return q, s, q_t, s_t
+        return q, s
+    raise ValueError(f"unsupported quant_method {quant_method!r} (expected '1x128' or '128x128')")
+
+
+# ---------------------------------------------------------------------------------------------
+# fused_stack_transpose_quant
+# ---------------------------------------------------------------------------------------------
+
+
+def fused_stack_transpose_quant(weight_list: Sequence[torch.Tensor], transpose: bool = False, using_pow2_scale: bool = False):
+    """Stack E bf16 [R, C] weights, optionally transposing each, and quantize in 128x128 tiles.
+
+    transformers/fp8_utils.py:101; un-fused equivalent ernie token_dispatcher/fp8_utils.py:276-287.
+    Returns q [E*R, C] (or [E*C, R] with transpose) and s [E*R/128, C/128] (or [E*C/128, R/128]).
+    """
+    if len(weight_list) == 0:
+        raise ValueError("weight_list is empty")
+    R, Cc = weight_list[0].shape
+    ws = []
+    for w in weight_list:
+        _dev(w, "weight")
+        if w.dtype != torch.bfloat16 or tuple(w.shape) != (R, Cc):
+            raise ValueError("all weights must be bfloat16 with the same 2-D shape")
+        ws.append(w if w.is_contiguous() else w.contiguous())
+    if R % 128 != 0 or Cc % 128 != 0:
+        raise ValueError(f"weight dimensions must be divisible by 128, got [{R}, {Cc}]")
+    E = len(ws)
+    dev = ws[0].device
+    if transpose:
+        q = torch.empty((E * Cc, R), dtype=FP8, device=dev)
+        s = torch.empty((E * Cc // 128, R // 128), dtype=torch.float32, device=dev)
+    else:
+        q = torch.empty((E * R, Cc), dtype=FP8, device=dev)
+        s = torch.empty((E * R // 128, Cc // 128), dtype=torch.float32, device=dev)
+    ptrs = (C.c_void_p * E)(*[w.data_ptr() for w in ws])
+    _lib.call("pf8_stack_transpose_quant", ptrs, E, R, Cc, int(bool(transpose)), _p(q), _p(s), int(bool(using_pow2_scale)), _stream())
+    return q, s
+
+
+# ---------------------------------------------------------------------------------------------
+# fused_weighted_swiglu_act_quant
+# ---------------------------------------------------------------------------------------------
+
+
+def fused_weighted_swiglu_act_quant(o1: torch.Tensor, probs: Optional[torch.Tensor] = None, using_pow2_scaling: bool = False,
+                                    return_o2: bool = False):
+    """quant_1x128( bf16( bf16(swiglu(o1)) * probs ) ) in one pass.
+
+    transformers/fp8_utils.py:984-986; un-fused equivalent ernie token_dispatcher/fp8_utils.py:996-1004.
+    o1 bf16 [M, 2I] with the gate in the first half; probs fp32 [M] (or [M, 1]) or None.
+    Returns (q [M, I], s [M, I/128]); with return_o2 also the bf16 activations before quantization.
+    """
+    _dev(o1, "o1")
+    if o1.dtype != torch.bfloat16 or o1.dim() != 2:
+        raise ValueError("o1 must be a 2-D bfloat16 tensor")
+    if not o1.is_contiguous():
+        o1 = o1.contiguous()
+    M, I2 = o1.shape
+    if I2 % 256 != 0:
+        raise ValueError(f"o1 last dimension must be a multiple of 256, got {I2}")
+    I = I2 // 2
+    if probs is not None:
+        _dev(probs, "probs")
+        probs = probs.reshape(-1)
+        if probs.numel() != M:
+            raise ValueError("probs must have one entry per row of o1")
+        if probs.dtype != torch.float32:
+            probs = probs.float()
+        probs = probs.contiguous()
+    q = torch.empty((M, I), dtype=FP8, device=o1.device)
+    s = torch.empty((M, I // 128), dtype=torch.float32, device=o1.device)
+    o2 = torch.empty((M, I), dtype=torch.bfloat16, device=o1.device) if return_o2 else None
+    _lib.call("pf8_swiglu_weighted_quant", _p(o1), _p(probs), M, I, _p(q), _p(s), _p(o2), 0, int(bool(using_pow2_scaling)), _stream())
+    return (q, s, o2) if return_o2 else (q, s)
+
+
+# ---------------------------------------------------------------------------------------------
+# fused_transpose_split_quant
+# ---------------------------------------------------------------------------------------------
+
+
+def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], tokens_per_expert: Sequence[int],
+                                pow_2_scales: bool = False) -> Tuple[List[torch.Tensor], List[torch.Tensor]]:
+    """Per-expert split along rows -> transpose -> 1x128 quantization along the token axis.
+
+    transformers/fp8_utils.py:1096-1100; un-fused equivalent ernie token_dispatcher/fp8_utils.py:1199-1210.
+    x is bf16 [sum(M_e), K], or e4m3 with its [sum(M_e), K/128] scales (dequantized to bf16 first).
+    Returns lists with one q_t [K, M_e] and one s_t [M_e/128, K] per expert (empty tensors for
+    experts without rows).
+    """
+    _dev(x, "x")
+    if x.dim() != 2:
+        raise ValueError("x must be 2-D")
+    if not x.is_contiguous():
+        x = x.contiguous()
+    Mtot, K = x.shape
+    rows = [int(t) for t in tokens_per_expert]
+    if sum(rows) != Mtot:
+        raise ValueError(f"tokens_per_expert sums to {sum(rows)} but x has {Mtot} rows")
+    if any(r % 128 != 0 or r < 0 for r in rows):
+        raise ValueError("every tokens_per_expert entry must be a non-negative multiple of 128")
+    if K % 128 != 0:
+        raise ValueError(f"last dimension must be divisible by 128, got {K}")
+    is_fp8 = x.dtype == FP8
+    xs_layout = 0
+    if is_fp8:
+        if scale is None:
+            raise ValueError("an e4m3 input needs its scale tensor")
+        _dev(scale, "scale")
+        scale, xs_layout = _scale_layout_of(scale, Mtot, K // 128, "scale")
+    elif x.dtype != torch.bfloat16:
+        raise ValueError("x must be bfloat16 or float8_e4m3fn")
+    E = len(rows)
+    q_t = torch.empty((K * Mtot,), dtype=FP8, device=x.device)
+    s_t = torch.empty(((Mtot // 128) * K,), dtype=torch.float32, device=x.device)
+    for e0 in range(0, E, 256):
+        chunk = rows[e0:e0 + 256]
+        off = sum(rows[:e0])
+        n = sum(chunk)
+        arr = (C.c_int64 * len(chunk))(*chunk)
+        xs_ptr, lay, keep = None, 0, None
+        if is_fp8:
+            if n == Mtot:
+                xs_ptr, lay = _p(scale), xs_layout
+            else:
+                # more than 256 experts: hand each chunk its own row-major slice of the scales
+                keep = scale[off:off + n].contiguous()
+                xs_ptr, lay = _p(keep), 0
+        xp = C.c_void_p(x.data_ptr() + off * K * x.element_size())
+        qp = C.c_void_p(q_t.data_ptr() + off * K)
+        sp = C.c_void_p(s_t.data_ptr() + (off // 128) * K * 4)
+        _lib.call("pf8_transpose_split_quant", xp, xs_ptr, int(is_fp8), lay, arr, len(chunk), K, qp, sp, int(bool(pow_2_scales)), _stream())
+    qs, ss, off = [], [], 0
+    for r in rows:
+        qs.append(q_t[off * K:(off + r) * K].view(K, r))
+        ss.append(s_t[(off // 128) * K:((off + r) // 128) * K].view(r // 128, K))
+        off += r
+    return qs, ss
+
+
+# ---------------------------------------------------------------------------------------------
+# dequantizers
+# ---------------------------------------------------------------------------------------------
+
+
+def fused_act_dequant(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """1x128 dequantization to bf16: bf16(float(q) * s).  transformers/fp8_utils.py:136-138, :779."""
+    _dev(q, "q")
+    _dev(scale, "scale")
+    if q.dtype != FP8 or q.dim() != 2:
+        raise ValueError("q must be a 2-D float8_e4m3fn tensor")
+    if not q.is_contiguous():
+        q = q.contiguous()
+    M, K = q.shape
+    if K % 128 != 0:
+        raise ValueError(f"last dimension must be divisible by 128, got {K}")
+    scale, lay = _scale_layout_of(scale, M, K // 128, "scale")
+    out = torch.empty((M, K), dtype=torch.bfloat16, device=q.device)
+    _lib.call("pf8_act_dequant", _p(q), _p(scale), lay, M, K, _p(out), _stream())
+    return out
+
+
+def weight_dequant(q: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> torch.Tensor:
+    """128x128 dequantization to bf16.  cli/train/deepseek_v3_pretrain/kernel.py:100-118 (same
+    asserts: contiguous, 2-D); quantization/checkpoint_dequant.py:277-292 for ragged edges."""
+    _dev(q, "x")
+    _dev(s, "s")
+    assert q.is_contiguous() and s.is_contiguous(), "Input tensors must be contiguous"
+    assert q.dim() == 2 and s.dim() == 2, "Input tensors must have 2 dimensions"
+    if block_size != 128:
+        raise ValueError("only block_size=128 is supported")
+    if q.dtype not in (FP8, torch.uint8, torch.int8):
+        raise ValueError("x must hold e4m3 codes (float8_e4m3fn, uint8 or int8 storage)")
+    R, Cc = q.shape
+    if tuple(s.shape) != ((R + 127) // 128, (Cc + 127) // 128) or s.dtype != torch.float32:
+        raise ValueError("s must be float32 [ceil(R/128), ceil(C/128)]")
+    out = torch.empty((R, Cc), dtype=torch.bfloat16, device=q.device)
+    _lib.call("pf8_weight_dequant", _p(q), _p(s), R, Cc, _p(out), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# fused_swiglu_weighted_bwd
+# ---------------------------------------------------------------------------------------------
+
+
+def fused_swiglu_weighted_bwd(o1: torch.Tensor, do2_s: torch.Tensor, probs: torch.Tensor):
+    """SwiGLU backward with per-row probs.  transformers/fp8_utils.py:1050; un-fused equivalent
+    ernie token_dispatcher/fp8_utils.py:1088-1092.  Returns (do1 [M,2I] bf16, probs_grad [M] fp32,
+    o2_s [M,I] bf16)."""
+    for t, n in ((o1, "o1"), (do2_s, "do2_s"), (probs, "probs")):
+        _dev(t, n)
+    if o1.dtype != torch.bfloat16 or do2_s.dtype != torch.bfloat16:
+        raise ValueError("o1 and do2_s must be bfloat16")
+    o1 = o1.contiguous()
+    do2_s = do2_s.contiguous()
+    M, I2 = o1.shape
+    I = I2 // 2
+    if tuple(do2_s.shape) != (M, I):
+        raise ValueError(f"do2_s must be [{M}, {I}]")
+    if I % 8 != 0:
+        raise ValueError("I must be a multiple of 8")
+    probs = probs.reshape(-1).float().contiguous()
+    if probs.numel() != M:
+        raise ValueError("probs must have one entry per row")
+    do1 = torch.empty((M, I2), dtype=torch.bfloat16, device=o1.device)
+    pg = torch.empty((M,), dtype=torch.float32, device=o1.device)
+    o2s = torch.empty((M, I), dtype=torch.bfloat16, device=o1.device)
+    _lib.call("pf8_swiglu_weighted_bwd", _p(o1), _p(do2_s), _p(probs), M, I, _p(do1), _p(pg), _p(o2s), _stream())
+    return do1, pg, o2s
+
+
+# ---------------------------------------------------------------------------------------------
+# fp8_gemm_blockwise (weight-gradient GEMM)
+# ---------------------------------------------------------------------------------------------
+
+
+def fp8_gemm_blockwise(a, a_decode_scale, b, b_decode_scale, out_dtype=torch.float32, out=None, accumulate=False,
+                       use_split_accumulator=True, is_a_1d_scaled=True, is_b_1d_scaled=True):
+    """y[Ka, Nb] (+)= a[Ka, M] . b[Nb, M]^T with both operands 1x128-scaled along M.
+
+    transformers/fp8_utils.py:203-214 (kitchen_gemm): a_decode_scale [M/128, Ka], b_decode_scale
+    [M/128, Nb]; fp32 output; accumulate adds into `out`.
+    """
+    if not (is_a_1d_scaled and is_b_1d_scaled):
+        raise ValueError("only the 1x128-by-1x128 scaled form is implemented (is_a_1d_scaled = is_b_1d_scaled = True)")
+    for t, n in ((a, "a"), (b, "b"), (a_decode_scale, "a_decode_scale"), (b_decode_scale, "b_decode_scale")):
+        _dev(t, n)
+    if a.dtype != FP8 or b.dtype != FP8:
+        raise ValueError("a and b must be float8_e4m3fn")
+    a, b = a.contiguous(), b.contiguous()
+    Ka, M = a.shape
+    Nb, M2 = b.shape
+    if M != M2 or M % 128 != 0:
+        raise ValueError("a and b must share a reduction length that is a multiple of 128")
+    sa = a_decode_scale.contiguous()
+    sb = b_decode_scale.contiguous()
+    if tuple(sa.shape) != (M // 128, Ka) or tuple(sb.shape) != (M // 128, Nb):
+        raise ValueError("decode scales must be [M/128, rows]")
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate=True needs out")
+        if out_dtype != torch.float32:
+            raise ValueError("the weight-gradient GEMM produces float32")
+        out = torch.empty((Ka, Nb), dtype=torch.float32, device=a.device)
+    else:
+        if out.dtype != torch.float32 or tuple(out.shape) != (Ka, Nb) or not out.is_contiguous():
+            raise ValueError("out must be a contiguous float32 [Ka, Nb] tensor")
+    _lib.call("pf8_gemm_nt_1d1d_f32", _p(a), _p(sa), _p(b), _p(sb), Ka, Nb, M, _p(out), int(bool(accumulate)), _stream())
+    return out
+
+
+def grouped_wgrad(a_t_list, sa_t_list, b_t_list, sb_t_list, out: torch.Tensor, accumulate: bool = True):
+    """All experts' weight gradients in one launch: out[e] (+)= a_t[e] . b_t[e]^T.
+
+    Replaces the per-expert Python loops of transformers/fp8_utils.py:1117-1129 and :1170-1182.
+    The lists must be the outputs of fused_transpose_split_quant (views of one packed buffer).
+    """
+    E = len(a_t_list)
+    rows = [int(t.shape[1]) for t in a_t_list]
+    Kin = int(a_t_list[0].shape[0])
+    N = int(b_t_list[0].shape[0])
+    if tuple(out.shape) != (E, Kin, N) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise ValueError("out must be a contiguous float32 [E, Kin, N] tensor")
+
+    def base(lst):
+        t0 = lst[0]
+        st = t0.untyped_storage()
+        p = st.data_ptr() + t0.storage_offset() * t0.element_size()
+        # verify the packing: each tensor must start where the previous one ends
+        exp = p
+        for t in lst:
+            if t.numel() and t.data_ptr() != exp:
+                raise ValueError("operands are not the packed outputs of fused_transpose_split_quant")
+            exp += t.numel() * t.element_size()
+        return C.c_void_p(p)
+
+    arr = (C.c_int64 * E)(*rows)
+    _lib.call("pf8_grouped_wgrad", base(a_t_list), base(sa_t_list), base(b_t_list), base(sb_t_list), arr, E, Kin, N, _p(out),
+              int(bool(accumulate)), _stream())
+    return out
+
+
+def swiglu(x: torch.Tensor, y: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16 SwiGLU with the kernel's arithmetic: silu(x[:, :I]) * x[:, I:].  transformers/fp8_utils.py:23-29."""
+    if y is not None:
+        x = torch.cat([x, y], dim=-1)
+    _dev(x, "x")
+    x2 = _as2d(x).contiguous()
+    M, I2 = x2.shape
+    I = I2 // 2
+    if I % 128 != 0:
+        raise ValueError("swiglu needs a half width that is a multiple of 128")
+    q = torch.empty((M, I), dtype=FP8, device=x.device)
+    s = torch.empty((M, I // 128), dtype=torch.float32, device=x.device)
+    o2 = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+    _lib.call("pf8_swiglu_weighted_quant", _p(x2), None, M, I, _p(q), _p(s), _p(o2), 0, 0, _stream())
+    return o2.reshape(*x.shape[:-1], I)
