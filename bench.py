@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 MoE hot path on one MI355X.
+
+One "step" = one forward pass of the DeepSeek-V3-shaped FP8 MoE expert MLP over one batch of
+synthetic routed tokens (BASELINE config 3, one GPU's local share):
+    1x128 quant of X -> up+gate grouped GEMM -> fused SwiGLU + 1x128 requant -> down grouped GEMM.
+Expert weights are quantised once before the timed region (the reference re-quantises them once
+per optimizer step in a callback, outside the MoE forward); that kernel is reported separately.
+
+Prints ONE JSON line.  `value` is algorithmic TFLOP/s of the whole step (padded rows not counted),
+`roofline` describes the dominant kernel (the up+gate grouped GEMM), `cpu_baseline` is the CPU
+oracle timed on a bounded sample of the same pipeline, `quant` lists the bandwidth-bound
+quantizers (GB/s against 8 TB/s HBM) measured on rotating buffers larger than the 256 MB
+Infinity Cache.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FP8_PEAK_TFLOPS = 5000.0
+
+
+def zipf_counts(total, E, s, seed, n_empty=2, pad=128):
+    import numpy as np
+
+    rng = np.random.default_rng(seed)
+    p = np.arange(1, E + 1, dtype=np.float64) ** (-s)
+    if n_empty:
+        p[-n_empty:] = 0.0
+    p /= p.sum()
+    perm = rng.permutation(E)
+    pe = np.empty(E)
+    pe[perm] = p
+    counts = rng.multinomial(total, pe)
+    return counts.astype(np.int64), (((counts + pad - 1) // pad) * pad).astype(np.int64)
+
+
+def time_kernel(fn, sets, iters, warmup):
+    """Median-free average time (ms) of fn(*sets[i % len(sets)]) over `iters` launches, with
+    HIP events on the launch stream."""
+    import torch
+
+    for i in range(warmup):
+        fn(*sets[i % len(sets)])
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(iters):
+        fn(*sets[i % len(sets)])
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def bench_quantizers(iters=20, warmup=5):
+    """GB/s of the bandwidth-bound quantizers on BASELINE configs 1, 3 (SwiGLU) and 4."""
+    import torch
+
+    from paddleformers_amd import functional as F8
+
+    out = {}
+
+    def mk(shape, n, std=1.0):
+        return [(torch.randn(shape, device="cuda", dtype=torch.float32) * std).to(torch.bfloat16) for _ in range(n)]
+
+    # C1a: 1x128 on [4096, 7168]
+    xs = mk((4096, 7168), 6)
+    ms = time_kernel(lambda x: F8.fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True), [(x,) for x in xs], iters, warmup)
+    out["quant_1x128_4096x7168"] = {"bytes": 88997888, "ms": ms}
+    del xs
+    # C1b: 128x128 on [7168, 2048]
+    ws = mk((7168, 2048), 10, 0.02)
+    ms = time_kernel(lambda w: F8.fp8_quant_blockwise(w, quant_method="128x128"), [(w,) for w in ws], iters, warmup)
+    out["quant_128x128_7168x2048"] = {"bytes": 44043776, "ms": ms}
+    del ws
+    # C3-q: fused SwiGLU + requant on [8192, 4096]
+    os_ = mk((8192, 4096), 5)
+    ms = time_kernel(lambda o: F8.fused_weighted_swiglu_act_quant(o, None, using_pow2_scaling=False), [(o,) for o in os_], iters, warmup)
+    out["swiglu_quant_8192x4096"] = {"bytes": 84443136 - 32768, "ms": ms}
+    del os_
+    # C4: fused quant + transpose on [16384, 7168]
+    xs = mk((16384, 7168), 2)
+    ms = time_kernel(lambda x: F8.fp8_quant_blockwise(x, quant_method="1x128", input_transpose=True, output_scale_transpose=True),
+                     [(x,) for x in xs], iters, warmup)
+    out["quant_transpose_16384x7168"] = {"bytes": 477102080, "ms": ms}
+    del xs
+    torch.cuda.empty_cache()
+    for v in out.values():
+        v["GBps"] = v["bytes"] / (v["ms"] * 1e-3) / 1e9
+        v["frac_hbm"] = v["GBps"] / HBM_PEAK_GBS
+        v["ms"] = round(v["ms"], 5)
+        v["GBps"] = round(v["GBps"], 1)
+        v["frac_hbm"] = round(v["frac_hbm"], 4)
+    return out
+
+
+def cpu_baseline(H, I, rows=256):
+    """The CPU oracle on a bounded sample of the same pipeline: `rows` token rows of ONE expert
+    (quant -> up+gate GEMM -> SwiGLU+requant -> down GEMM), OpenMP over the host cores."""
+    import numpy as np
+
+    from oracle import pf8_oracle as O
+
+    rng = np.random.default_rng(0)
+    x = O.f32_to_bf16_bits(rng.standard_normal((rows, H), dtype=np.float32))
+    w1 = O.f32_to_bf16_bits(rng.standard_normal((H, 2 * I), dtype=np.float32) * np.float32(0.02))
+    w2 = O.f32_to_bf16_bits(rng.standard_normal((I, H), dtype=np.float32) * np.float32(0.02))
+    w1q, w1s = O.stack_transpose_quant([w1], transpose=True)
+    w2q, w2s = O.stack_transpose_quant([w2], transpose=True)
+    t0 = time.perf_counter()
+    xq, xs = O.quant_1x128(x, 0)
+    o1 = O.gemm_nt(xq, xs, w1q, w1s)
+    o2q, o2s = O.swiglu_weighted_quant(o1, None, 0, False)
+    O.gemm_nt(o2q, o2s, w2q, w2s)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * rows * H * 2 * I + 2.0 * rows * I * H
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    return {"value": round(flops / dt / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{rows} token rows of one expert through quant/up+gate GEMM/SwiGLU+requant/down GEMM ({flops / 1e9:.1f} GFLOP, {dt:.1f} s)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-quant", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path uses no collectives and the run has a single MI355X; use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from paddleformers_amd import _lib, deep_gemm
+    from paddleformers_amd import functional as F8
+
+    _lib.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    torch.manual_seed(3)
+
+    E, H, I, ROUTED = 32, 7168, 2048, 8192
+    counts, padded = zipf_counts(ROUTED, E, 1.1, seed=3)
+    Mpad = int(padded.sum())
+    m_idx = torch.from_numpy(np.repeat(np.arange(E, dtype=np.int32), padded)).cuda()
+
+    # synthetic inputs: X ~ N(0,1) in the routed rows, zeros in the padding rows
+    x = torch.zeros((Mpad, H), dtype=torch.bfloat16, device="cuda")
+    off = 0
+    for e in range(E):
+        c = int(counts[e])
+        if c:
+            x[off:off + c] = torch.randn((c, H), device="cuda").to(torch.bfloat16)
+        off += int(padded[e])
+    w1q = torch.empty((E, 2 * I, H), dtype=torch.float8_e4m3fn, device="cuda")
+    w1s = torch.empty((E, 2 * I // 128, H // 128), dtype=torch.float32, device="cuda")
+    w2q = torch.empty((E, H, I), dtype=torch.float8_e4m3fn, device="cuda")
+    w2s = torch.empty((E, H // 128, I // 128), dtype=torch.float32, device="cuda")
+    t_wq = 0.0
+    for e in range(E):   # quantise expert by expert to keep the bf16 masters out of memory
+        w1 = (torch.randn((H, 2 * I), device="cuda") * 0.02).to(torch.bfloat16)
+        w2 = (torch.randn((I, H), device="cuda") * 0.02).to(torch.bfloat16)
+        q, s = F8.fused_stack_transpose_quant([w1], transpose=True)
+        w1q[e], w1s[e] = q.view(2 * I, H), s.view(2 * I // 128, H // 128)
+        q, s = F8.fused_stack_transpose_quant([w2], transpose=True)
+        w2q[e], w2s[e] = q.view(H, I), s.view(H // 128, I // 128)
+    torch.cuda.synchronize()
+
+    o1 = torch.empty((Mpad, 2 * I), dtype=torch.bfloat16, device="cuda")
+    o3 = torch.empty((Mpad, H), dtype=torch.bfloat16, device="cuda")
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+
+    def step(evs=None):
+        if evs: evs[0].record()
+        xq, xs = F8.fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True)
+        if evs: evs[1].record()
+        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((xq, xs.T), (w1q, w1s), o1, m_idx)
+        if evs: evs[2].record()
+        o2q, o2s = F8.fused_weighted_swiglu_act_quant(o1, None, using_pow2_scaling=False)
+        if evs: evs[3].record()
+        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2q, w2s), o3, m_idx)
+        if evs: evs[4].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(ev[k])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    names = ["quant_x", "gemm_up_gate", "swiglu_requant", "gemm_down"]
+    kms = {n: sum(ev[k][i].elapsed_time(ev[k][i + 1]) for k in range(args.steps)) / args.steps for i, n in enumerate(names)}
+
+    flops_up = 2.0 * ROUTED * H * 2 * I
+    flops_down = 2.0 * ROUTED * I * H
+    flops = flops_up + flops_down
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    ach = flops_up / (kms["gemm_up_gate"] * 1e-3) / 1e12
+
+    res = {
+        "metric": "FP8 MoE grouped-GEMM TFLOP/s + block-quant GB/s on 1 MI355X (% of peak)",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3 (fp32 accumulate, bf16 out)",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE config 3: DeepSeek-V3-shaped MoE FP8 forward, one GPU's local share",
+            "experts": E, "hidden": H, "moe_intermediate": I, "routed_rows": ROUTED, "padded_rows": Mpad,
+            "zipf_s": 1.1, "empty_experts": int((counts == 0).sum()),
+            "pipeline": "quant_1x128(X) -> grouped GEMM up+gate -> fused SwiGLU+requant -> grouped GEMM down",
+        },
+        "frac_fp8_peak": round(value / FP8_PEAK_TFLOPS, 4),
+        "kernel_ms": {k: round(v, 4) for k, v in kms.items()},
+        "roofline": {
+            "kernel": "k_gemm<fwd> (up+gate grouped GEMM)",
+            "bound": "mfma",
+            "achieved": round(ach, 2),
+            "peak": FP8_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(ach / FP8_PEAK_TFLOPS, 4),
+            "traffic": None,
+        },
+    }
+    if not args.no_quant:
+        res["quant"] = bench_quantizers()
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(H, I)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -118,21 +118,16 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const GemmArgs a) {
         lofs[i] = swz(row, cchunk);
     }
     uint4 rp[4], rq[4];
-    auto g_load = [&](int64_t kb) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            rp[i] = *reinterpret_cast<const uint4*>(gp[i] + kb * 128);
-            rq[i] = *reinterpret_cast<const uint4*>(gq[i] + kb * 128);
-        }
-    };
-    auto l_store = [&](int stage) {
-        uint8_t* base = lds + stage * 32768;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<uint4*>(base + lofs[i]) = rp[i];
-            *reinterpret_cast<uint4*>(base + 16384 + lofs[i]) = rq[i];
-        }
-    };
+#define PF8_G_LOAD(kb_)                                                          \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                              \
+        rp[i] = *reinterpret_cast<const uint4*>(gp[i] + (kb_) * 128);            \
+        rq[i] = *reinterpret_cast<const uint4*>(gq[i] + (kb_) * 128);            \
+    }
+#define PF8_L_STORE(stage_)                                                      \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                              \
+        *reinterpret_cast<uint4*>(lds + (stage_) * 32768 + lofs[i]) = rp[i];     \
+        *reinterpret_cast<uint4*>(lds + (stage_) * 32768 + 16384 + lofs[i]) = rq[i]; \
+    }
 
     // ---- fragment addresses --------------------------------------------------------------------
     int fofs_p[4][2], fofs_q[4][2];
@@ -187,15 +182,17 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const GemmArgs a) {
         for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     if (KBn > 0) {
-        g_load(0);
-        l_store(0);
+        PF8_G_LOAD(0)
+        PF8_L_STORE(0)
     }
     __syncthreads();
 
     for (int64_t kb = 0; kb < KBn; ++kb) {
         const int cur = (int)(kb & 1);
-        const bool more = kb + 1 < KBn;
-        if (more) g_load(kb + 1);
+        // prefetch the next K block into registers (the last iteration re-reads its own block:
+        // no branch, so the staging registers never leave the register file)
+        const int64_t kbn = kb + 1 < KBn ? kb + 1 : kb;
+        PF8_G_LOAD(kbn)
         s_load(kb);
         const uint8_t* base = lds + cur * 32768;
         i32x8 pf[4];
@@ -223,7 +220,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const GemmArgs a) {
                 }
             }
         }
-        if (more) l_store(cur ^ 1);
+        PF8_L_STORE(cur ^ 1)
         __syncthreads();
     }
 
