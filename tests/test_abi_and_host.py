@@ -1,0 +1,131 @@
+"""CPU-only checks of the boundary: libpf8.so loads and exports every symbol include/pf8.h
+declares, the ctypes table matches the header's arity, argument validation rejects bad input
+without touching a GPU, and the host-side mirror raises instead of falling back."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_decls():
+    text = open(os.path.join(ROOT, "include", "pf8.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = {}
+    for m in re.finditer(r"\b(?:int|const char\*)\s+(pf8_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        args = m.group(2).strip()
+        n = 0 if args in ("", "void") else len([a for a in args.split(",") if a.strip()])
+        decls[m.group(1)] = n
+    return decls
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from paddleformers_amd import _lib
+
+    return _lib.lib()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    decls = _header_decls()
+    assert len(decls) >= 20
+    for name in decls:
+        assert hasattr(lib, name), f"{name} declared in include/pf8.h but not exported"
+
+
+def test_ctypes_table_matches_header_arity():
+    from paddleformers_amd import _lib
+
+    decls = _header_decls()
+    for name, argtypes in _lib.SIGNATURES.items():
+        assert name in decls, f"{name} bound in _lib.py but not declared"
+        assert len(argtypes) == decls[name], f"{name}: {len(argtypes)} bound arguments vs {decls[name]} declared"
+    assert set(decls) - set(_lib.SIGNATURES) == {"pf8_last_error"}
+
+
+def test_version_and_cu_budget(lib):
+    assert lib.pf8_version() >= 100
+    prev = lib.pf8_set_num_cus(112)
+    assert lib.pf8_get_num_cus() == 112
+    lib.pf8_set_num_cus(prev)
+    assert lib.pf8_get_num_cus() == prev
+
+
+def test_argument_validation_without_a_gpu(lib):
+    """Every rejection happens before any launch, so it can be exercised on a CPU-only host."""
+    from paddleformers_amd import _lib
+
+    buf = (C.c_char * 64)()
+    p = C.cast(buf, C.c_void_p)
+    aligned = C.c_void_p((p.value + 15) & ~15)
+    # K not a multiple of 128
+    assert lib.pf8_quant_1x128(aligned, 4, 100, 100, aligned, aligned, 0, 0, None) == -1
+    assert "multiple of 128" in _lib.last_error()
+    # null pointers
+    assert lib.pf8_quant_1x128(None, 4, 128, 128, aligned, aligned, 0, 0, None) == -1
+    # misaligned pointer
+    assert lib.pf8_quant_1x128(C.c_void_p(aligned.value + 2), 4, 128, 128, aligned, aligned, 0, 0, None) == -1
+    # bad layout flag
+    assert lib.pf8_quant_1x128(aligned, 4, 128, 128, aligned, aligned, 7, 0, None) == -1
+    # zero-sized problems are legal no-ops
+    assert lib.pf8_quant_1x128(None, 0, 128, 128, None, None, 0, 0, None) == 0
+    assert lib.pf8_gemm_nt(None, None, 0, None, None, 0, 128, 128, None, 128, None) == 0
+    assert lib.pf8_grouped_gemm_nt_contiguous(None, None, 0, None, None, 4, 0, 128, 128, None, None, None) == 0
+    # grouped: rows not padded to 128
+    assert lib.pf8_grouped_gemm_nt_contiguous(aligned, aligned, 0, aligned, aligned, 1, 100, 128, 128, aligned, aligned, None) == -1
+    rows = (C.c_int64 * 2)(128, 100)
+    assert lib.pf8_transpose_split_quant(aligned, None, 0, 0, rows, 2, 128, aligned, aligned, 0, None) == -1
+    assert lib.pf8_grouped_wgrad(aligned, aligned, aligned, aligned, rows, 2, 128, 128, aligned, 1, None) == -1
+    # q/s must come as pairs
+    assert lib.pf8_quant_128x128(aligned, 128, 128, aligned, None, None, None, 0, None) == -1
+
+
+def test_cpu_tensors_raise_instead_of_falling_back():
+    from paddleformers_amd import deep_gemm
+    from paddleformers_amd import functional as F8
+
+    x = torch.zeros((128, 128), dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        F8.fp8_quant_blockwise(x, quant_method="1x128")
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        F8.fused_stack_transpose_quant([x])
+    q = torch.zeros((128, 128), dtype=torch.float8_e4m3fn)
+    s = torch.ones((128, 1))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        deep_gemm.fp8_gemm_nt((q, s), (q, torch.ones((1, 1))), torch.zeros((128, 128), dtype=torch.bfloat16))
+
+
+def test_product_package_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "paddleformers_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.replace("CPU checker", ""), f"{f} mentions the oracle"
+
+
+def test_padding_rule_matches_the_reference_branches():
+    """transformers/fp8_utils.py:140-152 always lands on the next multiple of 512."""
+    from paddleformers_amd.fp8_utils import FP8LinearFunctionBase as B
+
+    for n in (1, 127, 128, 129, 300, 384, 385, 511, 512, 513, 640, 900, 1024, 1100):
+        out = B.padding(torch.ones((n, 4)), 0)
+        exp = n if n % 512 == 0 else (n // 512 + 1) * 512
+        assert out.shape[0] == exp, (n, out.shape[0], exp)
+        assert torch.equal(out[:n], torch.ones((n, 4))) and (out[n:] == 0).all()
+        out = B.padding(torch.ones((4, n)), 1)
+        assert out.shape[1] == exp
+
+
+def test_zipf_expert_counts_generator():
+    from tests import _gen as G
+
+    counts, padded = G.zipf_counts(8192, 32, 1.1, seed=3)
+    assert counts.sum() == 8192 and (counts == 0).sum() >= 2
+    assert (padded % 128 == 0).all() and (padded >= counts).all() and (padded - counts < 128).all()
+    c2, _ = G.zipf_counts(8192, 32, 1.1, seed=3)
+    assert np.array_equal(counts, c2)

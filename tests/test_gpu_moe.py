@@ -1,0 +1,182 @@
+"""GPU tests of the fused FP8 MoE node (forward and backward) through the reference-named host
+mirror: against the CPU oracle chain stage by stage, and against a plain fp32 MoE at FP8 accuracy."""
+import numpy as np
+import pytest
+
+from oracle import pf8_oracle as O
+from tests import _gen as G
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+class _Expert:
+    def __init__(self, w1, w2):
+        self.w1, self.w2 = w1, w2
+
+
+class _Map:
+    def __init__(self, experts):
+        self.experts = experts
+
+
+def _make(E, H, I, rows, seed):
+    w1 = [G.bf16_normal((H, 2 * I), seed=seed + e, std=0.03) for e in range(E)]
+    w2 = [G.bf16_normal((I, H), seed=seed + 100 + e, std=0.03) for e in range(E)]
+    experts = []
+    for e in range(E):
+        t1, t2 = G.to_torch_bf16(w1[e]), G.to_torch_bf16(w2[e])
+        t1.main_grad = None
+        t2.main_grad = None
+        experts.append(_Expert(t1, t2))
+    M = sum(rows)
+    x = G.bf16_normal((M, H), seed=seed + 500)
+    probs = np.random.default_rng(seed).random(M, dtype=np.float32) * 0.5 + 0.25
+    return w1, w2, experts, x, probs
+
+
+def _oracle_forward(x, probs, w1, w2, rows):
+    E = len(rows)
+    H, I2 = w1[0].shape
+    I = I2 // 2
+    m_idx = np.repeat(np.arange(E, dtype=np.int32), rows)
+    xq, xs = O.quant_1x128(x, 0)
+    w1q, w1s = O.stack_transpose_quant(w1, transpose=True)
+    w2q, w2s = O.stack_transpose_quant(w2, transpose=True)
+    o1 = O.grouped_gemm_nt_contiguous(xq, xs, w1q.reshape(E, I2, H), w1s.reshape(E, I2 // 128, H // 128), m_idx)
+    return o1, m_idx, (w2q.reshape(E, H, I), w2s.reshape(E, H // 128, I // 128))
+
+
+@pytest.mark.parametrize("split", [False, True])
+def test_moe_node_forward_against_oracle_chain(split):
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 4, 512, 256
+    rows = [128, 0, 256, 128]
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=1)
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts), is_split_group_gemm=split)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    o3 = node.forward(G.to_torch_bf16(x), tp, rows)
+    assert tuple(o3.shape) == (sum(rows), H) and o3.dtype == torch.bfloat16
+    # stage 1: up+gate GEMM vs oracle
+    eo1, m_idx, (w2q, w2s) = _oracle_forward(x, probs, w1, w2, rows)
+    o1 = G.from_torch_bf16(node.o1)
+    assert G.rel_fro(O.bf16_bits_to_f32(o1), O.bf16_bits_to_f32(eo1)) <= 1e-3
+    # stage 2+3 from the GPU's own o1: requant bit-exact (pow2 scales, as the node asks), then down GEMM
+    q2, s2 = O.swiglu_weighted_quant(o1, probs, 0, True)
+    eo3 = O.grouped_gemm_nt_contiguous(q2, s2, w2q, w2s, m_idx)
+    assert G.rel_fro(O.bf16_bits_to_f32(G.from_torch_bf16(o3)), O.bf16_bits_to_f32(eo3)) <= 1e-3
+    # cached quantised input is what a re-run with hs_out=None consumes
+    o3b = node.forward(None, tp, rows)
+    assert torch.equal(o3.view(torch.int16), o3b.view(torch.int16))
+    # (fp8, scale) tuple input gives the same result
+    from paddleformers_amd import functional as F8
+
+    xq, xs = F8.fp8_quant_blockwise(G.to_torch_bf16(x), quant_method="1x128", output_scale_transpose=False)
+    node2 = FP8GroupGemmMlpFunctionNode(_Map(experts), is_split_group_gemm=split)
+    o3c = node2.forward((xq, xs), tp, rows)
+    assert torch.equal(o3.view(torch.int16), o3c.view(torch.int16))
+
+
+def test_moe_node_zero_rows_and_recompute():
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 2, 256, 128
+    w1, w2, experts, x, probs = _make(E, H, I, [128, 128], seed=3)
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts), recompute_fwd_gate_up=True)
+    out = node.forward(torch.zeros((0, H), dtype=torch.bfloat16, device="cuda"), torch.zeros((0, 1), device="cuda"), [0, 0])
+    assert tuple(out.shape) == (0, H)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    o3 = node.forward(G.to_torch_bf16(x), tp, [128, 128])
+    assert node.o1 is None       # recompute mode does not keep o1
+    dx, pg = node.backward(torch.randn((256, H), device="cuda").to(torch.bfloat16) * 1e-3, tp, [128, 128])
+    assert tuple(dx.shape) == (256, H) and tuple(pg.shape) == (256,)
+
+
+def _fp32_moe(x, probs, w1, w2, rows, dout):
+    """Plain fp32 autograd MoE on the bf16 values: the semantics of nn/experts.py:50-69 with the
+    probs multiply of the fused node."""
+    xt = torch.tensor(O.bf16_bits_to_f32(x), dtype=torch.float32, requires_grad=True)
+    pt = torch.tensor(probs, dtype=torch.float32, requires_grad=True)
+    w1t = [torch.tensor(O.bf16_bits_to_f32(w), requires_grad=True) for w in w1]
+    w2t = [torch.tensor(O.bf16_bits_to_f32(w), requires_grad=True) for w in w2]
+    outs, off = [], 0
+    for e, r in enumerate(rows):
+        if r == 0:
+            continue
+        h = xt[off:off + r] @ w1t[e]
+        I = h.shape[1] // 2
+        act = torch.nn.functional.silu(h[:, :I]) * h[:, I:] * pt[off:off + r, None]
+        outs.append(act @ w2t[e])
+        off += r
+    out = torch.cat(outs)
+    out.backward(torch.tensor(O.bf16_bits_to_f32(dout)))
+    return out.detach().numpy(), xt.grad.numpy(), pt.grad.numpy(), [w.grad for w in w1t], [w.grad for w in w2t]
+
+
+def test_moe_node_forward_backward_against_fp32_moe():
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 3, 512, 256
+    rows = [256, 0, 128]
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=7)
+    dout = G.bf16_normal((sum(rows), H), seed=9, std=1e-3)
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts))
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    o3 = node.forward(G.to_torch_bf16(x), tp, rows)
+    dx, pg = node.backward(G.to_torch_bf16(dout), tp, rows)
+    ref_o3, ref_dx, ref_pg, ref_dw1, ref_dw2 = _fp32_moe(x, probs, w1, w2, rows, dout)
+    # FP8 quantisation noise: a few percent relative Frobenius at these sizes
+    assert G.rel_fro(o3.float().cpu().numpy(), ref_o3) < 0.08
+    assert G.rel_fro(dx.float().cpu().numpy(), ref_dx) < 0.08
+    assert G.rel_fro(pg.cpu().numpy(), ref_pg) < 0.08
+    for e, r in enumerate(rows):
+        if r == 0:
+            assert experts[e].w1.main_grad is None and experts[e].w2.main_grad is None
+            continue
+        assert G.rel_fro(experts[e].w1.main_grad.cpu().numpy(), ref_dw1[e].numpy()) < 0.08
+        assert G.rel_fro(experts[e].w2.main_grad.cpu().numpy(), ref_dw2[e].numpy()) < 0.08
+    # a second backward accumulates into main_grad
+    g1 = experts[0].w1.main_grad.clone()
+    node.forward(G.to_torch_bf16(x), tp, rows)
+    node.backward(G.to_torch_bf16(dout), tp, rows)
+    assert torch.allclose(experts[0].w1.main_grad, 2 * g1, rtol=1e-5, atol=1e-8)
+
+
+def test_moe_backward_stages_against_oracle():
+    """dgrad-down -> SwiGLU backward -> dgrad-up, each stage fed with the GPU's previous stage and
+    compared with the oracle; weight gradients compared with the oracle's wgrad GEMM."""
+    from paddleformers_amd import functional as F8
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 2, 256, 128
+    rows = [128, 256]
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=11)
+    dout = G.bf16_normal((sum(rows), H), seed=12, std=1e-3)
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts))
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    node.forward(G.to_torch_bf16(x), tp, rows)
+    o1 = node.o1
+    expert_w1 = [e.w1 for e in experts]
+    expert_w2 = [e.w2 for e in experts]
+    do1, o2_s, pg = node.bwd_dowm_input(expert_w2, G.to_torch_bf16(dout), o1, rows, unzipped_probs=tp)
+    m_idx = np.repeat(np.arange(E, dtype=np.int32), rows)
+    dq, ds = O.quant_1x128(dout, 0)
+    w2q, w2s = O.stack_transpose_quant(w2, transpose=False)         # [E*I, H]: NT operand of dgrad-down
+    edo2 = O.grouped_gemm_nt_contiguous(dq, ds, w2q.reshape(E, I, H), w2s.reshape(E, I // 128, H // 128), m_idx)
+    edo1, epg, eo2s = O.swiglu_weighted_bwd(G.from_torch_bf16(o1), edo2, probs)
+    assert np.array_equal(G.from_torch_bf16(o2_s), eo2s)
+    assert G.rel_fro(O.bf16_bits_to_f32(G.from_torch_bf16(do1)), O.bf16_bits_to_f32(edo1)) <= 5e-3
+    dx = node.bwd_gate_up_input(do1, expert_w1, rows)
+    d1q, d1s = O.quant_1x128(G.from_torch_bf16(do1), 0)
+    w1q, w1s = O.stack_transpose_quant(w1, transpose=False)          # [E*H, 2I]
+    edx = O.grouped_gemm_nt_contiguous(d1q, d1s, w1q.reshape(E, H, 2 * I), w1s.reshape(E, H // 128, 2 * I // 128), m_idx)
+    assert G.rel_fro(O.bf16_bits_to_f32(G.from_torch_bf16(dx)), O.bf16_bits_to_f32(edx)) <= 1e-3
+    # weight gradient of w2 for expert 1 from the GPU's transposed operands vs the oracle GEMM
+    a_t, sa_t = F8.fused_transpose_split_quant(o2_s, None, rows, True)
+    b_t, sb_t = F8.fused_transpose_split_quant(G.to_torch_bf16(dout), None, rows, True)
+    node.bwd_down_weight((b_t, sb_t), (a_t, sa_t), expert_w2, rows)
+    e = 1
+    exp = O.gemm_nt_1d1d_f32(G.from_torch_fp8(a_t[e]), sa_t[e].cpu().numpy(), G.from_torch_fp8(b_t[e]), sb_t[e].cpu().numpy())
+    assert G.rel_fro(experts[e].w2.main_grad.cpu().numpy(), exp) <= 5e-5
