@@ -92,22 +92,28 @@ __device__ __forceinline__ uint32_t amax_bits8(uint4 w) {
 }
 
 struct TileScale {
-    float s;     // decode scale stored next to the bytes
-    float r;     // approximate reciprocal used by the fast path
-    bool slow;   // tile must take the IEEE division path (scale too small for a finite reciprocal)
+    float s;      // decode scale stored next to the bytes
+    float r_lo;   // reciprocal of s nudged down by 2^-20 (relative)
+    float r_hi;   // reciprocal of s nudged up by 2^-20
+    bool slow;    // tile must take the IEEE division path (scale too small for a finite reciprocal)
 };
 
 // s = amax/448 (IEEE divide), amax == 0 -> 1; pow2: decode scale rounded up to a power of two.
-__device__ __forceinline__ TileScale make_scale(uint32_t amax_bits, bool pow2) {
+__device__ __forceinline__ TileScale make_scale_from(float s) {
     TileScale t;
+    t.s = s;
+    const float r = __builtin_amdgcn_rcpf(s);
+    t.r_lo = r * 0.99999904632568359375f;   // 1 - 2^-20
+    t.r_hi = r * 1.00000095367431640625f;   // 1 + 2^-20
+    t.slow = !(s >= 1.0e-30f);
+    return t;
+}
+__device__ __forceinline__ TileScale make_scale(uint32_t amax_bits, bool pow2) {
     float amax = u2f(amax_bits);
     float s = amax / 448.0f;
     if (pow2) s = u2f((f2u(s) + 0x007FFFFFu) & 0x7F800000u);
     if (amax_bits == 0u) s = 1.0f;
-    t.s = s;
-    t.r = __builtin_amdgcn_rcpf(s);
-    t.slow = !(s >= 1.0e-30f);
-    return t;
+    return make_scale_from(s);
 }
 
 // two fp32 -> two e4m3 codes in the low / high half of a dword (hardware OCP convert, RNE)
@@ -122,26 +128,23 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 }
 
 // Quantise 8 values of one tile: bytes == e4m3_rne(v / s) with v / s the correctly rounded fp32
-// quotient.  Fast path: y = v * rcp(s) is within 4 ulp of that quotient; the e4m3 code can differ
-// only if a rounding boundary of the 3-bit mantissa grid (fp32 mantissa low 19 bits == 0, which
-// also covers the coarser subnormal grid) lies within that distance, so any element that close to a
-// boundary sends the lane through the exact division instead.
+// quotient.  Fast path: the quotient is bracketed by v*r_lo and v*r_hi (the reciprocal is good to
+// 1 ulp, the nudges are 2^-20, so the bracket holds with a wide margin); rounding is monotone, so
+// when both ends convert to the same e4m3 codes those are the codes of the exact quotient.  Only
+// when an end pair differs (a rounding boundary lies inside the 2^-19-wide bracket, about 3e-5 per
+// element) does the lane redo its 8 elements with the IEEE division.
 __device__ __forceinline__ uint2 quant8(const float (&v)[8], const TileScale& t) {
-    float y[8];
-    bool redo = t.slow;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        y[i] = v[i] * t.r;
-        redo |= (((f2u(y[i]) + 8u) & 0x7FFFFu) <= 16u);
-    }
+    uint2 lo, hi;
+    lo.x = pack4_e4m3(v[0] * t.r_lo, v[1] * t.r_lo, v[2] * t.r_lo, v[3] * t.r_lo);
+    lo.y = pack4_e4m3(v[4] * t.r_lo, v[5] * t.r_lo, v[6] * t.r_lo, v[7] * t.r_lo);
+    hi.x = pack4_e4m3(v[0] * t.r_hi, v[1] * t.r_hi, v[2] * t.r_hi, v[3] * t.r_hi);
+    hi.y = pack4_e4m3(v[4] * t.r_hi, v[5] * t.r_hi, v[6] * t.r_hi, v[7] * t.r_hi);
+    const bool redo = t.slow | (lo.x != hi.x) | (lo.y != hi.y);
     if (__builtin_expect(redo, 0)) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) y[i] = v[i] / t.s;
+        lo.x = pack4_e4m3(v[0] / t.s, v[1] / t.s, v[2] / t.s, v[3] / t.s);
+        lo.y = pack4_e4m3(v[4] / t.s, v[5] / t.s, v[6] / t.s, v[7] / t.s);
     }
-    uint2 o;
-    o.x = pack4_e4m3(y[0], y[1], y[2], y[3]);
-    o.y = pack4_e4m3(y[4], y[5], y[6], y[7]);
-    return o;
+    return lo;
 }
 
 __device__ __forceinline__ void unpack8(uint4 w, float (&v)[8]) {

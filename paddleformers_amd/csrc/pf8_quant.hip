@@ -16,36 +16,36 @@ namespace pf8 {
 // 1x128 quantizer: one wavefront per row, four tiles per load instruction
 // ---------------------------------------------------------------------------------------------
 
-template <int LAYOUT>
-__global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict__ x, int64_t M, int KB, int64_t ldx,
+// grid.x = column chunks of 4*U tiles, grid.y = groups of 4 rows; every lane issues its U 16-byte
+// loads before any arithmetic, so a wavefront is one load phase, one compute phase, one store phase
+template <int LAYOUT, int U>
+__global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict__ x, int64_t M, int64_t m0, int KB, int64_t ldx,
                                                      uint8_t* __restrict__ q, float* __restrict__ s, int pow2) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, l = lane & 15;
-    const int64_t r = (int64_t)blockIdx.x * 4 + wave;
+    const int64_t r = m0 + (int64_t)blockIdx.y * 4 + wave;   // m0: first row of this launch's slab
     if (r >= M) return;
+    const int kb0 = blockIdx.x * (4 * U);
     const uint4* xr = reinterpret_cast<const uint4*>(x + r * ldx);
     uint2* qr = reinterpret_cast<uint2*>(q + r * (int64_t)KB * 128);
-    constexpr int U = 4;   // tiles in flight per 16-lane group
-    for (int kb0 = 0; kb0 < KB; kb0 += 4 * U) {
-        uint4 w[U];
+    uint4 w[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int kb = kb0 + 4 * u + g;
-            w[u] = make_uint4(0, 0, 0, 0);
-            if (kb < KB) w[u] = ld16(xr + kb * 16 + l);
-        }
+    for (int u = 0; u < U; ++u) {
+        int kb = kb0 + 4 * u + g;
+        w[u] = make_uint4(0, 0, 0, 0);
+        if (kb < KB) w[u] = ld16(xr + kb * 16 + l);
+    }
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int kb = kb0 + 4 * u + g;
-            if (kb < KB) {
-                TileScale t = make_scale(row16_max(amax_bits8(w[u])), pow2 != 0);
-                float v[8];
-                unpack8(w[u], v);
-                uint2 o = quant8(v, t);
-                st8(qr + kb * 16 + l, o);
-                if (l == 0) {
-                    if (LAYOUT == 0) s[r * KB + kb] = t.s;
-                    else s[(int64_t)kb * M + r] = t.s;
-                }
+    for (int u = 0; u < U; ++u) {
+        int kb = kb0 + 4 * u + g;
+        if (kb < KB) {
+            TileScale t = make_scale(row16_max(amax_bits8(w[u])), pow2 != 0);
+            float v[8];
+            unpack8(w[u], v);
+            uint2 o = quant8(v, t);
+            st8(qr + kb * 16 + l, o);
+            if (l == 0) {
+                if (LAYOUT == 0) s[r * KB + kb] = t.s;
+                else s[(int64_t)kb * M + r] = t.s;
             }
         }
     }
@@ -57,59 +57,59 @@ __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict_
 
 template <int LAYOUT>
 __global__ __launch_bounds__(256) void k_swiglu_quant(const uint16_t* __restrict__ o1, const float* __restrict__ probs,
-                                                      int64_t M, int IB, uint8_t* __restrict__ q, float* __restrict__ s,
-                                                      uint16_t* __restrict__ o2, int pow2) {
+                                                      int64_t M, int64_t m0, int IB, uint8_t* __restrict__ q,
+                                                      float* __restrict__ s, uint16_t* __restrict__ o2, int pow2) {
+    constexpr int U = 2;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, l = lane & 15;
-    const int64_t r = (int64_t)blockIdx.x * 4 + wave;
+    const int64_t r = m0 + (int64_t)blockIdx.y * 4 + wave;
     if (r >= M) return;
+    const int kb0 = blockIdx.x * (4 * U);
     const int64_t I = (int64_t)IB * 128;
     const uint4* gr = reinterpret_cast<const uint4*>(o1 + r * 2 * I);
     const uint4* ur = reinterpret_cast<const uint4*>(o1 + r * 2 * I + I);
     uint2* qr = reinterpret_cast<uint2*>(q + r * I);
     const bool has_p = probs != nullptr;
     const float p = has_p ? probs[r] : 1.0f;
-    for (int kb0 = 0; kb0 < IB; kb0 += 8) {
-        uint4 wg[2], wu[2];
+    uint4 wg[U], wu[U];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            int kb = kb0 + 4 * u + g;
-            wg[u] = make_uint4(0, 0, 0, 0);
-            wu[u] = make_uint4(0, 0, 0, 0);
-            if (kb < IB) {
-                wg[u] = ld16(gr + kb * 16 + l);
-                wu[u] = ld16(ur + kb * 16 + l);
-            }
+    for (int u = 0; u < U; ++u) {
+        int kb = kb0 + 4 * u + g;
+        wg[u] = make_uint4(0, 0, 0, 0);
+        wu[u] = make_uint4(0, 0, 0, 0);
+        if (kb < IB) {
+            wg[u] = ld16(gr + kb * 16 + l);
+            wu[u] = ld16(ur + kb * 16 + l);
         }
+    }
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            int kb = kb0 + 4 * u + g;
-            if (kb < IB) {
-                float gv[8], uv[8], v[8];
-                unpack8(wg[u], gv);
-                unpack8(wu[u], uv);
-                uint32_t am = 0;
+    for (int u = 0; u < U; ++u) {
+        int kb = kb0 + 4 * u + g;
+        if (kb < IB) {
+            float gv[8], uv[8], v[8];
+            unpack8(wg[u], gv);
+            unpack8(wu[u], uv);
+            uint32_t am = 0;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    float y = round_bf16(silu_exact(gv[i]) * uv[i]);
-                    if (has_p) y = round_bf16(y * p);
-                    v[i] = y;
-                    am = umax(am, f2u(y) & 0x7FFFFFFFu);
-                }
-                if (o2) {
-                    uint4 ob;
-                    ob.x = (f2u(v[0]) >> 16) | (f2u(v[1]) & 0xFFFF0000u);
-                    ob.y = (f2u(v[2]) >> 16) | (f2u(v[3]) & 0xFFFF0000u);
-                    ob.z = (f2u(v[4]) >> 16) | (f2u(v[5]) & 0xFFFF0000u);
-                    ob.w = (f2u(v[6]) >> 16) | (f2u(v[7]) & 0xFFFF0000u);
-                    reinterpret_cast<uint4*>(o2 + r * I)[kb * 16 + l] = ob;
-                }
-                TileScale t = make_scale(row16_max(am), pow2 != 0);
-                uint2 o = quant8(v, t);
-                st8(qr + kb * 16 + l, o);
-                if (l == 0) {
-                    if (LAYOUT == 0) s[r * IB + kb] = t.s;
-                    else s[(int64_t)kb * M + r] = t.s;
-                }
+            for (int i = 0; i < 8; ++i) {
+                float y = round_bf16(silu_exact(gv[i]) * uv[i]);
+                if (has_p) y = round_bf16(y * p);
+                v[i] = y;
+                am = umax(am, f2u(y) & 0x7FFFFFFFu);
+            }
+            if (o2) {
+                uint4 ob;
+                ob.x = (f2u(v[0]) >> 16) | (f2u(v[1]) & 0xFFFF0000u);
+                ob.y = (f2u(v[2]) >> 16) | (f2u(v[3]) & 0xFFFF0000u);
+                ob.z = (f2u(v[4]) >> 16) | (f2u(v[5]) & 0xFFFF0000u);
+                ob.w = (f2u(v[6]) >> 16) | (f2u(v[7]) & 0xFFFF0000u);
+                st16(o2 + r * I + kb * 128 + l * 8, ob);
+            }
+            TileScale t = make_scale(row16_max(am), pow2 != 0);
+            uint2 o = quant8(v, t);
+            st8(qr + kb * 16 + l, o);
+            if (l == 0) {
+                if (LAYOUT == 0) s[r * IB + kb] = t.s;
+                else s[(int64_t)kb * M + r] = t.s;
             }
         }
     }
@@ -454,10 +454,7 @@ __global__ void k_debug_encode(const float* v, int64_t n, uint8_t* out) {
 __global__ void k_debug_div_encode(const float* x, const float* s, int64_t n, uint8_t* out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    TileScale t;
-    t.s = s[i];
-    t.r = __builtin_amdgcn_rcpf(t.s);
-    t.slow = !(t.s >= 1.0e-30f);
+    TileScale t = make_scale_from(s[i]);
     float v[8] = {x[i], 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     uint2 o = quant8(v, t);
     out[i] = (uint8_t)(o.x & 0xFFu);
@@ -487,12 +484,21 @@ extern "C" int pf8_quant_1x128(const uint16_t* x, int64_t M, int64_t K, int64_t 
     PF8_REQUIRE(ldx >= K && ldx % 8 == 0, "ldx must be >= K and a multiple of 8");
     PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q) && (reinterpret_cast<uintptr_t>(s) & 3u) == 0, "pointers must be 16-byte aligned");
     PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
-    PF8_REQUIRE(M <= (int64_t)4 * 0x7FFFFFFF && K / 128 <= 0x7FFFFF, "shape too large");
-    dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    PF8_REQUIRE(K / 128 <= 0x7FFFFF, "shape too large");
     hipStream_t st = (hipStream_t)stream;
-    if (scale_layout == 0) hipLaunchKernelGGL(k_quant_1x128<0>, grid, block, 0, st, x, M, (int)(K / 128), ldx, q, s, pow2);
-    else hipLaunchKernelGGL(k_quant_1x128<1>, grid, block, 0, st, x, M, (int)(K / 128), ldx, q, s, pow2);
-    return pf8_check_launch(__func__);
+    const int KB = (int)(K / 128);
+    constexpr int U = 4;
+    // grid.y is limited to 65535 workgroups of 4 rows: larger inputs are walked in slabs
+    const int64_t slab = (int64_t)65535 * 4;
+    for (int64_t m0 = 0; m0 < M; m0 += slab) {
+        const int64_t m = M - m0 < slab ? M - m0 : slab;
+        dim3 grid((unsigned)((KB + 4 * U - 1) / (4 * U)), (unsigned)((m + 3) / 4)), block(256);
+        if (scale_layout == 0) hipLaunchKernelGGL((k_quant_1x128<0, U>), grid, block, 0, st, x, M, m0, KB, ldx, q, s, pow2);
+        else hipLaunchKernelGGL((k_quant_1x128<1, U>), grid, block, 0, st, x, M, m0, KB, ldx, q, s, pow2);
+        int rc = pf8_check_launch(__func__);
+        if (rc) return rc;
+    }
+    return PF8_OK;
 }
 
 extern "C" int pf8_quant_128x128(const uint16_t* w, int64_t R, int64_t C, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
@@ -603,13 +609,20 @@ extern "C" int pf8_swiglu_weighted_quant(const uint16_t* o1, const float* probs,
     PF8_REQUIRE(o1 && q && s, "null pointer");
     PF8_REQUIRE(PF8_ALIGNED16(o1) && PF8_ALIGNED16(q) && PF8_ALIGNED16(o2), "pointers must be 16-byte aligned");
     PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
-    PF8_REQUIRE(M <= (int64_t)4 * 0x7FFFFFFF, "shape too large");
-    dim3 grid((unsigned)((M + 3) / 4)), block(256);
-    if (scale_layout == 0)
-        hipLaunchKernelGGL(k_swiglu_quant<0>, grid, block, 0, (hipStream_t)stream, o1, probs, M, (int)(I / 128), q, s, o2, pow2);
-    else
-        hipLaunchKernelGGL(k_swiglu_quant<1>, grid, block, 0, (hipStream_t)stream, o1, probs, M, (int)(I / 128), q, s, o2, pow2);
-    return pf8_check_launch(__func__);
+    PF8_REQUIRE(I / 128 <= 0x7FFFFF, "shape too large");
+    const int IB = (int)(I / 128);
+    const int64_t slab = (int64_t)65535 * 4;
+    for (int64_t m0 = 0; m0 < M; m0 += slab) {
+        const int64_t m = M - m0 < slab ? M - m0 : slab;
+        dim3 grid((unsigned)((IB + 7) / 8), (unsigned)((m + 3) / 4)), block(256);
+        if (scale_layout == 0)
+            hipLaunchKernelGGL(k_swiglu_quant<0>, grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
+        else
+            hipLaunchKernelGGL(k_swiglu_quant<1>, grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
+        int rc = pf8_check_launch(__func__);
+        if (rc) return rc;
+    }
+    return PF8_OK;
 }
 
 extern "C" int pf8_swiglu_weighted_bwd(const uint16_t* o1, const uint16_t* do2_s, const float* probs, int64_t M, int64_t I,
