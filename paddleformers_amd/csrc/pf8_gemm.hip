@@ -44,7 +44,19 @@ struct GemmArgs {
     int32_t tile_start[257];    // GROUP_WGRAD: first 128-row block of each expert along the reduction axis
 };
 
-__device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
+#ifndef PF8_SWZ
+#define PF8_SWZ 2
+#endif
+__device__ __forceinline__ int swz_key(int row) {
+#if PF8_SWZ == 0
+    return (row >> 1) & 7;
+#elif PF8_SWZ == 1
+    return row & 7;
+#else
+    return (row & 7) ^ ((row >> 3) & 1);
+#endif
+}
+__device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ swz_key(row)) << 4); }
 
 template <int MODE, int SQL>
 __global__ __launch_bounds__(256, 2) void k_gemm(const GemmArgs a) {
@@ -248,11 +260,266 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const GemmArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Forward / dgrad kernel, 256(P) x 256(Q) x 128(K) tiles, 512 threads = 8 wavefronts (4 along Q,
+// 2 along P), each owning 64(Q) x 128(P) = 4 x 8 MFMA tiles (128 accumulator registers).
+//
+// Budget per compute unit and 128-wide K block: 2048 cycles of MFMA work (32 MFMAs of 32 cycles on
+// each of the two wavefronts a SIMD holds) against 64 KB of L2->LDS traffic and 8 x 12 fragment
+// reads of 2 KB; LDS delivers 128 B/clk (measured), so LDS is as busy as the matrix pipe and the
+// schedule has to overlap them:
+//   * both operand tiles go global -> LDS with global_load_lds_dwordx4 (no staging registers; the
+//     16-byte chunk each lane fetches is chosen so that the linear 1 KB an instruction writes lands
+//     XOR-swizzled, which the fragment reads see conflict-free); two stages of 64 KB, one barrier
+//     per K block;
+//   * fragment reads are issued in the order the MFMAs consume them (P0, Q0..Q3, P1, P2, then one P
+//     fragment two steps ahead), so the first MFMA of a block waits for two fragments only;
+//   * the four scale-FMAs that fold product j-2 into the fp32 accumulators sit between MFMA j and
+//     j+1 (scheduling barriers pin this: left alone, the scheduler pairs every MFMA with its own
+//     FMAs and waits out the MFMA latency 32 times per block).
+// Reading the activation fragments straight from global memory instead (tried) is slower: 16 rows
+// per load instruction defeat the coalescer.
+//
+// Grouped (contiguous) rows come in 128-row expert segments: a 256-row tile whose halves belong to
+// two experts runs the K loop twice, once per expert, storing only that expert's half.
+// ---------------------------------------------------------------------------------------------
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void gbl_void;
+
+// 16 bytes per lane, global -> LDS without passing through registers.  lds_dst is the wave-uniform
+// LDS byte address of the 1 KB the instruction fills (lane l writes bytes [16 l, 16 l + 16)).
+// Written as inline assembly on purpose: the compiler's wait-count pass treats a visible
+// global_load_lds as a pending FLAT access and then turns every later LDS wait into a full drain
+// (lgkmcnt(0)), which serialises the fragment reads of a K block with its first MFMA.  The copy
+// is tracked by vmcnt in hardware; the K loop waits for it explicitly before its barrier.
+// M0 is written here and used by nothing else in these kernels.
+__device__ __forceinline__ void dma16_to_lds(const uint8_t* src, uint32_t lds_dst) {
+    const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(m0v) : "memory");
+}
+
+__device__ __forceinline__ i32x8 ld_frag_lds(const uint8_t* p0, const uint8_t* p1) {
+    i32x4 lo = *reinterpret_cast<const i32x4*>(p0);
+    i32x4 hi = *reinterpret_cast<const i32x4*>(p1);
+    return (i32x8){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+}
+
+constexpr int FWD_STAGE = 65536;   // P tile 32 KB | Q tile 32 KB
+
+template <int SQL>
+__global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wq = wave >> 1, wp = wave & 1;
+    const int li = lane & 15, kg = lane >> 4;
+
+    const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = (a.Qrows + 255) / 256;
+    const int64_t T = p_tiles * q_tiles;
+    // hardware deals consecutive workgroups round-robin to the 8 XCDs (each with its own L2): give
+    // every XCD a contiguous run of logical tiles, ordered in groups of 8 q-tiles x all p-tiles so
+    // that the ~32 tiles an XCD runs at once share 4 weight tiles and 8 activation tiles
+    const int64_t per_xcd = (T + 7) / 8;
+    const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= T) return;
+    constexpr int G = 8;
+    const int64_t grp = logical / (G * p_tiles), rem = logical % (G * p_tiles);
+    const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;   // q-tiles in this group
+    const int64_t q_tile = grp * G + rem % gq, p_tile = rem / gq;
+    const int64_t p0 = p_tile * 256, q0 = q_tile * 256;
+
+    const int64_t KB = a.red / 128;
+    const int64_t PB = (a.Prows + 127) / 128;
+    const uint8_t* qbase = a.q;
+    const float* sqb = a.sq;
+    uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
+    const int64_t q_rows_total = a.Qrows;
+
+    // up to two passes: (expert, first valid row, end valid row) relative to the tile
+    int n_pass = 1;
+    int e_a = 0, e_b = 0, lo_a = 0, hi_a = 256, lo_b = 0, hi_b = 256;
+    if (a.group == GROUP_CONTIG) {
+        const int e0 = a.m_indices[q0];
+        const int e1 = (q0 + 128 < a.Qrows) ? a.m_indices[q0 + 128] : e0;
+        if (e0 == e1) {
+            if (e0 < 0) return;
+            e_a = e0;
+        } else if (e0 >= 0 && e1 >= 0) {
+            n_pass = 2; e_a = e0; hi_a = 128; e_b = e1; lo_b = 128;
+        } else if (e0 >= 0) {
+            e_a = e0; hi_a = 128;
+        } else if (e1 >= 0) {
+            e_a = e1; lo_a = 128;
+        } else {
+            return;
+        }
+    } else if (a.group == GROUP_MASKED) {
+        const int e = blockIdx.y;
+        const int64_t valid = a.masked_m[e];
+        if (q0 >= valid) return;
+        e_a = e;
+        hi_a = valid - q0 < 256 ? (int)(valid - q0) : 256;
+        qbase += (int64_t)e * a.Qrows * a.red;
+        sqb += (int64_t)e * a.Qrows * KB;
+        outb += (int64_t)e * a.Qrows * a.ldo * 2;
+    }
+
+    // ---- global -> LDS: wave-instruction i (0..3) copies rows (i*8 + wave)*8 .. +8 of a tile ----
+    const int crow = lane >> 3, cpos = lane & 7;
+    uint32_t p_src[4], q_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = (i * 8 + wave) * 8 + crow;             // 0..255
+        const int chunk = cpos ^ swz_key(row);
+        int64_t pr = p0 + row; if (pr > a.Prows - 1) pr = a.Prows - 1;
+        int64_t qr = q0 + row; if (qr > q_rows_total - 1) qr = q_rows_total - 1;
+        p_src[i] = (uint32_t)((pr - p0) * a.red + chunk * 16);
+        q_src[i] = (uint32_t)((qr - q0) * a.red + chunk * 16);
+    }
+    const uint8_t* qtile = qbase + q0 * a.red;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    // fragment offsets inside a stage; the swizzle key repeats every 16 rows, so sub-tile t is +t*2048
+    int fp_ofs[2], fq_ofs[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        fp_ofs[h] = swz(wp * 128 + li, 2 * kg + h);
+        fq_ofs[h] = 32768 + swz(wq * 64 + li, 2 * kg + h);
+    }
+    int64_t qrow_g[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        int64_t r = q0 + wq * 64 + t * 16 + li;
+        if (r > q_rows_total - 1) r = q_rows_total - 1;
+        qrow_g[t] = r;
+    }
+    int64_t pblk = p_tile * 2 + wp;
+    if (pblk > PB - 1) pblk = PB - 1;
+
+    for (int pass = 0; pass < n_pass; ++pass) {
+        const int e = pass == 0 ? e_a : e_b;
+        const int row_lo = pass == 0 ? lo_a : lo_b, row_hi = pass == 0 ? hi_a : hi_b;
+        const uint8_t* ptile = a.p + ((int64_t)e * a.Prows + p0) * a.red;
+        const float* spb = a.sp + ((int64_t)e * PB + pblk) * KB;
+        const bool wave_active = (wq * 64 < row_hi) && (wq * 64 + 64 > row_lo);
+
+        f32x4 acc[8][4];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        float fq_nxt[4], fpb_nxt = 0.f;
+
+#define PF8_DMA(kb_, stage_)                                                                           \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                      \
+        dma16_to_lds(ptile + p_src[i] + (kb_) * 128, lds_base + (stage_) * FWD_STAGE + (i * 8 + wave) * 1024); \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                      \
+        dma16_to_lds(qtile + q_src[i] + (kb_) * 128, lds_base + (stage_) * FWD_STAGE + 32768 + (i * 8 + wave) * 1024);
+#define PF8_LOAD_S(kb_)                                                                                \
+    _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                      \
+        fq_nxt[t] = SQL == 0 ? sqb[qrow_g[t] * KB + (kb_)] : sqb[(kb_) * q_rows_total + qrow_g[t]];
+#define PF8_PFRAG(ps_) ld_frag_lds(base + fp_ofs[0] + (ps_) * 2048, base + fp_ofs[1] + (ps_) * 2048)
+#define PF8_QFRAG(qs_) ld_frag_lds(base + fq_ofs[0] + (qs_) * 2048, base + fq_ofs[1] + (qs_) * 2048)
+
+        __syncthreads();   // the previous pass is done with both stages
+        if (KB > 0) {
+            PF8_DMA(0, 0)
+            PF8_LOAD_S(0)
+            fpb_nxt = spb[0];
+        }
+        for (int64_t kb = 0; kb < KB; ++kb) {
+            const int cur = (int)(kb & 1);
+            __builtin_amdgcn_s_waitcnt(0);   // this wave's DMA and scale loads have landed
+            __syncthreads();                 // everyone's DMA landed; everyone is done with stage cur^1
+            float fq_cur[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) fq_cur[t] = fq_nxt[t] * fpb_nxt;
+            const int64_t kbn = kb + 1 < KB ? kb + 1 : kb;
+#ifndef PF8_ABL_NOLOAD
+            PF8_DMA(kbn, cur ^ 1)
+#endif
+            PF8_LOAD_S(kbn)
+            if (wave_active) {
+                const uint8_t* base = lds + cur * FWD_STAGE;
+                i32x8 pf[3], qf[4];
+                f32x4 d[3];
+                // reads in consumption order (the barriers keep the scheduler from regrouping them,
+                // so the first MFMA waits for P0 and Q0 only)
+                pf[0] = PF8_PFRAG(0);
+                __builtin_amdgcn_sched_barrier(0);
+                qf[0] = PF8_QFRAG(0);
+                __builtin_amdgcn_sched_barrier(0);
+                qf[1] = PF8_QFRAG(1);
+                __builtin_amdgcn_sched_barrier(0);
+                qf[2] = PF8_QFRAG(2);
+                __builtin_amdgcn_sched_barrier(0);
+                qf[3] = PF8_QFRAG(3);
+                __builtin_amdgcn_sched_barrier(0);
+                pf[1] = PF8_PFRAG(1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < 32; ++j) {
+                    const int ps = j >> 2, qs = j & 3;
+                    d[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps % 3], qf[qs], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (qs == 0 && ps + 2 < 8) {
+                        pf[(ps + 2) % 3] = PF8_PFRAG(ps + 2);   // two steps ahead
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    if (j >= 2) {
+                        const int jj = j - 2;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[jj & 3], acc[jj >> 2][jj & 3][r]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+#pragma unroll
+                for (int jj = 30; jj < 32; ++jj)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[jj & 3], acc[jj >> 2][jj & 3][r]);
+            }
+            // the block scale of P is a scalar load; scalar loads share the LDS wait counter and
+            // return out of order, so issuing it any earlier would turn every fragment wait of
+            // this block into a full drain
+            __builtin_amdgcn_sched_barrier(0);
+            fpb_nxt = spb[kbn];
+        }
+        __builtin_amdgcn_s_waitcnt(0);   // the redundant last prefetch must land before LDS is reused or the kernel ends
+
+        // ---- epilogue: 4 consecutive bf16 per lane ----
+        if (wave_active) {
+#pragma unroll
+            for (int qs = 0; qs < 4; ++qs) {
+                const int rt = wq * 64 + qs * 16 + li;          // row inside the tile
+                const int64_t row = q0 + rt;
+                if (rt < row_lo || rt >= row_hi || row >= q_rows_total) continue;
+#pragma unroll
+                for (int ps = 0; ps < 8; ++ps) {
+                    const int64_t col = p0 + wp * 128 + ps * 16 + 4 * kg;
+                    if (col + 4 > a.Prows) continue;
+                    uint2 o;
+                    o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
+                    o.y = pack_bf16(acc[ps][qs][2], acc[ps][qs][3]);
+                    *reinterpret_cast<uint2*>(outb + (row * a.ldo + col) * 2) = o;
+                }
+            }
+        }
+    }
+#undef PF8_DMA
+#undef PF8_LOAD_S
+#undef PF8_PFRAG
+#undef PF8_QFRAG
+}
+
 static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, const char* where) {
     const size_t lds_bytes = 65536;
     if (mode == MODE_FWD) {
-        if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm<MODE_FWD, 0>), grid, dim3(256), lds_bytes, st, a);
-        else hipLaunchKernelGGL((k_gemm<MODE_FWD, 1>), grid, dim3(256), lds_bytes, st, a);
+        // 256x256 tiles; the grid is padded to a multiple of 8 so that every XCD gets an equal run
+        const int64_t T = ((a.Prows + 255) / 256) * ((a.Qrows + 255) / 256);
+        dim3 g256((unsigned)(((T + 7) / 8) * 8), grid.y);
+        if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd256<0>), g256, dim3(512), 131072, st, a);
+        else hipLaunchKernelGGL((k_gemm_fwd256<1>), g256, dim3(512), 131072, st, a);
     } else {
         hipLaunchKernelGGL((k_gemm<MODE_WGRAD, 1>), grid, dim3(256), lds_bytes, st, a);
     }
@@ -274,6 +541,8 @@ static int ensure_lds_attr() {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_FWD, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_FWD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_WGRAD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
     done = 1;
     return PF8_OK;
