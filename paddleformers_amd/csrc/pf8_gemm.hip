@@ -305,16 +305,23 @@ __device__ __forceinline__ i32x8 ld_frag_lds(const uint8_t* p0, const uint8_t* p
     return (i32x8){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 }
 
-constexpr int FWD_STAGE = 65536;   // P tile 32 KB | Q tile 32 KB
-
-template <int SQL>
+// BQ = rows of Q per tile: 256 (4 wavefronts along Q x 2 along P, 64x128 each) for large row
+// counts, 128 (2 x 4 wavefronts, 64x64 each) when expert segments are short: a 128-row tile never
+// straddles two experts and wastes no MFMA work on a short segment.
+template <int SQL, int BQ>
 __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
+    constexpr int WQ = BQ / 64;            // wavefronts along Q
+    constexpr int WP = 8 / WQ;             // wavefronts along P
+    constexpr int PEXT = 256 / WP;         // P rows per wavefront
+    constexpr int NPS = PEXT / 16;         // P fragments per wavefront
+    constexpr int FWD_STAGE = 32768 + BQ * 128;   // P tile 32 KB | Q tile
+    constexpr int QDMA = BQ / 64;          // 1 KB copies of the Q tile per wavefront
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wq = wave >> 1, wp = wave & 1;
+    const int wq = wave / WP, wp = wave % WP;
     const int li = lane & 15, kg = lane >> 4;
 
-    const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = (a.Qrows + 255) / 256;
+    const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = (a.Qrows + BQ - 1) / BQ;
     const int64_t T = p_tiles * q_tiles;
     // hardware deals consecutive workgroups round-robin to the 8 XCDs (each with its own L2): give
     // every XCD a contiguous run of logical tiles, ordered in groups of 8 q-tiles x all p-tiles so
@@ -326,7 +333,7 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
     const int64_t grp = logical / (G * p_tiles), rem = logical % (G * p_tiles);
     const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;   // q-tiles in this group
     const int64_t q_tile = grp * G + rem % gq, p_tile = rem / gq;
-    const int64_t p0 = p_tile * 256, q0 = q_tile * 256;
+    const int64_t p0 = p_tile * 256, q0 = q_tile * BQ;
 
     const int64_t KB = a.red / 128;
     const int64_t PB = (a.Prows + 127) / 128;
@@ -337,10 +344,10 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
 
     // up to two passes: (expert, first valid row, end valid row) relative to the tile
     int n_pass = 1;
-    int e_a = 0, e_b = 0, lo_a = 0, hi_a = 256, lo_b = 0, hi_b = 256;
+    int e_a = 0, e_b = 0, lo_a = 0, hi_a = BQ, lo_b = 0, hi_b = BQ;
     if (a.group == GROUP_CONTIG) {
         const int e0 = a.m_indices[q0];
-        const int e1 = (q0 + 128 < a.Qrows) ? a.m_indices[q0 + 128] : e0;
+        const int e1 = (BQ == 256 && q0 + 128 < a.Qrows) ? a.m_indices[q0 + 128] : e0;
         if (e0 == e1) {
             if (e0 < 0) return;
             e_a = e0;
@@ -358,7 +365,7 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
         const int64_t valid = a.masked_m[e];
         if (q0 >= valid) return;
         e_a = e;
-        hi_a = valid - q0 < 256 ? (int)(valid - q0) : 256;
+        hi_a = valid - q0 < BQ ? (int)(valid - q0) : BQ;
         qbase += (int64_t)e * a.Qrows * a.red;
         sqb += (int64_t)e * a.Qrows * KB;
         outb += (int64_t)e * a.Qrows * a.ldo * 2;
@@ -366,15 +373,17 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
 
     // ---- global -> LDS: wave-instruction i (0..3) copies rows (i*8 + wave)*8 .. +8 of a tile ----
     const int crow = lane >> 3, cpos = lane & 7;
-    uint32_t p_src[4], q_src[4];
+    uint32_t p_src[4], q_src[QDMA];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = (i * 8 + wave) * 8 + crow;             // 0..255
         const int chunk = cpos ^ swz_key(row);
         int64_t pr = p0 + row; if (pr > a.Prows - 1) pr = a.Prows - 1;
-        int64_t qr = q0 + row; if (qr > q_rows_total - 1) qr = q_rows_total - 1;
         p_src[i] = (uint32_t)((pr - p0) * a.red + chunk * 16);
-        q_src[i] = (uint32_t)((qr - q0) * a.red + chunk * 16);
+        if (i < QDMA) {
+            int64_t qr = q0 + row; if (qr > q_rows_total - 1) qr = q_rows_total - 1;
+            q_src[i] = (uint32_t)((qr - q0) * a.red + chunk * 16);
+        }
     }
     const uint8_t* qtile = qbase + q0 * a.red;
     const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
@@ -382,7 +391,7 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
     int fp_ofs[2], fq_ofs[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        fp_ofs[h] = swz(wp * 128 + li, 2 * kg + h);
+        fp_ofs[h] = swz(wp * PEXT + li, 2 * kg + h);
         fq_ofs[h] = 32768 + swz(wq * 64 + li, 2 * kg + h);
     }
     int64_t qrow_g[4];
@@ -392,7 +401,7 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
         if (r > q_rows_total - 1) r = q_rows_total - 1;
         qrow_g[t] = r;
     }
-    int64_t pblk = p_tile * 2 + wp;
+    int64_t pblk = p_tile * 2 + (wp * PEXT) / 128;
     if (pblk > PB - 1) pblk = PB - 1;
 
     for (int pass = 0; pass < n_pass; ++pass) {
@@ -402,9 +411,9 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
         const float* spb = a.sp + ((int64_t)e * PB + pblk) * KB;
         const bool wave_active = (wq * 64 < row_hi) && (wq * 64 + 64 > row_lo);
 
-        f32x4 acc[8][4];
+        f32x4 acc[NPS][4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < NPS; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
         float fq_nxt[4], fpb_nxt = 0.f;
@@ -412,7 +421,7 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
 #define PF8_DMA(kb_, stage_)                                                                           \
     _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                      \
         dma16_to_lds(ptile + p_src[i] + (kb_) * 128, lds_base + (stage_) * FWD_STAGE + (i * 8 + wave) * 1024); \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                      \
+    _Pragma("unroll") for (int i = 0; i < QDMA; ++i)                                                   \
         dma16_to_lds(qtile + q_src[i] + (kb_) * 128, lds_base + (stage_) * FWD_STAGE + 32768 + (i * 8 + wave) * 1024);
 #define PF8_LOAD_S(kb_)                                                                                \
     _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                      \
@@ -457,14 +466,19 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
                 pf[1] = PF8_PFRAG(1);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < 32; ++j) {
+                for (int j = 0; j < NPS * 4; ++j) {
                     const int ps = j >> 2, qs = j & 3;
                     d[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps % 3], qf[qs], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (qs == 0 && ps + 2 < 8) {
+#ifdef PF8_ABL_NOPFRAG
+                    if (false) {
+#else
+                    if (qs == 0 && ps + 2 < NPS) {
+#endif
                         pf[(ps + 2) % 3] = PF8_PFRAG(ps + 2);   // two steps ahead
                         __builtin_amdgcn_sched_barrier(0);
                     }
+
                     if (j >= 2) {
                         const int jj = j - 2;
 #pragma unroll
@@ -474,7 +488,7 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
                     }
                 }
 #pragma unroll
-                for (int jj = 30; jj < 32; ++jj)
+                for (int jj = NPS * 4 - 2; jj < NPS * 4; ++jj)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
                         acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[jj & 3], acc[jj >> 2][jj & 3][r]);
@@ -495,8 +509,8 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
                 const int64_t row = q0 + rt;
                 if (rt < row_lo || rt >= row_hi || row >= q_rows_total) continue;
 #pragma unroll
-                for (int ps = 0; ps < 8; ++ps) {
-                    const int64_t col = p0 + wp * 128 + ps * 16 + 4 * kg;
+                for (int ps = 0; ps < NPS; ++ps) {
+                    const int64_t col = p0 + wp * PEXT + ps * 16 + 4 * kg;
                     if (col + 4 > a.Prows) continue;
                     uint2 o;
                     o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
@@ -516,10 +530,18 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
     const size_t lds_bytes = 65536;
     if (mode == MODE_FWD) {
         // 256x256 tiles; the grid is padded to a multiple of 8 so that every XCD gets an equal run
-        const int64_t T = ((a.Prows + 255) / 256) * ((a.Qrows + 255) / 256);
+        // short expert segments (grouped layouts with few rows per expert) take 128-row tiles
+        const bool short_rows = a.group != GROUP_NONE && a.E > 0 && a.Qrows / a.E < 768 && a.group == GROUP_CONTIG;
+        const int bq = short_rows ? 128 : 256;
+        const int64_t T = ((a.Prows + 255) / 256) * ((a.Qrows + bq - 1) / bq);
         dim3 g256((unsigned)(((T + 7) / 8) * 8), grid.y);
-        if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd256<0>), g256, dim3(512), 131072, st, a);
-        else hipLaunchKernelGGL((k_gemm_fwd256<1>), g256, dim3(512), 131072, st, a);
+        if (bq == 256) {
+            if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd256<0, 256>), g256, dim3(512), 131072, st, a);
+            else hipLaunchKernelGGL((k_gemm_fwd256<1, 256>), g256, dim3(512), 131072, st, a);
+        } else {
+            if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd256<0, 128>), g256, dim3(512), 98304, st, a);
+            else hipLaunchKernelGGL((k_gemm_fwd256<1, 128>), g256, dim3(512), 98304, st, a);
+        }
     } else {
         hipLaunchKernelGGL((k_gemm<MODE_WGRAD, 1>), grid, dim3(256), lds_bytes, st, a);
     }
@@ -541,8 +563,10 @@ static int ensure_lds_attr() {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_FWD, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_FWD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_WGRAD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<0, 256>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<1, 256>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<0, 128>), hipFuncAttributeMaxDynamicSharedMemorySize, 98304);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<1, 128>), hipFuncAttributeMaxDynamicSharedMemorySize, 98304);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
     done = 1;
     return PF8_OK;
