@@ -26,6 +26,12 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 FP8_PEAK_TFLOPS = 5000.0
+# HBM bytes one launch of the up+gate grouped GEMM moves on this workload, from two rocprofv3 --pmc
+# runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
+# counter reads for the 1 GiB pf8::k_debug_copy launched with --copy-yardstick (FETCH_SIZE reads
+# 0.5 KiB per KiB copied -> factor 2.0; WRITE_SIZE reads 1.0 -> factor 1.0):
+#   703,826 KiB x 2.0 + 79,874 KiB x 1.0 = 1,487,526 KiB.   Summary: profiles/gemm_up_gate_config3_hbm_traffic.md
+GEMM_UP_GATE_TRAFFIC_BYTES = 1487526 * 1024
 
 
 def zipf_counts(total, E, s, seed, n_empty=2, pad=128):
@@ -102,7 +108,7 @@ def bench_quantizers(iters=20, warmup=5):
     return out
 
 
-def cpu_baseline(H, I, rows=256):
+def cpu_baseline(H, I, rows=12288):
     """The CPU oracle on a bounded sample of the same pipeline: `rows` token rows of ONE expert
     (quant -> up+gate GEMM -> SwiGLU+requant -> down GEMM), OpenMP over the host cores."""
     import numpy as np
@@ -138,6 +144,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-quant", action="store_true")
+    ap.add_argument("--copy-yardstick", action="store_true",
+                    help="also launch one plain 1 GiB copy (pf8::k_debug_copy) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                         "readings of the GEMM can be scaled by a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path uses no collectives and the run has a single MI355X; use --gpus 1",
@@ -207,6 +216,16 @@ def main():
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
 
+    if args.copy_yardstick:
+        import ctypes as C
+
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        _lib.call("pf8_debug_copy", C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), src.numel(),
+                  C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        del src, dst
+
     names = ["quant_x", "gemm_up_gate", "swiglu_requant", "gemm_down"]
     kms = {n: sum(ev[k][i].elapsed_time(ev[k][i + 1]) for k in range(args.steps)) / args.steps for i, n in enumerate(names)}
 
@@ -244,7 +263,8 @@ def main():
             "peak": FP8_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(ach / FP8_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": GEMM_UP_GATE_TRAFFIC_BYTES,
+            "algorithmic_bytes": int(w1q[counts > 0].numel() + Mpad * H + Mpad * 2 * I * 2),
         },
     }
     if not args.no_quant:

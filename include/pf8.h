@@ -149,6 +149,10 @@ int pf8_grouped_wgrad(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t,
                       const int64_t* rows_per_expert, int E, int64_t Kin, int64_t N, float* out,
                       int accumulate, pf8_stream_t stream);
 
+/* Measurement hook: a plain device-to-device copy of nbytes (multiple of 16).  bench.py launches it
+ * so that hardware traffic counters (FETCH_SIZE / WRITE_SIZE) can be scaled by a kernel whose
+ * traffic is known. */
+int pf8_debug_copy(const void* src, void* dst, int64_t nbytes, pf8_stream_t stream);
 /* Self-test hook used by the GPU tests: converts n floats to e4m3 with the same device routine the
  * quantizers use (hardware OCP convert), so the codec can be swept exhaustively. */
 int pf8_debug_encode(const float* v, int64_t n, uint8_t* out, pf8_stream_t stream);

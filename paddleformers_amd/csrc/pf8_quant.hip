@@ -447,6 +447,11 @@ __global__ __launch_bounds__(256) void k_weight_dequant(const uint8_t* __restric
 // self-test kernels
 // ---------------------------------------------------------------------------------------------
 
+// plain 16-byte-per-lane copy of known size: the yardstick the HBM traffic counters are scaled by
+__global__ __launch_bounds__(256) void k_debug_copy(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n16) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
 __global__ void k_debug_encode(const float* v, int64_t n, uint8_t* out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) out[i] = (uint8_t)(cvt_e4m3_lo(v[i], 0.0f, 0u) & 0xFFu);
@@ -663,6 +668,16 @@ extern "C" int pf8_weight_dequant(const uint8_t* q, const float* s, int64_t R, i
     return pf8_check_launch(__func__);
 }
 
+extern "C" int pf8_debug_copy(const void* src, void* dst, int64_t nbytes, pf8_stream_t stream) {
+    PF8_REQUIRE(nbytes >= 0 && nbytes % 16 == 0, "nbytes must be a non-negative multiple of 16");
+    if (nbytes == 0) return PF8_OK;
+    PF8_REQUIRE(src && dst && PF8_ALIGNED16(src) && PF8_ALIGNED16(dst), "null or misaligned pointer");
+    const int64_t n16 = nbytes / 16;
+    PF8_REQUIRE((n16 + 255) / 256 <= 0x7FFFFFFF, "too large");
+    hipLaunchKernelGGL(k_debug_copy, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4*)src, (uint4*)dst, n16);
+    return pf8_check_launch(__func__);
+}
 extern "C" int pf8_debug_encode(const float* v, int64_t n, uint8_t* out, pf8_stream_t stream) {
     if (n <= 0) return PF8_OK;
     PF8_REQUIRE(v && out, "null pointer");
