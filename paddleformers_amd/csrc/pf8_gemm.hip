@@ -12,10 +12,11 @@
 //   forward / dgrad : P = weights [N,K] (128x128 scales), Q = activations [M,K] (1x128 scales)
 //   weight gradient : P = dout^T [N,M], Q = x^T [Kin,M], both 1x128-scaled along M
 //
-// Workgroup: 256 threads = 4 wavefronts in a 2x2 arrangement, tile 128(P) x 128(Q) x 128(K);
-// each wavefront owns 64x64 = 4x4 MFMA tiles.  LDS: two stages of P and Q tiles (64 KB), rows of
-// 128 B with the 16-byte chunks XOR-swizzled by (row>>1)&7 so both the 16 B global->LDS writes and
-// the fragment reads are bank-conflict free.
+// Two kernels: k_gemm_fwd128 (forward / dgrad, 128x256x128 tiles, described at its definition) and
+// k_gemm (the weight-gradient form: 256 threads = 4 wavefronts in a 2x2 arrangement, tile
+// 128(P) x 128(Q) x 128(K), each wavefront 64x64 = 4x4 MFMA tiles, operands staged through
+// registers into two 32 KB LDS stages).  LDS rows are 128 B with their 16-byte chunks XOR-swizzled
+// so that fragment reads (16 rows x 32 B per quarter-wave) are bank-conflict free.
 #include "pf8_device.h"
 #include "pf8_host.h"
 
@@ -260,30 +261,6 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const GemmArgs a) {
     }
 }
 
-// ---------------------------------------------------------------------------------------------
-// Forward / dgrad kernel, 256(P) x 256(Q) x 128(K) tiles, 512 threads = 8 wavefronts (4 along Q,
-// 2 along P), each owning 64(Q) x 128(P) = 4 x 8 MFMA tiles (128 accumulator registers).
-//
-// Budget per compute unit and 128-wide K block: 2048 cycles of MFMA work (32 MFMAs of 32 cycles on
-// each of the two wavefronts a SIMD holds) against 64 KB of L2->LDS traffic and 8 x 12 fragment
-// reads of 2 KB; LDS delivers 128 B/clk (measured), so LDS is as busy as the matrix pipe and the
-// schedule has to overlap them:
-//   * both operand tiles go global -> LDS with global_load_lds_dwordx4 (no staging registers; the
-//     16-byte chunk each lane fetches is chosen so that the linear 1 KB an instruction writes lands
-//     XOR-swizzled, which the fragment reads see conflict-free); two stages of 64 KB, one barrier
-//     per K block;
-//   * fragment reads are issued in the order the MFMAs consume them (P0, Q0..Q3, P1, P2, then one P
-//     fragment two steps ahead), so the first MFMA of a block waits for two fragments only;
-//   * the four scale-FMAs that fold product j-2 into the fp32 accumulators sit between MFMA j and
-//     j+1 (scheduling barriers pin this: left alone, the scheduler pairs every MFMA with its own
-//     FMAs and waits out the MFMA latency 32 times per block).
-// Reading the activation fragments straight from global memory instead (tried) is slower: 16 rows
-// per load instruction defeat the coalescer.
-//
-// Grouped (contiguous) rows come in 128-row expert segments: a 256-row tile whose halves belong to
-// two experts runs the K loop twice, once per expert, storing only that expert's half.
-// ---------------------------------------------------------------------------------------------
-
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
 
@@ -305,33 +282,53 @@ __device__ __forceinline__ i32x8 ld_frag_lds(const uint8_t* p0, const uint8_t* p
     return (i32x8){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 }
 
-// BQ = rows of Q per tile: 256 (4 wavefronts along Q x 2 along P, 64x128 each) for large row
-// counts, 128 (2 x 4 wavefronts, 64x64 each) when expert segments are short: a 128-row tile never
-// straddles two experts and wastes no MFMA work on a short segment.
-template <int SQL, int BQ>
-__global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
-    constexpr int WQ = BQ / 64;            // wavefronts along Q
-    constexpr int WP = 8 / WQ;             // wavefronts along P
-    constexpr int PEXT = 256 / WP;         // P rows per wavefront
-    constexpr int NPS = PEXT / 16;         // P fragments per wavefront
-    constexpr int FWD_STAGE = 32768 + BQ * 128;   // P tile 32 KB | Q tile
-    constexpr int QDMA = BQ / 64;          // 1 KB copies of the Q tile per wavefront
+// ---------------------------------------------------------------------------------------------
+// Forward / dgrad kernel: 128(Q) x 256(P) x 128(K) tiles, 256 threads = 4 wavefronts (2 along Q x
+// 2 along P), each owning 64(Q) x 128(P) = 4 x 8 MFMA tiles (128 accumulator registers).
+//
+// Budget per compute unit and 128-wide K block (two workgroups resident): 2048 cycles of MFMA work
+// per SIMD against 96 KB of L2->LDS traffic (1536 cycles at 64 B/clk) and 8 x 12 fragment reads of
+// 2 KB (LDS delivers 128 B/clk, measured: 1536 cycles, plus 768 for the incoming copies).  LDS is
+// as busy as the matrix pipe, so the schedule is built to overlap them:
+//   * both operand tiles go global -> LDS with global_load_lds_dwordx4 (no staging registers; the
+//     16-byte chunk each lane fetches is chosen so that the linear 1 KB an instruction writes lands
+//     XOR-swizzled, which the fragment reads see conflict-free);
+//   * 80 KB of LDS per workgroup so that TWO workgroups share a compute unit: while one sits at a
+//     barrier or waits for its first fragments, the other keeps the matrix pipe busy.  The P tile
+//     is double-buffered (2 x 32 KB); the Q tile (16 KB) is single-buffered: its fragments are read
+//     into registers at the head of a K block, and once every wavefront has done so (second
+//     barrier, placed after the first eight MFMAs) the buffer is refilled for the next block;
+//   * fragment reads are issued in the order the MFMAs consume them (P0, Q0..Q3, P1, then one P
+//     fragment two steps ahead), so the first MFMA of a block waits for two fragments only;
+//   * the four scale-FMAs that fold product j-2 into the fp32 accumulators sit between MFMA j and
+//     j+1 (scheduling barriers pin this: left alone, the scheduler pairs every MFMA with its own
+//     FMAs and waits out the MFMA latency 32 times per block).
+// Tried and dropped: a 256x256 tile with 8 wavefronts in one workgroup per compute unit (fewer LDS
+// bytes per MFMA, but its single barrier domain left the matrix pipe idle at every block boundary:
+// 1.7-1.9 PFLOP/s dense against 1.8-2.0 here, and 0.85 against 1.4 on short expert segments), and
+// reading the activation fragments straight from global memory (16 rows per load instruction
+// defeat the coalescer).
+// A 128-row tile never straddles two experts of the grouped layout.
+// ---------------------------------------------------------------------------------------------
+template <int SQL>
+__global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
+    constexpr int BQ = 128, NPS = 8;
+    constexpr int P_STAGE = 32768, Q_OFS = 65536;   // [P stage 0 | P stage 1 | Q]
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wq = wave / WP, wp = wave % WP;
+    const int wq = wave >> 1, wp = wave & 1;
     const int li = lane & 15, kg = lane >> 4;
 
     const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = (a.Qrows + BQ - 1) / BQ;
     const int64_t T = p_tiles * q_tiles;
-    // hardware deals consecutive workgroups round-robin to the 8 XCDs (each with its own L2): give
-    // every XCD a contiguous run of logical tiles, ordered in groups of 8 q-tiles x all p-tiles so
-    // that the ~32 tiles an XCD runs at once share 4 weight tiles and 8 activation tiles
+    // consecutive workgroups go round-robin to the 8 XCDs: give every XCD a contiguous run of logical
+    // tiles, ordered in groups of 16 q-tiles x all p-tiles
     const int64_t per_xcd = (T + 7) / 8;
     const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (logical >= T) return;
-    constexpr int G = 8;
+    constexpr int G = 16;
     const int64_t grp = logical / (G * p_tiles), rem = logical % (G * p_tiles);
-    const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;   // q-tiles in this group
+    const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;
     const int64_t q_tile = grp * G + rem % gq, p_tile = rem / gq;
     const int64_t p0 = p_tile * 256, q0 = q_tile * BQ;
 
@@ -341,58 +338,42 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
     const float* sqb = a.sq;
     uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
     const int64_t q_rows_total = a.Qrows;
-
-    // up to two passes: (expert, first valid row, end valid row) relative to the tile
-    int n_pass = 1;
-    int e_a = 0, e_b = 0, lo_a = 0, hi_a = BQ, lo_b = 0, hi_b = BQ;
+    int e = 0, row_hi = BQ;
     if (a.group == GROUP_CONTIG) {
-        const int e0 = a.m_indices[q0];
-        const int e1 = (BQ == 256 && q0 + 128 < a.Qrows) ? a.m_indices[q0 + 128] : e0;
-        if (e0 == e1) {
-            if (e0 < 0) return;
-            e_a = e0;
-        } else if (e0 >= 0 && e1 >= 0) {
-            n_pass = 2; e_a = e0; hi_a = 128; e_b = e1; lo_b = 128;
-        } else if (e0 >= 0) {
-            e_a = e0; hi_a = 128;
-        } else if (e1 >= 0) {
-            e_a = e1; lo_a = 128;
-        } else {
-            return;
-        }
+        e = a.m_indices[q0];
+        if (e < 0) return;
     } else if (a.group == GROUP_MASKED) {
-        const int e = blockIdx.y;
+        e = blockIdx.y;
         const int64_t valid = a.masked_m[e];
         if (q0 >= valid) return;
-        e_a = e;
-        hi_a = valid - q0 < BQ ? (int)(valid - q0) : BQ;
+        row_hi = valid - q0 < BQ ? (int)(valid - q0) : BQ;
         qbase += (int64_t)e * a.Qrows * a.red;
         sqb += (int64_t)e * a.Qrows * KB;
         outb += (int64_t)e * a.Qrows * a.ldo * 2;
     }
 
-    // ---- global -> LDS: wave-instruction i (0..3) copies rows (i*8 + wave)*8 .. +8 of a tile ----
+    // global -> LDS: P tile = 32 copies of 1 KB (8 per wavefront), Q tile = 16 copies (4 per wavefront)
     const int crow = lane >> 3, cpos = lane & 7;
-    uint32_t p_src[4], q_src[QDMA];
+    uint32_t p_src[8], q_src[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = (i * 8 + wave) * 8 + crow;             // 0..255
+    for (int i = 0; i < 8; ++i) {
+        const int row = (i * 4 + wave) * 8 + crow;             // 0..255
         const int chunk = cpos ^ swz_key(row);
         int64_t pr = p0 + row; if (pr > a.Prows - 1) pr = a.Prows - 1;
         p_src[i] = (uint32_t)((pr - p0) * a.red + chunk * 16);
-        if (i < QDMA) {
-            int64_t qr = q0 + row; if (qr > q_rows_total - 1) qr = q_rows_total - 1;
+        if (i < 4) {
+            int64_t qr = q0 + row; if (qr > q_rows_total - 1) qr = q_rows_total - 1;   // row < 128 for i < 4
             q_src[i] = (uint32_t)((qr - q0) * a.red + chunk * 16);
         }
     }
     const uint8_t* qtile = qbase + q0 * a.red;
+    const uint8_t* ptile = a.p + ((int64_t)e * a.Prows + p0) * a.red;
     const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
-    // fragment offsets inside a stage; the swizzle key repeats every 16 rows, so sub-tile t is +t*2048
     int fp_ofs[2], fq_ofs[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        fp_ofs[h] = swz(wp * PEXT + li, 2 * kg + h);
-        fq_ofs[h] = 32768 + swz(wq * 64 + li, 2 * kg + h);
+        fp_ofs[h] = swz(wp * 128 + li, 2 * kg + h);
+        fq_ofs[h] = Q_OFS + swz(wq * 64 + li, 2 * kg + h);
     }
     int64_t qrow_g[4];
 #pragma unroll
@@ -401,126 +382,113 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
         if (r > q_rows_total - 1) r = q_rows_total - 1;
         qrow_g[t] = r;
     }
-    int64_t pblk = p_tile * 2 + (wp * PEXT) / 128;
+    int64_t pblk = p_tile * 2 + wp;
     if (pblk > PB - 1) pblk = PB - 1;
+    const float* spb = a.sp + ((int64_t)e * PB + pblk) * KB;
 
-    for (int pass = 0; pass < n_pass; ++pass) {
-        const int e = pass == 0 ? e_a : e_b;
-        const int row_lo = pass == 0 ? lo_a : lo_b, row_hi = pass == 0 ? hi_a : hi_b;
-        const uint8_t* ptile = a.p + ((int64_t)e * a.Prows + p0) * a.red;
-        const float* spb = a.sp + ((int64_t)e * PB + pblk) * KB;
-        const bool wave_active = (wq * 64 < row_hi) && (wq * 64 + 64 > row_lo);
-
-        f32x4 acc[NPS][4];
+    f32x4 acc[NPS][4];
 #pragma unroll
-        for (int i = 0; i < NPS; ++i)
+    for (int i = 0; i < NPS; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        float fq_nxt[4], fpb_nxt = 0.f;
+        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float fq_nxt[4], fpb_nxt = 0.f;
 
-#define PF8_DMA(kb_, stage_)                                                                           \
+#define PF8_DMA_P(kb_, stage_)                                                                         \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i)                                                      \
+        dma16_to_lds(ptile + p_src[i] + (kb_) * 128, lds_base + (stage_) * P_STAGE + (i * 4 + wave) * 1024);
+#define PF8_DMA_Q(kb_)                                                                                 \
     _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                      \
-        dma16_to_lds(ptile + p_src[i] + (kb_) * 128, lds_base + (stage_) * FWD_STAGE + (i * 8 + wave) * 1024); \
-    _Pragma("unroll") for (int i = 0; i < QDMA; ++i)                                                   \
-        dma16_to_lds(qtile + q_src[i] + (kb_) * 128, lds_base + (stage_) * FWD_STAGE + 32768 + (i * 8 + wave) * 1024);
+        dma16_to_lds(qtile + q_src[i] + (kb_) * 128, lds_base + Q_OFS + (i * 4 + wave) * 1024);
 #define PF8_LOAD_S(kb_)                                                                                \
     _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                      \
         fq_nxt[t] = SQL == 0 ? sqb[qrow_g[t] * KB + (kb_)] : sqb[(kb_) * q_rows_total + qrow_g[t]];
-#define PF8_PFRAG(ps_) ld_frag_lds(base + fp_ofs[0] + (ps_) * 2048, base + fp_ofs[1] + (ps_) * 2048)
-#define PF8_QFRAG(qs_) ld_frag_lds(base + fq_ofs[0] + (qs_) * 2048, base + fq_ofs[1] + (qs_) * 2048)
+#define PF8_PFRAG(ps_) ld_frag_lds(pbase + fp_ofs[0] + (ps_) * 2048, pbase + fp_ofs[1] + (ps_) * 2048)
+#define PF8_QFRAG(qs_) ld_frag_lds(lds + fq_ofs[0] + (qs_) * 2048, lds + fq_ofs[1] + (qs_) * 2048)
 
-        __syncthreads();   // the previous pass is done with both stages
-        if (KB > 0) {
-            PF8_DMA(0, 0)
-            PF8_LOAD_S(0)
-            fpb_nxt = spb[0];
-        }
-        for (int64_t kb = 0; kb < KB; ++kb) {
-            const int cur = (int)(kb & 1);
-            __builtin_amdgcn_s_waitcnt(0);   // this wave's DMA and scale loads have landed
-            __syncthreads();                 // everyone's DMA landed; everyone is done with stage cur^1
-            float fq_cur[4];
+    if (KB > 0) {
+        PF8_DMA_P(0, 0)
+        PF8_DMA_Q(0)
+        PF8_LOAD_S(0)
+        fpb_nxt = spb[0];
+    }
+    for (int64_t kb = 0; kb < KB; ++kb) {
+        const int cur = (int)(kb & 1);
+        __builtin_amdgcn_s_waitcnt(0);   // this wave's copies and scale loads have landed
+        __syncthreads();                 // everyone's copies landed; everyone is done with P stage cur^1
+        float fq_cur[4];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) fq_cur[t] = fq_nxt[t] * fpb_nxt;
-            const int64_t kbn = kb + 1 < KB ? kb + 1 : kb;
-#ifndef PF8_ABL_NOLOAD
-            PF8_DMA(kbn, cur ^ 1)
-#endif
-            PF8_LOAD_S(kbn)
-            if (wave_active) {
-                const uint8_t* base = lds + cur * FWD_STAGE;
-                i32x8 pf[3], qf[4];
-                f32x4 d[3];
-                // reads in consumption order (the barriers keep the scheduler from regrouping them,
-                // so the first MFMA waits for P0 and Q0 only)
-                pf[0] = PF8_PFRAG(0);
-                __builtin_amdgcn_sched_barrier(0);
-                qf[0] = PF8_QFRAG(0);
-                __builtin_amdgcn_sched_barrier(0);
-                qf[1] = PF8_QFRAG(1);
-                __builtin_amdgcn_sched_barrier(0);
-                qf[2] = PF8_QFRAG(2);
-                __builtin_amdgcn_sched_barrier(0);
-                qf[3] = PF8_QFRAG(3);
-                __builtin_amdgcn_sched_barrier(0);
-                pf[1] = PF8_PFRAG(1);
-                __builtin_amdgcn_sched_barrier(0);
+        for (int t = 0; t < 4; ++t) fq_cur[t] = fq_nxt[t] * fpb_nxt;
+        const int64_t kbn = kb + 1 < KB ? kb + 1 : kb;
+        PF8_DMA_P(kbn, cur ^ 1)
+        PF8_LOAD_S(kbn)
+        const uint8_t* pbase = lds + cur * P_STAGE;
+        i32x8 pf[3], qf[4];
+        f32x4 d[3];
+        pf[0] = PF8_PFRAG(0);
+        __builtin_amdgcn_sched_barrier(0);
+        qf[0] = PF8_QFRAG(0);
+        __builtin_amdgcn_sched_barrier(0);
+        qf[1] = PF8_QFRAG(1);
+        __builtin_amdgcn_sched_barrier(0);
+        qf[2] = PF8_QFRAG(2);
+        __builtin_amdgcn_sched_barrier(0);
+        qf[3] = PF8_QFRAG(3);
+        __builtin_amdgcn_sched_barrier(0);
+        pf[1] = PF8_PFRAG(1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < NPS * 4; ++j) {
-                    const int ps = j >> 2, qs = j & 3;
-                    d[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps % 3], qf[qs], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-#ifdef PF8_ABL_NOPFRAG
-                    if (false) {
-#else
-                    if (qs == 0 && ps + 2 < NPS) {
-#endif
-                        pf[(ps + 2) % 3] = PF8_PFRAG(ps + 2);   // two steps ahead
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-
-                    if (j >= 2) {
-                        const int jj = j - 2;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[jj & 3], acc[jj >> 2][jj & 3][r]);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-#pragma unroll
-                for (int jj = NPS * 4 - 2; jj < NPS * 4; ++jj)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[jj & 3], acc[jj >> 2][jj & 3][r]);
-            }
-            // the block scale of P is a scalar load; scalar loads share the LDS wait counter and
-            // return out of order, so issuing it any earlier would turn every fragment wait of
-            // this block into a full drain
+        for (int j = 0; j < NPS * 4; ++j) {
+            const int ps = j >> 2, qs = j & 3;
+            d[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps % 3], qf[qs], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            fpb_nxt = spb[kbn];
-        }
-        __builtin_amdgcn_s_waitcnt(0);   // the redundant last prefetch must land before LDS is reused or the kernel ends
-
-        // ---- epilogue: 4 consecutive bf16 per lane ----
-        if (wave_active) {
-#pragma unroll
-            for (int qs = 0; qs < 4; ++qs) {
-                const int rt = wq * 64 + qs * 16 + li;          // row inside the tile
-                const int64_t row = q0 + rt;
-                if (rt < row_lo || rt >= row_hi || row >= q_rows_total) continue;
-#pragma unroll
-                for (int ps = 0; ps < NPS; ++ps) {
-                    const int64_t col = p0 + wp * PEXT + ps * 16 + 4 * kg;
-                    if (col + 4 > a.Prows) continue;
-                    uint2 o;
-                    o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
-                    o.y = pack_bf16(acc[ps][qs][2], acc[ps][qs][3]);
-                    *reinterpret_cast<uint2*>(outb + (row * a.ldo + col) * 2) = o;
-                }
+            if (qs == 0 && ps + 2 < NPS) {
+                pf[(ps + 2) % 3] = PF8_PFRAG(ps + 2);
+                __builtin_amdgcn_sched_barrier(0);
             }
+            if (j == 7) {
+                // every wavefront has its four Q fragments in registers by now: refill the Q buffer
+                __syncthreads();
+                PF8_DMA_Q(kbn)
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (j >= 2) {
+                const int jj = j - 2;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[jj & 3], acc[jj >> 2][jj & 3][r]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int jj = NPS * 4 - 2; jj < NPS * 4; ++jj)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[jj & 3], acc[jj >> 2][jj & 3][r]);
+        __builtin_amdgcn_sched_barrier(0);
+        // the block scale of P is a scalar load; scalar loads share the LDS wait counter and return
+        // out of order, so issuing it any earlier would turn every fragment wait of this block
+        // into a full drain
+        fpb_nxt = spb[kbn];
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+
+#pragma unroll
+    for (int qs = 0; qs < 4; ++qs) {
+        const int rt = wq * 64 + qs * 16 + li;
+        const int64_t row = q0 + rt;
+        if (rt >= row_hi || row >= q_rows_total) continue;
+#pragma unroll
+        for (int ps = 0; ps < NPS; ++ps) {
+            const int64_t col = p0 + wp * 128 + ps * 16 + 4 * kg;
+            if (col + 4 > a.Prows) continue;
+            uint2 o;
+            o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
+            o.y = pack_bf16(acc[ps][qs][2], acc[ps][qs][3]);
+            *reinterpret_cast<uint2*>(outb + (row * a.ldo + col) * 2) = o;
         }
     }
-#undef PF8_DMA
+#undef PF8_DMA_P
+#undef PF8_DMA_Q
 #undef PF8_LOAD_S
 #undef PF8_PFRAG
 #undef PF8_QFRAG
@@ -529,19 +497,11 @@ __global__ __launch_bounds__(512) void k_gemm_fwd256(const GemmArgs a) {
 static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, const char* where) {
     const size_t lds_bytes = 65536;
     if (mode == MODE_FWD) {
-        // 256x256 tiles; the grid is padded to a multiple of 8 so that every XCD gets an equal run
-        // short expert segments (grouped layouts with few rows per expert) take 128-row tiles
-        const bool short_rows = a.group != GROUP_NONE && a.E > 0 && a.Qrows / a.E < 768 && a.group == GROUP_CONTIG;
-        const int bq = short_rows ? 128 : 256;
-        const int64_t T = ((a.Prows + 255) / 256) * ((a.Qrows + bq - 1) / bq);
-        dim3 g256((unsigned)(((T + 7) / 8) * 8), grid.y);
-        if (bq == 256) {
-            if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd256<0, 256>), g256, dim3(512), 131072, st, a);
-            else hipLaunchKernelGGL((k_gemm_fwd256<1, 256>), g256, dim3(512), 131072, st, a);
-        } else {
-            if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd256<0, 128>), g256, dim3(512), 98304, st, a);
-            else hipLaunchKernelGGL((k_gemm_fwd256<1, 128>), g256, dim3(512), 98304, st, a);
-        }
+        const int64_t T128 = ((a.Prows + 255) / 256) * ((a.Qrows + 127) / 128);
+        // the grid is padded to a multiple of 8 so that every XCD gets an equal run of tiles
+        dim3 g128((unsigned)(((T128 + 7) / 8) * 8), grid.y);
+        if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd128<0>), g128, dim3(256), 81920, st, a);
+        else hipLaunchKernelGGL((k_gemm_fwd128<1>), g128, dim3(256), 81920, st, a);
     } else {
         hipLaunchKernelGGL((k_gemm<MODE_WGRAD, 1>), grid, dim3(256), lds_bytes, st, a);
     }
@@ -563,10 +523,8 @@ static int ensure_lds_attr() {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_FWD, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_FWD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_WGRAD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<0, 256>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<1, 256>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<0, 128>), hipFuncAttributeMaxDynamicSharedMemorySize, 98304);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd256<1, 128>), hipFuncAttributeMaxDynamicSharedMemorySize, 98304);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
     done = 1;
     return PF8_OK;
