@@ -302,79 +302,139 @@ struct SplitArgs {
     int32_t E;
 };
 
+// this thread's 8x8 patch as packed bf16 (one 16-byte chunk per row); an e4m3 source is dequantised
+// to bf16 first (q * s rounded to nearest even), which is what the un-fused chain feeds the quantizer
+__device__ __forceinline__ void load_patch_packed(const TileSrc& src, int64_t row0, int64_t col0, int g, int l, uint4 (&w)[8]) {
+    if (src.x) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w[i] = ld16(src.x + (row0 + 8 * g + i) * src.ld + col0 + 8 * l);
+    } else {
+        uint2 q[8];
+        float sc[8];
+        const int64_t KB = src.ld / 128;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int64_t r = row0 + 8 * g + i;
+            q[i] = *reinterpret_cast<const uint2*>(src.xq + r * src.ld + col0 + 8 * l);
+            sc[i] = src.xs_layout == 0 ? src.xs[r * KB + col0 / 128] : src.xs[(col0 / 128) * src.rows + r];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float f[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                f[j] = e4m3_to_f32((q[i].x >> (8 * j)) & 0xFFu) * sc[i];
+                f[4 + j] = e4m3_to_f32((q[i].y >> (8 * j)) & 0xFFu) * sc[i];
+            }
+            w[i] = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
+        }
+    }
+}
+
 // Row-scaled copy (optional) + column-scaled transposed copy of one 128x128 tile.
 //   SPLIT=false: q[M,K] + s, qt[K,M] + st                (fused quant+transpose)
 //   SPLIT=true : qt / st packed per expert               (transpose-split-quant), source bf16 or e4m3
+// Per element the kernel spends one masked copy, two packed-u16 max (row and column amax), one
+// unpack and two bracketing conversions; the 128 row scales and 128 column scales are each computed
+// once (threads 0..127 / 128..255) and handed round through LDS instead of sixteen times over.
 template <bool SPLIT, int LAYOUT>
-__global__ __launch_bounds__(256) void k_quant_rowcol(TileSrc src, int64_t M, int64_t K, uint8_t* __restrict__ q,
+__global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M, int64_t K, uint8_t* __restrict__ q,
                                                       float* __restrict__ s, uint8_t* __restrict__ qt, float* __restrict__ st,
                                                       SplitArgs sp, int pow2) {
-    __shared__ uint32_t lds_t[128 * LDT];
-    __shared__ uint32_t lds_cm[4 * 64];
+    __shared__ uint32_t lds_t[128 * LDT];      // transposed byte tile
+    __shared__ uint32_t lds_cm[4 * 64];        // per-wave packed column maxima
+    __shared__ uint32_t lds_rm[128];           // row maxima
+    __shared__ float4 lds_sc[256];             // (s, r_lo, r_hi, slow) for rows 0..127, columns 128..255
     const int tid = threadIdx.x, g = tid >> 4, l = tid & 15, wave = tid >> 6, lane = tid & 63;
     const int64_t tc = blockIdx.x, tr = blockIdx.y;
     const int64_t row0 = tr * 128, col0 = tc * 128;
     const int64_t KB = K / 128, MB = M / 128;
-    float v[8][8];
-    load_patch(src, row0, col0, g, l, v);
+    const bool want_rows = q != nullptr;
 
-    // column amax: this thread's 8 rows, then the 4 row groups of the wave, then the 4 waves via LDS
-    uint32_t cm[8];
+    uint4 w[8];
+    load_patch_packed(src, row0, col0, g, l, w);
+
+    // ---- amax on the packed magnitudes ----
+    uint32_t cmx = 0, cmy = 0, cmz = 0, cmw = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        uint32_t m = 0;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) m = umax(m, f2u(v[i][j]) & 0x7FFFFFFFu);
-        m = umax(m, (uint32_t)__shfl_xor((int)m, 16));
-        m = umax(m, (uint32_t)__shfl_xor((int)m, 32));
-        cm[j] = m;
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t ax = w[i].x & 0x7FFF7FFFu, ay = w[i].y & 0x7FFF7FFFu, az = w[i].z & 0x7FFF7FFFu, aw = w[i].w & 0x7FFF7FFFu;
+        cmx = pkmax_u16(cmx, ax); cmy = pkmax_u16(cmy, ay); cmz = pkmax_u16(cmz, az); cmw = pkmax_u16(cmw, aw);
+        if (want_rows) {
+            const uint32_t m = pkmax_u16(pkmax_u16(ax, ay), pkmax_u16(az, aw));
+            const uint32_t rm = row16_max(umax(m << 16, m & 0xFFFF0000u));
+            if (l == i) lds_rm[8 * g + i] = rm;
+        }
     }
+    // columns: the 4 row groups of this wave, then the 4 waves through LDS
+    cmx = pkmax_u16(cmx, (uint32_t)__shfl_xor((int)cmx, 16)); cmx = pkmax_u16(cmx, (uint32_t)__shfl_xor((int)cmx, 32));
+    cmy = pkmax_u16(cmy, (uint32_t)__shfl_xor((int)cmy, 16)); cmy = pkmax_u16(cmy, (uint32_t)__shfl_xor((int)cmy, 32));
+    cmz = pkmax_u16(cmz, (uint32_t)__shfl_xor((int)cmz, 16)); cmz = pkmax_u16(cmz, (uint32_t)__shfl_xor((int)cmz, 32));
+    cmw = pkmax_u16(cmw, (uint32_t)__shfl_xor((int)cmw, 16)); cmw = pkmax_u16(cmw, (uint32_t)__shfl_xor((int)cmw, 32));
     if (lane < 16) {
-        // bf16-derived magnitudes have 16 significant bits: pack two per dword
-#pragma unroll
-        for (int j = 0; j < 4; ++j) lds_cm[wave * 64 + 4 * l + j] = (cm[2 * j] >> 16) | (cm[2 * j + 1] & 0xFFFF0000u);
+        uint32_t* p = lds_cm + wave * 64 + 4 * l;
+        p[0] = cmx; p[1] = cmy; p[2] = cmz; p[3] = cmw;
     }
+    __syncthreads();
 
-    // row-scaled copy while the column maxima settle
-    if (q) {
+    // ---- one scale per row (threads 0..127) and per column (threads 128..255) ----
+    {
+        uint32_t am;
+        if (tid < 128) {
+            am = lds_rm[tid];
+        } else {
+            const int c = tid - 128;
+            const uint32_t pk = pkmax_u16(pkmax_u16(lds_cm[c >> 1], lds_cm[64 + (c >> 1)]), pkmax_u16(lds_cm[128 + (c >> 1)], lds_cm[192 + (c >> 1)]));
+            am = (c & 1) ? (pk & 0xFFFF0000u) : (pk << 16);
+        }
+        if (tid >= 128 || want_rows) {
+            const TileScale t = make_scale(am, pow2 != 0);
+            lds_sc[tid] = make_float4(t.s, t.r_lo, t.r_hi, t.slow ? 1.0f : 0.0f);
+        }
+    }
+    __syncthreads();
+
+    // ---- quantise: rows straight to memory, columns into the transposed LDS tile.  Values are
+    // unpacked from the packed patch where they are used (twice per element) instead of keeping 64
+    // floats live: the kernel stays under 128 registers, so four workgroups share a compute unit.
+    if (want_rows) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            uint32_t m = 0;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) m = umax(m, f2u(v[i][j]) & 0x7FFFFFFFu);
-            TileScale t = make_scale(row16_max(m), pow2 != 0);
-            uint2 o = quant8(v[i], t);
+            const float4 f = lds_sc[8 * g + i];
+            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f;
             const int64_t r = row0 + 8 * g + i;
-            st8(q + r * K + col0 + 8 * l, o);
+            float v[8];
+            unpack8(w[i], v);
+            st8(q + r * K + col0 + 8 * l, quant8(v, t));
             if (l == i) {
                 if (LAYOUT == 0) s[r * KB + tc] = t.s;
                 else s[tc * M + r] = t.s;
             }
         }
     }
-    __syncthreads();
-    uint32_t cmp[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        uint32_t a = pkmax_u16(lds_cm[0 * 64 + 4 * l + j], lds_cm[1 * 64 + 4 * l + j]);
-        uint32_t b = pkmax_u16(lds_cm[2 * 64 + 4 * l + j], lds_cm[3 * 64 + 4 * l + j]);
-        cmp[j] = pkmax_u16(a, b);
-    }
     float cs[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        uint32_t am = (j & 1) ? (cmp[j >> 1] & 0xFFFF0000u) : (cmp[j >> 1] << 16);
-        TileScale t = make_scale(am, pow2 != 0);
-        cs[j] = t.s;
-        float col[8];
+    for (int k = 0; k < 4; ++k) {
+        float lo[8], hi[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) col[i] = v[i][j];
-        lds_put_col(lds_t, l, g, j, quant8(col, t));
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t d = k == 0 ? w[i].x : k == 1 ? w[i].y : k == 2 ? w[i].z : w[i].w;
+            lo[i] = bf16_lo(d);
+            hi[i] = bf16_hi(d);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int j = 2 * k + h;
+            const float4 f = lds_sc[128 + 8 * l + j];
+            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f;
+            cs[j] = t.s;
+            lds_put_col(lds_t, l, g, j, h == 0 ? quant8(lo, t) : quant8(hi, t));
+        }
     }
     __syncthreads();
 
     // destination of the transposed tile
-    int64_t qt_base, st_row, ldq;
+    int64_t qt_base, ldq;
     if (SPLIT) {
         // expert of this row tile: linear scan of the prefix table (E <= 256, uniform per workgroup)
         int e = 0;
@@ -383,11 +443,9 @@ __global__ __launch_bounds__(256) void k_quant_rowcol(TileSrc src, int64_t M, in
         const int64_t Me = (int64_t)(sp.tile_start[e + 1] - sp.tile_start[e]) * 128;
         qt_base = off * K + (row0 - off);      // + c*Me
         ldq = Me;
-        st_row = tr;                           // scale rows are tile rows, globally numbered
     } else {
         qt_base = row0;
         ldq = M;
-        st_row = tr;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -397,7 +455,8 @@ __global__ __launch_bounds__(256) void k_quant_rowcol(TileSrc src, int64_t M, in
     }
     if (g == 0) {
         if (LAYOUT == 1 || SPLIT) {
-            float4* p = reinterpret_cast<float4*>(st + st_row * K + col0 + 8 * l);
+            // scale rows are tile rows, globally numbered (an expert's block starts at its first tile)
+            float4* p = reinterpret_cast<float4*>(st + tr * K + col0 + 8 * l);
             p[0] = make_float4(cs[0], cs[1], cs[2], cs[3]);
             p[1] = make_float4(cs[4], cs[5], cs[6], cs[7]);
         } else {
