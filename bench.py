@@ -108,6 +108,71 @@ def bench_quantizers(iters=20, warmup=5):
     return out
 
 
+def bench_other_gemms(iters=10, warmup=3):
+    """Kernel-only timings of the other BASELINE GEMM workloads (random e4m3 bytes and scales):
+    config 2 dense, config 5 forward grouped GEMMs and the config-5 weight gradient."""
+    import numpy as np
+    import torch
+
+    from paddleformers_amd import deep_gemm
+    from paddleformers_amd import functional as F8
+
+    fp8 = torch.float8_e4m3fn
+    out = {}
+
+    def rnd8(*shape):
+        return torch.randint(0, 120, shape, dtype=torch.uint8, device="cuda").view(fp8)
+
+    # config 2: [8192, 7168] x [4096, 7168]^T
+    M, N, K = 8192, 4096, 7168
+    a, b = rnd8(M, K), rnd8(N, K)
+    sa, sb = torch.rand((K // 128, M), device="cuda"), torch.rand((N // 128, K // 128), device="cuda")
+    o = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    ms = time_kernel(lambda: deep_gemm.fp8_gemm_nt((a, sa.T), (b, sb), o), [()], iters, warmup)
+    out["dense_config2_8192x4096x7168"] = {"flop": 2.0 * M * N * K, "ms": ms}
+    del a, b, o
+    # config 5 forward: E=128, H=4096, I=1408, 131072 routed rows, Zipf(1.0)
+    E, H, I, ROUTED = 128, 4096, 1408, 131072
+    counts, padded = zipf_counts(ROUTED, E, 1.0, seed=5, n_empty=0)
+    Mp = int(padded.sum())
+    mi = torch.from_numpy(np.repeat(np.arange(E, dtype=np.int32), padded)).cuda()
+    a = rnd8(Mp, H)
+    sa = torch.rand((H // 128, Mp), device="cuda")
+    w1, s1 = rnd8(E, 2 * I, H), torch.rand((E, 2 * I // 128, H // 128), device="cuda")
+    o1 = torch.empty((Mp, 2 * I), dtype=torch.bfloat16, device="cuda")
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa.T), (w1, s1), o1, mi), [()], iters, warmup)
+    out["grouped_config5_up_gate"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms, "padded_rows": Mp}
+    del w1, o1
+    a2, sa2 = rnd8(Mp, I), torch.rand((Mp, I // 128), device="cuda")
+    w2, s2 = rnd8(E, H, I), torch.rand((E, H // 128, I // 128), device="cuda")
+    o3 = torch.empty((Mp, H), dtype=torch.bfloat16, device="cuda")
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a2, sa2), (w2, s2), o3, mi), [()], iters, warmup)
+    out["grouped_config5_down"] = {"flop": 2.0 * ROUTED * I * H, "ms": ms, "padded_rows": Mp}
+    del a2, w2, o3
+    # config 5 weight gradient dW1[e] [H, 2I] += x_e^T . do1_e, all experts in one launch
+    rows = [int(r) for r in padded]
+    x = torch.randn((Mp, H), device="cuda").to(torch.bfloat16)
+    d = (torch.randn((Mp, 2 * I), device="cuda") * 1e-3).to(torch.bfloat16)
+    ms_q = time_kernel(lambda: F8.fused_transpose_split_quant(x, None, rows, True), [()], 5, 2)
+    out["transpose_split_quant_config5_x"] = {"bytes": Mp * H * 3 + (Mp // 128) * H * 4, "ms": ms_q}
+    a_t, sa_t = F8.fused_transpose_split_quant(x, None, rows, True)
+    b_t, sb_t = F8.fused_transpose_split_quant(d, None, rows, True)
+    del x, d
+    g = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True), [()], 5, 2)
+    out["grouped_wgrad_config5_dw1"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms}
+    for v in out.values():
+        if "flop" in v:
+            v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)
+            v["frac_fp8_peak"] = round(v["TFLOPs"] / FP8_PEAK_TFLOPS, 4)
+        else:
+            v["GBps"] = round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)
+            v["frac_hbm"] = round(v["GBps"] / HBM_PEAK_GBS, 4)
+        v["ms"] = round(v["ms"], 4)
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(H, I, rows=12288):
     """The CPU oracle on a bounded sample of the same pipeline: `rows` token rows of ONE expert
     (quant -> up+gate GEMM -> SwiGLU+requant -> down GEMM), OpenMP over the host cores."""
@@ -268,7 +333,10 @@ def main():
         },
     }
     if not args.no_quant:
+        del x, w1q, w1s, w2q, w2s, o1, o3
+        torch.cuda.empty_cache()
         res["quant"] = bench_quantizers()
+        res["other_gemm"] = bench_other_gemms()
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(H, I)
     print(json.dumps(res))
