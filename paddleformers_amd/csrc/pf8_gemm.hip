@@ -22,8 +22,6 @@
 
 namespace pf8 {
 
-constexpr int TILE = 128;
-
 enum { MODE_FWD = 0, MODE_WGRAD = 1 };
 enum { GROUP_NONE = 0, GROUP_CONTIG = 1, GROUP_MASKED = 2, GROUP_WGRAD = 3 };
 
@@ -58,208 +56,6 @@ __device__ __forceinline__ int swz_key(int row) {
 #endif
 }
 __device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ swz_key(row)) << 4); }
-
-template <int MODE, int SQL>
-__global__ __launch_bounds__(256, 2) void k_gemm(const GemmArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    // lds: [stage][P tile 16 KB | Q tile 16 KB]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wp = wave & 1, wq = wave >> 1;
-    const int li = lane & 15, kg = lane >> 4;
-
-    const int64_t p_tiles = (a.Prows + TILE - 1) / TILE;
-    const int64_t p_tile = blockIdx.x % p_tiles, q_tile = blockIdx.x / p_tiles;
-    const int64_t p0 = p_tile * TILE, q0 = q_tile * TILE;
-
-    const uint8_t* pbase = a.p;
-    const uint8_t* qbase = a.q;
-    const float* spb = a.sp;
-    const float* sqb = a.sq;
-    uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
-    int64_t ldp = a.red, ldq = a.red;        // row strides of the operands (bytes)
-    int64_t KBn = a.red / 128;               // K blocks to reduce over
-    int64_t q_valid = a.Qrows;               // rows of Q that may be stored
-    int64_t KBs = KBn;                       // K blocks per row in the scale tensors (forward)
-    const int64_t PB = (a.Prows + 127) / 128;
-
-    if (MODE == MODE_FWD) {
-        if (a.group == GROUP_CONTIG) {
-            const int e = a.m_indices[q0];
-            if (e < 0) return;
-            pbase += (int64_t)e * a.Prows * a.red;
-            spb += (int64_t)e * PB * KBs;
-        } else if (a.group == GROUP_MASKED) {
-            const int e = blockIdx.y;
-            const int64_t valid = a.masked_m[e];
-            if (q0 >= valid) return;
-            q_valid = valid;
-            pbase += (int64_t)e * a.Prows * a.red;
-            spb += (int64_t)e * PB * KBs;
-            qbase += (int64_t)e * a.Qrows * a.red;
-            sqb += (int64_t)e * a.Qrows * KBs;
-            outb += (int64_t)e * a.Qrows * a.ldo * 2;
-        }
-    } else {
-        if (a.group == GROUP_WGRAD) {
-            const int e = blockIdx.y;
-            const int64_t t0 = a.tile_start[e], t1 = a.tile_start[e + 1];
-            const int64_t Me = (t1 - t0) * 128;
-            // packed per-expert operands: [rows, Me] at rows*128*t0, scales [Me/128, rows] at t0*rows
-            pbase += a.Prows * 128 * t0;
-            qbase += a.Qrows * 128 * t0;
-            spb += t0 * a.Prows;
-            sqb += t0 * a.Qrows;
-            outb += (int64_t)e * a.Qrows * a.ldo * 4;
-            ldp = ldq = Me;
-            KBn = t1 - t0;
-            if (KBn == 0 && a.accumulate) return;
-        }
-    }
-
-    // ---- global -> LDS staging: thread copies chunk (tid&7) of rows (tid>>3) + 32*i ------------
-    const int crow = tid >> 3, cchunk = tid & 7;
-    const uint8_t* gp[4];
-    const uint8_t* gq[4];
-    int lofs[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = crow + 32 * i;
-        int64_t pr = p0 + row; if (pr > a.Prows - 1) pr = a.Prows - 1;
-        int64_t qr = q0 + row; if (qr > a.Qrows - 1) qr = a.Qrows - 1;
-        gp[i] = pbase + pr * ldp + cchunk * 16;
-        gq[i] = qbase + qr * ldq + cchunk * 16;
-        lofs[i] = swz(row, cchunk);
-    }
-    uint4 rp[4], rq[4];
-#define PF8_G_LOAD(kb_)                                                          \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                              \
-        rp[i] = *reinterpret_cast<const uint4*>(gp[i] + (kb_) * 128);            \
-        rq[i] = *reinterpret_cast<const uint4*>(gq[i] + (kb_) * 128);            \
-    }
-#define PF8_L_STORE(stage_)                                                      \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                              \
-        *reinterpret_cast<uint4*>(lds + (stage_) * 32768 + lofs[i]) = rp[i];     \
-        *reinterpret_cast<uint4*>(lds + (stage_) * 32768 + 16384 + lofs[i]) = rq[i]; \
-    }
-
-    // ---- fragment addresses --------------------------------------------------------------------
-    int fofs_p[4][2], fofs_q[4][2];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        const int prow = wp * 64 + t * 16 + li, qrow = wq * 64 + t * 16 + li;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            fofs_p[t][h] = swz(prow, 2 * kg + h);
-            fofs_q[t][h] = 16384 + swz(qrow, 2 * kg + h);
-        }
-    }
-
-    // ---- scale addressing ----------------------------------------------------------------------
-    // forward: lane needs sq of its 4 output rows (one per q sub-tile) and the block scale of P
-    // wgrad  : lane needs sq of its 4 output rows and sp of its 16 output columns (4 x float4)
-    int64_t qrow_g[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        int64_t r = q0 + wq * 64 + t * 16 + li;
-        if (r > a.Qrows - 1) r = a.Qrows - 1;
-        qrow_g[t] = r;
-    }
-    int64_t pcol_g[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        int64_t c = p0 + wp * 64 + t * 16 + 4 * kg;
-        if (c > a.Prows - 4) c = a.Prows - 4;
-        pcol_g[t] = c;
-    }
-    float fq[4];
-    f32x4 fp4[4];
-    float fpb = 0.0f;
-    auto s_load = [&](int64_t kb) {
-        if (MODE == MODE_FWD) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) fq[t] = SQL == 0 ? sqb[qrow_g[t] * KBs + kb] : sqb[kb * a.Qrows + qrow_g[t]];
-            fpb = spb[p_tile * KBs + kb];
-        } else {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                fq[t] = sqb[kb * a.Qrows + qrow_g[t]];
-                fp4[t] = *reinterpret_cast<const f32x4*>(spb + kb * a.Prows + pcol_g[t]);
-            }
-        }
-    };
-
-    f32x4 acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-    if (KBn > 0) {
-        PF8_G_LOAD(0)
-        PF8_L_STORE(0)
-    }
-    __syncthreads();
-
-    for (int64_t kb = 0; kb < KBn; ++kb) {
-        const int cur = (int)(kb & 1);
-        // prefetch the next K block into registers (the last iteration re-reads its own block:
-        // no branch, so the staging registers never leave the register file)
-        const int64_t kbn = kb + 1 < KBn ? kb + 1 : kb;
-        PF8_G_LOAD(kbn)
-        s_load(kb);
-        const uint8_t* base = lds + cur * 32768;
-        i32x8 pf[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            i32x4 lo = *reinterpret_cast<const i32x4*>(base + fofs_p[t][0]);
-            i32x4 hi = *reinterpret_cast<const i32x4*>(base + fofs_p[t][1]);
-            pf[t] = (i32x8){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        }
-#pragma unroll
-        for (int qs = 0; qs < 4; ++qs) {
-            i32x4 lo = *reinterpret_cast<const i32x4*>(base + fofs_q[qs][0]);
-            i32x4 hi = *reinterpret_cast<const i32x4*>(base + fofs_q[qs][1]);
-            i32x8 qf = (i32x8){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            float f = MODE == MODE_FWD ? fq[qs] * fpb : fq[qs];
-#pragma unroll
-            for (int ps = 0; ps < 4; ++ps) {
-                f32x4 d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps], qf, (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                if (MODE == MODE_FWD) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[ps][qs][r] = __builtin_fmaf(d[r], f, acc[ps][qs][r]);
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[ps][qs][r] = __builtin_fmaf(d[r] * f, fp4[ps][r], acc[ps][qs][r]);
-                }
-            }
-        }
-        PF8_L_STORE(cur ^ 1)
-        __syncthreads();
-    }
-
-    // ---- epilogue ------------------------------------------------------------------------------
-#pragma unroll
-    for (int qs = 0; qs < 4; ++qs) {
-        const int64_t row = q0 + wq * 64 + qs * 16 + li;
-        if (row >= q_valid) continue;
-#pragma unroll
-        for (int ps = 0; ps < 4; ++ps) {
-            const int64_t col = p0 + wp * 64 + ps * 16 + 4 * kg;
-            if (col + 4 > a.Prows) continue;
-            if (MODE == MODE_FWD) {
-                uint2 o;
-                o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
-                o.y = pack_bf16(acc[ps][qs][2], acc[ps][qs][3]);
-                *reinterpret_cast<uint2*>(outb + (row * a.ldo + col) * 2) = o;
-            } else {
-                f32x4* dst = reinterpret_cast<f32x4*>(outb + (row * a.ldo + col) * 4);
-                f32x4 v = acc[ps][qs];
-                if (a.accumulate) { f32x4 old = *dst; v = (f32x4){old.x + v.x, old.y + v.y, old.z + v.z, old.w + v.w}; }
-                *dst = v;
-            }
-        }
-    }
-}
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
@@ -472,19 +268,38 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
     }
     __builtin_amdgcn_s_waitcnt(0);
 
+    // ---- epilogue: bf16 through LDS so that every store instruction writes whole 256-byte rows
+    // (straight from the MFMA layout a lane owns 4 consecutive outputs and a store instruction
+    // covers 32-byte row pieces: measured 17% of the kernel's time on the dense configuration) ----
+    constexpr int EP_LD = 272;                   // 128 bf16 per row + 16 B pad
+    __syncthreads();                             // everyone is done reading fragments
+    uint8_t* ep = lds + wave * (64 * EP_LD);
 #pragma unroll
-    for (int qs = 0; qs < 4; ++qs) {
-        const int rt = wq * 64 + qs * 16 + li;
-        const int64_t row = q0 + rt;
-        if (rt >= row_hi || row >= q_rows_total) continue;
+    for (int qs = 0; qs < 4; ++qs)
 #pragma unroll
         for (int ps = 0; ps < NPS; ++ps) {
-            const int64_t col = p0 + wp * 128 + ps * 16 + 4 * kg;
-            if (col + 4 > a.Prows) continue;
             uint2 o;
             o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
             o.y = pack_bf16(acc[ps][qs][2], acc[ps][qs][3]);
-            *reinterpret_cast<uint2*>(outb + (row * a.ldo + col) * 2) = o;
+            *reinterpret_cast<uint2*>(ep + (qs * 16 + li) * EP_LD + (ps * 16 + 4 * kg) * 2) = o;
+        }
+    // LDS operations of one wavefront execute in order: the reads below see the writes above
+    const int er = lane >> 4, ec = lane & 15;
+    const int64_t col = p0 + wp * 128 + ec * 8;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int rt = wq * 64 + er + 4 * i;     // row inside the tile
+        const int64_t row = q0 + rt;
+        const uint4 v = *reinterpret_cast<const uint4*>(ep + (er + 4 * i) * EP_LD + ec * 16);
+        if (rt >= row_hi || row >= q_rows_total) continue;
+        uint8_t* dst = outb + (row * a.ldo + col) * 2;
+        if (col + 8 <= a.Prows) {
+#ifdef PF8_ABL_NOSTORE
+            if (v.x == 0x12345678u)
+#endif
+            *reinterpret_cast<uint4*>(dst) = v;
+        } else if (col + 4 <= a.Prows) {
+            *reinterpret_cast<uint2*>(dst) = make_uint2(v.x, v.y);
         }
     }
 #undef PF8_DMA_P
@@ -494,8 +309,194 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
 #undef PF8_QFRAG
 }
 
+// ---------------------------------------------------------------------------------------------
+// Weight-gradient kernel: out[Q rows, P rows] (+)= Q . P^T with BOTH operands 1x128-scaled along the
+// reduction axis, fp32 output.  128(Q) x 128(P) x 128(K) tiles, 256 threads = 4 wavefronts (2 x 2,
+// 64x64 each), two double-buffered 32 KB LDS stages (64 KB: two workgroups per compute unit), the
+// same global->LDS copies, fragment order and pinned MFMA/FMA interleave as the forward kernel.
+// Every product needs two scales, sq[row] * sp[col], so eight VALU operations follow each MFMA
+// (one multiply and one FMA per element): this kernel is bound by the vector ALU at about half
+// the MFMA rate, and on the grouped layout by the fp32 read-modify-write of the gradients.
+// The per-lane scales of the next K block are loaded BEFORE that block's copies are issued: vector
+// memory operations complete in order, so a scale load issued after the copies would make every
+// later wait on it wait for the copies as well.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
+    constexpr int NPS = 4, STAGE = 32768, Q_OFS = 16384;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wq = wave >> 1, wp = wave & 1;
+    const int li = lane & 15, kg = lane >> 4;
+
+    const int64_t p_tiles = (a.Prows + 127) / 128, q_tiles = (a.Qrows + 127) / 128;
+    const int64_t T = p_tiles * q_tiles;
+    const int64_t per_xcd = (T + 7) / 8;
+    const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= T) return;
+    const int64_t p_tile = logical % p_tiles, q_tile = logical / p_tiles;
+    const int64_t p0 = p_tile * 128, q0 = q_tile * 128;
+
+    const uint8_t* pbase = a.p;
+    const uint8_t* qbase = a.q;
+    const float* spb = a.sp;
+    const float* sqb = a.sq;
+    uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
+    int64_t ld = a.red;             // row stride of both operands = reduction length
+    int64_t KB = a.red / 128;
+    if (a.group == GROUP_WGRAD) {
+        const int e = blockIdx.y;
+        const int64_t t0 = a.tile_start[e], t1 = a.tile_start[e + 1];
+        // packed per-expert operands: [rows, M_e] at rows*128*t0, scales [M_e/128, rows] at t0*rows
+        pbase += a.Prows * 128 * t0;
+        qbase += a.Qrows * 128 * t0;
+        spb += t0 * a.Prows;
+        sqb += t0 * a.Qrows;
+        outb += (int64_t)e * a.Qrows * a.ldo * 4;
+        ld = (t1 - t0) * 128;
+        KB = t1 - t0;
+        if (KB == 0 && a.accumulate) return;
+    }
+
+    const int crow = lane >> 3, cpos = lane & 7;
+    uint32_t p_src[4], q_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = (i * 4 + wave) * 8 + crow;             // 0..127
+        const int chunk = cpos ^ swz_key(row);
+        int64_t pr = p0 + row; if (pr > a.Prows - 1) pr = a.Prows - 1;
+        int64_t qr = q0 + row; if (qr > a.Qrows - 1) qr = a.Qrows - 1;
+        p_src[i] = (uint32_t)((pr - p0) * ld + chunk * 16);
+        q_src[i] = (uint32_t)((qr - q0) * ld + chunk * 16);
+    }
+    const uint8_t* ptile = pbase + p0 * ld;
+    const uint8_t* qtile = qbase + q0 * ld;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    int fp_ofs[2], fq_ofs[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        fp_ofs[h] = swz(wp * 64 + li, 2 * kg + h);
+        fq_ofs[h] = Q_OFS + swz(wq * 64 + li, 2 * kg + h);
+    }
+    // scale addresses: one Q row per q sub-tile, four consecutive P rows per p sub-tile
+    const float* sq_ptr[4];
+    const float* sp_ptr[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        int64_t r = q0 + wq * 64 + t * 16 + li;
+        if (r > a.Qrows - 1) r = a.Qrows - 1;
+        sq_ptr[t] = sqb + r;
+        int64_t c = p0 + wp * 64 + t * 16 + 4 * kg;
+        if (c > a.Prows - 4) c = a.Prows - 4;
+        sp_ptr[t] = spb + c;
+    }
+
+    f32x4 acc[NPS][4];
+#pragma unroll
+    for (int i = 0; i < NPS; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float fq_nxt[4];
+    f32x4 fp_nxt[4];
+
+#define PF8_DMA(kb_, stage_)                                                                           \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                      \
+        dma16_to_lds(ptile + p_src[i] + (kb_) * 128, lds_base + (stage_) * STAGE + (i * 4 + wave) * 1024); \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                      \
+        dma16_to_lds(qtile + q_src[i] + (kb_) * 128, lds_base + (stage_) * STAGE + Q_OFS + (i * 4 + wave) * 1024);
+#define PF8_LOAD_S(kb_)                                                                                \
+    _Pragma("unroll") for (int t = 0; t < 4; ++t) {                                                    \
+        fq_nxt[t] = sq_ptr[t][(kb_) * a.Qrows];                                                        \
+        fp_nxt[t] = *reinterpret_cast<const f32x4*>(sp_ptr[t] + (kb_) * a.Prows);                      \
+    }
+#define PF8_PFRAG(ps_) ld_frag_lds(base + fp_ofs[0] + (ps_) * 2048, base + fp_ofs[1] + (ps_) * 2048)
+#define PF8_QFRAG(qs_) ld_frag_lds(base + fq_ofs[0] + (qs_) * 2048, base + fq_ofs[1] + (qs_) * 2048)
+
+    if (KB > 0) {
+        PF8_LOAD_S(0)
+        __builtin_amdgcn_sched_barrier(0);
+        PF8_DMA(0, 0)
+    }
+    for (int64_t kb = 0; kb < KB; ++kb) {
+        const int cur = (int)(kb & 1);
+        __builtin_amdgcn_s_waitcnt(0);   // this wave's copies and scale loads have landed
+        __syncthreads();                 // everyone's copies landed; everyone is done with stage cur^1
+        float fq_cur[4];
+        f32x4 fp_cur[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) { fq_cur[t] = fq_nxt[t]; fp_cur[t] = fp_nxt[t]; }
+        const int64_t kbn = kb + 1 < KB ? kb + 1 : kb;
+        PF8_LOAD_S(kbn)
+        __builtin_amdgcn_sched_barrier(0);
+        PF8_DMA(kbn, cur ^ 1)
+        const uint8_t* base = lds + cur * STAGE;
+        i32x8 pf[NPS], qf[4];
+        f32x4 d[3];
+        pf[0] = PF8_PFRAG(0);
+        __builtin_amdgcn_sched_barrier(0);
+        qf[0] = PF8_QFRAG(0);
+        __builtin_amdgcn_sched_barrier(0);
+        qf[1] = PF8_QFRAG(1);
+        __builtin_amdgcn_sched_barrier(0);
+        qf[2] = PF8_QFRAG(2);
+        __builtin_amdgcn_sched_barrier(0);
+        qf[3] = PF8_QFRAG(3);
+        __builtin_amdgcn_sched_barrier(0);
+        pf[1] = PF8_PFRAG(1);
+        __builtin_amdgcn_sched_barrier(0);
+        pf[2] = PF8_PFRAG(2);
+        __builtin_amdgcn_sched_barrier(0);
+        pf[3] = PF8_PFRAG(3);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < NPS * 4; ++j) {
+            const int ps = j >> 2, qs = j & 3;
+            d[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps], qf[qs], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j >= 2) {
+                const int jj = j - 2;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r] * fq_cur[jj & 3], fp_cur[jj >> 2][r], acc[jj >> 2][jj & 3][r]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int jj = NPS * 4 - 2; jj < NPS * 4; ++jj)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                acc[jj >> 2][jj & 3][r] = __builtin_fmaf(d[jj % 3][r] * fq_cur[jj & 3], fp_cur[jj >> 2][r], acc[jj >> 2][jj & 3][r]);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+
+    // ---- epilogue: fp32 through LDS so that every load/store instruction touches whole 256-byte
+    // rows of the gradient; optional read-modify-write ----
+    constexpr int EP_LD = 272;                   // 64 fp32 per row + 16 B pad
+    __syncthreads();                             // everyone is done reading fragments
+    uint8_t* ep = lds + wave * (64 * EP_LD);
+#pragma unroll
+    for (int qs = 0; qs < 4; ++qs)
+#pragma unroll
+        for (int ps = 0; ps < NPS; ++ps)
+            *reinterpret_cast<f32x4*>(ep + (qs * 16 + li) * EP_LD + (ps * 16 + 4 * kg) * 4) = acc[ps][qs];
+    const int er = lane >> 4, ec = lane & 15;
+    const int64_t col = p0 + wp * 64 + ec * 4;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int64_t row = q0 + wq * 64 + er + 4 * i;
+        f32x4 v = *reinterpret_cast<const f32x4*>(ep + (er + 4 * i) * EP_LD + ec * 16);
+        if (row >= a.Qrows || col + 4 > a.Prows) continue;
+        f32x4* dst = reinterpret_cast<f32x4*>(outb + (row * a.ldo + col) * 4);
+        if (a.accumulate) { const f32x4 old = *dst; v = (f32x4){old.x + v.x, old.y + v.y, old.z + v.z, old.w + v.w}; }
+        *dst = v;
+    }
+#undef PF8_DMA
+#undef PF8_LOAD_S
+#undef PF8_PFRAG
+#undef PF8_QFRAG
+}
+
 static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, const char* where) {
-    const size_t lds_bytes = 65536;
+    const size_t lds_bytes = 69632;   // two 32 KB stages; the fp32 epilogue staging needs 4 x 64 x 272 B
     if (mode == MODE_FWD) {
         const int64_t T128 = ((a.Prows + 255) / 256) * ((a.Qrows + 127) / 128);
         // the grid is padded to a multiple of 8 so that every XCD gets an equal run of tiles
@@ -503,7 +504,9 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd128<0>), g128, dim3(256), 81920, st, a);
         else hipLaunchKernelGGL((k_gemm_fwd128<1>), g128, dim3(256), 81920, st, a);
     } else {
-        hipLaunchKernelGGL((k_gemm<MODE_WGRAD, 1>), grid, dim3(256), lds_bytes, st, a);
+        const int64_t Tw = ((a.Prows + 127) / 128) * ((a.Qrows + 127) / 128);
+        dim3 gw((unsigned)(((Tw + 7) / 8) * 8), grid.y);
+        hipLaunchKernelGGL(k_gemm_wgrad, gw, dim3(256), lds_bytes, st, a);
     }
     return pf8_check_launch(where);
 }
@@ -520,9 +523,7 @@ static int ensure_lds_attr() {
     static int done = 0;
     if (done) return PF8_OK;
     hipError_t e = hipSuccess;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_FWD, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_FWD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm<MODE_WGRAD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_wgrad), hipFuncAttributeMaxDynamicSharedMemorySize, 69632);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
