@@ -294,9 +294,6 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
         if (rt >= row_hi || row >= q_rows_total) continue;
         uint8_t* dst = outb + (row * a.ldo + col) * 2;
         if (col + 8 <= a.Prows) {
-#ifdef PF8_ABL_NOSTORE
-            if (v.x == 0x12345678u)
-#endif
             *reinterpret_cast<uint4*>(dst) = v;
         } else if (col + 4 <= a.Prows) {
             *reinterpret_cast<uint2*>(dst) = make_uint2(v.x, v.y);
