@@ -30,8 +30,8 @@ FP8_PEAK_TFLOPS = 5000.0
 # runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
 # counter reads for the 1 GiB pf8::k_debug_copy launched with --copy-yardstick (FETCH_SIZE reads
 # 0.5 KiB per KiB copied -> factor 2.0; WRITE_SIZE reads 1.0 -> factor 1.0):
-#   1,078,419 KiB x 2.0 + 79,872 KiB x 1.0 = 2,236,710 KiB.   Summary: profiles/gemm_up_gate_config3_hbm_traffic.md
-GEMM_UP_GATE_TRAFFIC_BYTES = 2236710 * 1024
+#   868,055 KiB x 2.0 + 79,872 KiB x 1.0 = 1,815,982 KiB.   Summary: profiles/gemm_up_gate_config3_hbm_traffic.md
+GEMM_UP_GATE_TRAFFIC_BYTES = 1815982 * 1024
 
 
 def zipf_counts(total, E, s, seed, n_empty=2, pad=128):
@@ -341,7 +341,7 @@ def main():
         "frac_fp8_peak": round(value / FP8_PEAK_TFLOPS, 4),
         "kernel_ms": {k: round(v, 4) for k, v in kms.items()},
         "roofline": {
-            "kernel": "pf8::k_gemm_fwd128<1> (up+gate grouped GEMM)",
+            "kernel": "pf8::k_gemm_fwd_deep<1> (up+gate grouped GEMM)",
             "bound": "mfma",
             "achieved": round(ach, 2),
             "peak": FP8_PEAK_TFLOPS,
