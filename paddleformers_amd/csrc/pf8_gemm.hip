@@ -307,15 +307,25 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Deep-pipeline forward kernel for shapes without ragged tiles (Prows % 256 == 0, Qrows % 128 == 0):
-// one workgroup per compute unit, 144 KB of LDS as a three-stage ring of [P 32 KB | Q 16 KB] blocks.
-// The copies of block kb+2 are issued during block kb, one between every other MFMA, so a copy has
-// two block times to land and no wavefront ever queues a burst of twelve; one barrier per block.
-// All global addresses are a scalar base plus one per-lane 32-bit offset (the swizzled chunk a lane
-// fetches does not depend on the copy index), which keeps the kernel under 256 registers without
-// spilling MFMA results through AGPRs.  Every memory instruction of the loop is inline assembly so
-// that vmcnt is counted by hand: per block a wavefront issues 4 scale loads and 12 copies, in that
-// order, and the wait at the head of a block leaves exactly the 12 youngest copies outstanding.
+// Deep-pipeline forward kernel for shapes without ragged tiles (Prows % 256 == 0, Qrows % 128 == 0,
+// at least three K blocks; dense and contiguous-grouped layouts).
+//   * One persistent workgroup per compute unit walks its XCD's run of 128x256 tiles; 144 KB of LDS
+//     is a three-stage ring of [P 32 KB | Q 16 KB] blocks that runs on ACROSS tile boundaries: the
+//     copies of the block two ahead are issued during the current block, one between every other
+//     MFMA, whether that block belongs to this tile or the next.  A tile therefore has no fill
+//     phase of its own, and a copy has two block times to land.
+//   * One barrier per block, placed before MFMA 24 of 32: by then every fragment read of the block
+//     has been issued, and behind the barrier the first fragments of the next block are read into
+//     the registers that come free (P6 and P7 are interleaved at the end for that), so the matrix
+//     pipe does not drain at a block boundary.
+//   * All global addresses are a scalar base plus one per-lane 32-bit offset (the swizzled chunk a
+//     lane fetches does not depend on the copy index): 224 registers, MFMA results stay in VGPRs.
+//   * Every memory instruction of the loop is inline assembly so that vmcnt is counted by hand: per
+//     block a wavefront issues 4 scale loads and then 12 copies, loads retire in issue order, and
+//     the wait before the barrier leaves exactly the 12 youngest copies outstanding (the stores of a
+//     finished tile are older than those and simply retire with them).
+//   * The epilogue stages bf16 rows in the LDS stage the tile's last block has just left, 32 rows
+//     per wavefront at a time, and writes whole 256-byte rows.
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ void dma16_s(uint32_t voff, const uint8_t* sbase, uint32_t lds_dst) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase), "s"(lds_dst) : "memory");
@@ -333,42 +343,50 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
 
     const int64_t p_tiles = a.Prows / 256, q_tiles = a.Qrows / BQ;
     const int64_t T = p_tiles * q_tiles;
+    // consecutive workgroups go round-robin to the 8 XCDs: every XCD owns a contiguous run of
+    // logical tiles (groups of 16 q-tiles x all p-tiles), walked W tiles at a time by its W workgroups
     const int64_t per_xcd = (T + 7) / 8;
-    const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= T) return;
-    constexpr int G = 16;
-    const int64_t grp = logical / (G * p_tiles), rem = logical % (G * p_tiles);
-    const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;
-    const int64_t q_tile = grp * G + rem % gq, p_tile = rem / gq;
-    const int64_t p0 = p_tile * 256, q0 = q_tile * BQ;
-
+    const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, W = gridDim.x >> 3;
     const int64_t KB = a.red / 128;
     const int64_t PB = a.Prows / 128;
-    const uint8_t* qbase = a.q;
-    const float* sqb = a.sq;
-    uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
     const int64_t q_rows_total = a.Qrows;
-    int e = 0, row_hi = BQ;
-    if (a.group == GROUP_CONTIG) {
-        e = __builtin_amdgcn_readfirstlane(a.m_indices[q0]);
-        if (e < 0) return;
-    } else if (a.group == GROUP_MASKED) {
-        e = blockIdx.y;
-        const int64_t valid = a.masked_m[e];
-        if (q0 >= valid) return;
-        row_hi = valid - q0 < BQ ? (int)(valid - q0) : BQ;
-        qbase += (int64_t)e * a.Qrows * a.red;
-        sqb += (int64_t)e * a.Qrows * KB;
-        outb += (int64_t)e * a.Qrows * a.ldo * 2;
-    }
+    const bool grouped = a.group == GROUP_CONTIG;
+
+    auto tile_coords = [&](int64_t n, int64_t& q_tile, int64_t& p_tile) -> bool {
+        constexpr int G = 16;
+        const int64_t loc = slot + n * W, logical = xcd * per_xcd + loc;
+        if (loc >= per_xcd || logical >= T) return false;
+        const int64_t grp = logical / (G * p_tiles), rem = logical % (G * p_tiles);
+        const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;
+        q_tile = grp * G + rem % gq;
+        p_tile = rem / gq;
+        return true;
+    };
+
+    // current tile (c_*) and next tile (n_*): everything here is wave-uniform
+    int64_t cq = 0, cp = 0, nq = 0, np = 0;
+    if (!tile_coords(0, cq, cp)) return;
+    int ce = 0;
+    if (grouped) ce = __builtin_amdgcn_readfirstlane(a.m_indices[cq * BQ]);
+    int c_rows = ce < 0 ? 0 : BQ;          // rows of the tile that are stored (none for a padding tile)
+    if (ce < 0) ce = 0;
+    const uint8_t* c_ptile = a.p + ((int64_t)ce * a.Prows + cp * 256) * a.red;
+    const uint8_t* c_qtile = a.q + cq * BQ * a.red;
+    const float* c_spb = a.sp + ((int64_t)ce * PB + cp * 2 + wp) * KB;
+    const float* c_sq0 = SQL == 0 ? a.sq + (cq * BQ + wq * 64) * KB : a.sq + cq * BQ + wq * 64;
+    const uint8_t* n_ptile = c_ptile;
+    const uint8_t* n_qtile = c_qtile;
+    const float* n_spb = c_spb;
+    const float* n_sq0 = c_sq0;
+    int n_rows = 0;
 
     // copy i of a wavefront fills rows (4 i + wave) * 8 + (lane >> 3) of the tile; the 16-byte chunk a
     // lane fetches is (lane & 7) ^ swz_key(row), and swz_key depends on lane and wave only
     const int crow = lane >> 3, cpos = lane & 7;
     const uint32_t c_off = (uint32_t)((wave * 8 + crow) * a.red + ((cpos ^ swz_key(wave * 8 + crow)) << 4));
     const int64_t copy_step = 32 * a.red;                       // 32 rows between copy i and i+1
-    const uint8_t* qtile = qbase + q0 * a.red;
-    const uint8_t* ptile = a.p + ((int64_t)e * a.Prows + p0) * a.red;
+    const int64_t sq_t = SQL == 0 ? 16 * KB : 16;               // floats between the scale rows of t and t+1
+    const int64_t sq_k = SQL == 0 ? 1 : q_rows_total;           // floats between K blocks
     const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
     int fp_ofs[2], fq_ofs[2];
 #pragma unroll
@@ -376,47 +394,31 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         fp_ofs[h] = swz(wp * 128 + li, 2 * kg + h);
         fq_ofs[h] = Q_OFS + swz(wq * 64 + li, 2 * kg + h);
     }
-    // Q scales of rows q0 + wq*64 + 16 t + li: scalar base per t, per-lane offset li
-    const int64_t qr0 = q0 + wq * 64;
     const uint32_t s_off = SQL == 0 ? (uint32_t)(li * KB * 4) : (uint32_t)(li * 4);
-    const float* spb = a.sp + ((int64_t)e * PB + p_tile * 2 + wp) * KB;
 
     f32x4 acc[NPS][4];
-#pragma unroll
-    for (int i = 0; i < NPS; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float fq_nxt[4], fpb_nxt = 0.f;
 
-#define PF8_COPY(i_, kb_, stage_)                                                                      \
+#define PF8_COPY(i_, pt_, qt_, stage_)                                                                 \
     do {                                                                                               \
-        if ((i_) < 8) dma16_s(c_off, ptile + (kb_) * 128 + (i_) * copy_step,                           \
-                              lds_base + (stage_) * STAGE + ((i_) * 4 + wave) * 1024);                 \
-        else dma16_s(c_off, qtile + (kb_) * 128 + ((i_) - 8) * copy_step,                              \
-                     lds_base + (stage_) * STAGE + Q_OFS + (((i_) - 8) * 4 + wave) * 1024);            \
+        if ((i_) < 8) dma16_s(c_off, (pt_) + (i_) * copy_step, lds_base + (stage_) * STAGE + ((i_) * 4 + wave) * 1024); \
+        else dma16_s(c_off, (qt_) + ((i_) - 8) * copy_step, lds_base + (stage_) * STAGE + Q_OFS + (((i_) - 8) * 4 + wave) * 1024); \
     } while (0)
-#define PF8_LOAD_S(kb_)                                                                                \
+#define PF8_LOAD_S(sq_, sp_)                                                                           \
     _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                      \
-        asm volatile("global_load_dword %0, %1, %2" : "=v"(fq_nxt[t])                                  \
-                     : "v"(s_off), "s"(SQL == 0 ? sqb + (qr0 + 16 * t) * KB + (kb_) : sqb + (kb_) * q_rows_total + qr0 + 16 * t) \
-                     : "memory");                                                                      \
-    asm volatile("s_load_dword %0, %1, 0x0" : "=s"(fpb_nxt) : "s"(spb + (kb_)) : "memory");
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(fq_nxt[t]) : "v"(s_off), "s"((sq_) + t * sq_t) : "memory"); \
+    asm volatile("s_load_dword %0, %1, 0x0" : "=s"(fpb_nxt) : "s"(sp_) : "memory");
 #define PF8_PFRAG(ps_) ld_frag_lds(pbase + fp_ofs[0] + (ps_) * 2048, pbase + fp_ofs[1] + (ps_) * 2048)
 #define PF8_QFRAG(qs_) ld_frag_lds(pbase + fq_ofs[0] + (qs_) * 2048, pbase + fq_ofs[1] + (qs_) * 2048)
 
-    // MFMA order inside a block: P fragments 0..5 against Q0..Q3 each, then P6 and P7 interleaved
-    // (P6 Q0, P7 Q0, P6 Q1, ...) so that the Q registers come free one by one while the block still
-    // has MFMAs to issue; the first fragments of the NEXT block are read into them behind the
-    // block's only barrier, which sits before MFMA 24.  A block therefore starts with its operands
-    // in registers and the matrix pipe never drains at a block boundary.
     i32x8 pf[4], qf[4];
-    if (KB > 0) {
-        const int64_t k1 = KB > 1 ? 1 : 0;
+    {
+        // fill: blocks 0 and 1 of the first tile
 #pragma unroll
-        for (int i = 0; i < 12; ++i) PF8_COPY(i, 0, 0);
-        PF8_LOAD_S(0)
+        for (int i = 0; i < 12; ++i) PF8_COPY(i, c_ptile, c_qtile, 0);
+        PF8_LOAD_S(c_sq0, c_spb)
 #pragma unroll
-        for (int i = 0; i < 12; ++i) PF8_COPY(i, k1, 1);
+        for (int i = 0; i < 12; ++i) PF8_COPY(i, c_ptile + 128, c_qtile + 128, 1);
         asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)"
                      : "+v"(fq_nxt[0]), "+v"(fq_nxt[1]), "+v"(fq_nxt[2]), "+v"(fq_nxt[3]), "+s"(fpb_nxt) : : "memory");
         __syncthreads();
@@ -428,94 +430,139 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         qf[2] = PF8_QFRAG(2);
     }
     int cur = 0;
-    for (int64_t kb = 0; kb < KB; ++kb) {
-        float fq_cur[4];
+    for (int64_t n = 0;; ++n) {
+        // coordinates of the next tile; its expert id is fetched by a scalar load that the first
+        // barrier wait of this tile covers, and its addresses are formed at the head of block 1
+        const bool n_valid = tile_coords(n + 1, nq, np);
+        int ne = 0;
+        if (n_valid && grouped) asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ne) : "s"(a.m_indices + nq * BQ) : "memory");
 #pragma unroll
-        for (int t = 0; t < 4; ++t) fq_cur[t] = fq_nxt[t] * fpb_nxt;
-        const int nxt1 = cur == 2 ? 0 : cur + 1;         // stage of block kb+1
-        const int nxt2 = cur >= 1 ? cur - 1 : cur + 2;   // (cur + 2) % 3: the stage block kb-1 used
-        // past the end the copies and scale loads repeat the last block: the same instruction count
-        // in every block keeps the vmcnt arithmetic fixed, and the stage they land in is free
-        const int64_t kb1 = kb + 1 < KB ? kb + 1 : KB - 1, kb2 = kb + 2 < KB ? kb + 2 : KB - 1;
-        PF8_LOAD_S(kb1)
-        const uint8_t* pbase = lds + cur * STAGE;
-        const uint8_t* nbase = lds + nxt1 * STAGE;
-        f32x4 d[3];
-        qf[3] = PF8_QFRAG(3);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int i = 0; i < NPS; ++i)
 #pragma unroll
-        for (int j = 0; j < NPS * 4; ++j) {
-            const int ps = j < 24 ? (j >> 2) : 6 + (j & 1), qs = j < 24 ? (j & 3) : ((j - 24) >> 1);
-            if (j == 24) {
-                // every fragment read of this block has been issued (the last at MFMA 20): once they
-                // have returned, and this wavefront's copies of block kb+1 with them, meet the others
-                asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)"
-                             : "+v"(fq_nxt[0]), "+v"(fq_nxt[1]), "+v"(fq_nxt[2]), "+v"(fq_nxt[3]), "+s"(fpb_nxt) : : "memory");
-                __syncthreads();
-                __builtin_amdgcn_sched_barrier(0);
+            for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+        for (int64_t kb = 0; kb < KB; ++kb) {
+            if (kb == 1) {
+                if (n_valid) {
+                    asm volatile("" : "+s"(ne));      // the load above has been waited for in block 0
+                    n_rows = ne < 0 ? 0 : BQ;
+                    const int e = ne < 0 ? 0 : ne;
+                    n_ptile = a.p + ((int64_t)e * a.Prows + np * 256) * a.red;
+                    n_qtile = a.q + nq * BQ * a.red;
+                    n_spb = a.sp + ((int64_t)e * PB + np * 2 + wp) * KB;
+                    n_sq0 = SQL == 0 ? a.sq + (nq * BQ + wq * 64) * KB : a.sq + nq * BQ + wq * 64;
+                } else {
+                    // past the last tile the copies and scale loads re-read this tile's first blocks:
+                    // the same instruction count in every block keeps the vmcnt arithmetic fixed
+                    n_ptile = c_ptile; n_qtile = c_qtile; n_spb = c_spb; n_sq0 = c_sq0; n_rows = 0;
+                }
             }
-            d[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps % 4], qf[qs], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+            float fq_cur[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) fq_cur[t] = fq_nxt[t] * fpb_nxt;
+            const int nxt1 = cur == 2 ? 0 : cur + 1;         // stage of the next block
+            const int nxt2 = cur >= 1 ? cur - 1 : cur + 2;   // stage the previous block used
+            // scales of the next block, copies of the block after it: this tile's, or the next tile's
+            const bool in1 = kb + 1 < KB, in2 = kb + 2 < KB;
+            const float* s_sq = in1 ? c_sq0 + (kb + 1) * sq_k : n_sq0;
+            const float* s_sp = in1 ? c_spb + (kb + 1) : n_spb;
+            const uint8_t* cp_p = in2 ? c_ptile + (kb + 2) * 128 : n_ptile + (kb + 2 - KB) * 128;
+            const uint8_t* cp_q = in2 ? c_qtile + (kb + 2) * 128 : n_qtile + (kb + 2 - KB) * 128;
+            PF8_LOAD_S(s_sq, s_sp)
+            const uint8_t* pbase = lds + cur * STAGE;
+            const uint8_t* nbase = lds + nxt1 * STAGE;
+            f32x4 d[3];
+            qf[3] = PF8_QFRAG(3);
             __builtin_amdgcn_sched_barrier(0);
-            if (j < 24 && qs == 0 && ps + 2 < NPS) {
-                pf[(ps + 2) % 4] = PF8_PFRAG(ps + 2);
+#pragma unroll
+            for (int j = 0; j < NPS * 4; ++j) {
+                const int ps = j < 24 ? (j >> 2) : 6 + (j & 1), qs = j < 24 ? (j & 3) : ((j - 24) >> 1);
+                if (j == 24) {
+                    // every fragment read of this block has been issued (the last at MFMA 20): once
+                    // they have returned, and this wavefront's copies of the next block with them,
+                    // meet the other wavefronts
+                    asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)"
+                                 : "+v"(fq_nxt[0]), "+v"(fq_nxt[1]), "+v"(fq_nxt[2]), "+v"(fq_nxt[3]), "+s"(fpb_nxt), "+s"(ne) : : "memory");
+                    __syncthreads();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                d[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps % 4], qf[qs], (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
+                if (j < 24 && qs == 0 && ps + 2 < NPS) {
+                    pf[(ps + 2) % 4] = PF8_PFRAG(ps + 2);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if ((j & 1) == 1 && j < 24) {
+                    // no branch here: control flow inside the MFMA sequence lets the compiler sink
+                    // the scale-FMAs out of it
+                    PF8_COPY(j >> 1, cp_p, cp_q, nxt2);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // the next block's first fragments, from the stage that has just been declared landed
+                if (j == 24) { pf[0] = ld_frag_lds(nbase + fp_ofs[0], nbase + fp_ofs[1]); __builtin_amdgcn_sched_barrier(0); }
+                if (j == 25) { qf[0] = ld_frag_lds(nbase + fq_ofs[0], nbase + fq_ofs[1]); __builtin_amdgcn_sched_barrier(0); }
+                if (j == 26) { pf[1] = ld_frag_lds(nbase + fp_ofs[0] + 2048, nbase + fp_ofs[1] + 2048); __builtin_amdgcn_sched_barrier(0); }
+                if (j == 27) { qf[1] = ld_frag_lds(nbase + fq_ofs[0] + 2048, nbase + fq_ofs[1] + 2048); __builtin_amdgcn_sched_barrier(0); }
+                if (j == 29) { qf[2] = ld_frag_lds(nbase + fq_ofs[0] + 4096, nbase + fq_ofs[1] + 4096); __builtin_amdgcn_sched_barrier(0); }
+                if (j >= 2) {
+                    const int jj = j - 2;
+                    const int pj = jj < 24 ? (jj >> 2) : 6 + (jj & 1), qj = jj < 24 ? (jj & 3) : ((jj - 24) >> 1);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        acc[pj][qj][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[qj], acc[pj][qj][r]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
-            if ((j & 1) == 1 && j < 24) {
-                // no branch here: control flow inside the MFMA sequence lets the compiler sink the
-                // scale-FMAs out of it
-                PF8_COPY(j >> 1, kb2, nxt2);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // next block's first fragments, from the stage that has just been declared landed
-            if (j == 24) { pf[0] = ld_frag_lds(nbase + fp_ofs[0], nbase + fp_ofs[1]); __builtin_amdgcn_sched_barrier(0); }
-            if (j == 25) { qf[0] = ld_frag_lds(nbase + fq_ofs[0], nbase + fq_ofs[1]); __builtin_amdgcn_sched_barrier(0); }
-            if (j == 26) { pf[1] = ld_frag_lds(nbase + fp_ofs[0] + 2048, nbase + fp_ofs[1] + 2048); __builtin_amdgcn_sched_barrier(0); }
-            if (j == 27) { qf[1] = ld_frag_lds(nbase + fq_ofs[0] + 2048, nbase + fq_ofs[1] + 2048); __builtin_amdgcn_sched_barrier(0); }
-            if (j == 29) { qf[2] = ld_frag_lds(nbase + fq_ofs[0] + 4096, nbase + fq_ofs[1] + 4096); __builtin_amdgcn_sched_barrier(0); }
-            if (j >= 2) {
-                const int jj = j - 2;
-                const int pj = jj < 24 ? (jj >> 2) : 6 + (jj & 1), qj = jj < 24 ? (jj & 3) : ((jj - 24) >> 1);
+#pragma unroll
+            for (int jj = NPS * 4 - 2; jj < NPS * 4; ++jj) {
+                const int pj = 6 + (jj & 1), qj = (jj - 24) >> 1;
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
                     acc[pj][qj][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[qj], acc[pj][qj][r]);
-                __builtin_amdgcn_sched_barrier(0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            cur = nxt1;
+        }
+
+        // ---- epilogue of this tile.  Its last block's stage is free: every wavefront passed that
+        // block's barrier with its fragment reads returned, and no copy targets the stage before the
+        // next block starts.  Each wavefront stages 32 of its 64 rows at a time in a private slice
+        // (LDS operations of one wavefront execute in order) and stores whole 256-byte rows.
+        {
+            constexpr int EP_LD = 272;                   // 128 bf16 per row + 16 B pad
+            const int last = cur == 0 ? 2 : cur - 1;
+            uint8_t* ep = lds + last * STAGE + wave * (32 * EP_LD);
+            uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
+            const int er = lane >> 4, ec = lane & 15;
+            const int64_t col = cp * 256 + wp * 128 + ec * 8;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int qh = 0; qh < 2; ++qh) {
+                    const int qs = half * 2 + qh;
+#pragma unroll
+                    for (int ps = 0; ps < NPS; ++ps) {
+                        uint2 o;
+                        o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
+                        o.y = pack_bf16(acc[ps][qs][2], acc[ps][qs][3]);
+                        *reinterpret_cast<uint2*>(ep + (qh * 16 + li) * EP_LD + (ps * 16 + 4 * kg) * 2) = o;
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int rl = er + 4 * i;                        // row inside the 32-row slice
+                    const int64_t row = cq * BQ + wq * 64 + half * 32 + rl;
+                    const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
+                    if (c_rows) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
+                }
             }
         }
-#pragma unroll
-        for (int jj = NPS * 4 - 2; jj < NPS * 4; ++jj) {
-            const int pj = 6 + (jj & 1), qj = (jj - 24) >> 1;
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                acc[pj][qj][r] = __builtin_fmaf(d[jj % 3][r], fq_cur[qj], acc[pj][qj][r]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        cur = nxt1;
+        if (!n_valid) break;
+        __syncthreads();   // the staging slices are dead before any copy of the next block lands there
+        cq = nq; cp = np; c_rows = n_rows;
+        c_ptile = n_ptile; c_qtile = n_qtile; c_spb = n_spb; c_sq0 = n_sq0;
     }
-    __builtin_amdgcn_s_waitcnt(0);
-
-    // ---- epilogue: bf16 through LDS so that every store instruction writes whole 256-byte rows ----
-    constexpr int EP_LD = 272;                   // 128 bf16 per row + 16 B pad
-    __syncthreads();                             // everyone is done reading fragments, all copies landed
-    uint8_t* ep = lds + wave * (64 * EP_LD);
-#pragma unroll
-    for (int qs = 0; qs < 4; ++qs)
-#pragma unroll
-        for (int ps = 0; ps < NPS; ++ps) {
-            uint2 o;
-            o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
-            o.y = pack_bf16(acc[ps][qs][2], acc[ps][qs][3]);
-            *reinterpret_cast<uint2*>(ep + (qs * 16 + li) * EP_LD + (ps * 16 + 4 * kg) * 2) = o;
-        }
-    const int er = lane >> 4, ec = lane & 15;
-    const int64_t col = p0 + wp * 128 + ec * 8;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int rt = wq * 64 + er + 4 * i;     // row inside the tile
-        const int64_t row = q0 + rt;
-        const uint4 v = *reinterpret_cast<const uint4*>(ep + (er + 4 * i) * EP_LD + ec * 16);
-        if (rt >= row_hi) continue;
-        *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
-    }
+    __builtin_amdgcn_s_waitcnt(0);   // the copies issued past the end must land before the LDS is released
 #undef PF8_COPY
 #undef PF8_LOAD_S
 #undef PF8_PFRAG
@@ -714,20 +761,27 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         const int64_t T128 = ((a.Prows + 255) / 256) * ((a.Qrows + 127) / 128);
         // the grid is padded to a multiple of 8 so that every XCD gets an equal run of tiles
         dim3 g128((unsigned)(((T128 + 7) / 8) * 8), grid.y);
-        // The deep-pipeline kernel (one workgroup per compute unit, copies two blocks ahead) wins
-        // where the weight stream dominates: long reductions with at most a few tiles per compute
-        // unit.  Measured on MI355X: +15% on the 32-expert K=7168 grouped GEMM, +20% on dense
-        // M <= 2048, K=7168, -5% on dense M = 8192; -10% at K=2048, where its two-block prologue is
-        // an eighth of the loop.
+        // The persistent deep-pipeline kernel wins where the operand stream, not the matrix pipe, sets
+        // the pace.  Measured on MI355X against the two-workgroup kernel: +14..24% when all tiles
+        // fit one round of compute units (dense M <= 2048 at N = 4096), +15% / +7% on the up+gate /
+        // down GEMMs of 32 experts with a skewed 8192-row load, parity (0.92..1.06) elsewhere, where
+        // its static tile assignment loses what the deeper pipeline gains.
         // PF8_FWD_KERNEL=deep|wide overrides the choice (benchmarking).
         static const char* force = getenv("PF8_FWD_KERNEL");
-        const bool aligned = a.Prows % 256 == 0 && a.Qrows % 128 == 0;
-        bool deep = aligned && a.red >= 4096 && T128 <= (a.group == GROUP_NONE ? 2 : 8) * (int64_t)pf8_effective_cus();
-        if (force && force[0] == 'd') deep = aligned && a.red >= 128;
+        const bool aligned = a.Prows % 256 == 0 && a.Qrows % 128 == 0 && a.red >= 384 && a.group != GROUP_MASKED;
+        const int64_t cus = pf8_effective_cus();
+        bool deep = aligned && (T128 <= cus || (a.group == GROUP_CONTIG && a.red >= 2048 && T128 <= 10 * cus));
+        if (force && force[0] == 'd') deep = aligned;
         if (force && force[0] == 'w') deep = false;
         if (deep) {
-            if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0>), g128, dim3(256), 147456, st, a);
-            else hipLaunchKernelGGL((k_gemm_fwd_deep<1>), g128, dim3(256), 147456, st, a);
+            // persistent: one workgroup per compute unit (or per tile of an XCD's run, if fewer)
+            const int64_t per_xcd = (T128 + 7) / 8;
+            int64_t w = pf8_effective_cus() / 8;
+            if (w < 1) w = 1;
+            if (w > per_xcd) w = per_xcd;
+            dim3 gd((unsigned)(8 * w), 1);
+            if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0>), gd, dim3(256), 147456, st, a);
+            else hipLaunchKernelGGL((k_gemm_fwd_deep<1>), gd, dim3(256), 147456, st, a);
         } else if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd128<0>), g128, dim3(256), 81920, st, a);
         else hipLaunchKernelGGL((k_gemm_fwd128<1>), g128, dim3(256), 81920, st, a);
     } else {
