@@ -740,14 +740,28 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
             *reinterpret_cast<f32x4*>(ep + (qs * 16 + li) * EP_LD + (ps * 16 + 4 * kg) * 4) = acc[ps][qs];
     const int er = lane >> 4, ec = lane & 15;
     const int64_t col = p0 + wp * 64 + ec * 4;
+    const bool col_ok = col + 4 <= a.Prows;
+    const int64_t col_c = col_ok ? col : a.Prows - 4;
+    // read-modify-write: all 16 loads of the old gradient rows are in flight before the first add
+    // (one load-add-store round trip per row would cost sixteen memory latencies per tile)
+    f32x4 old[16];
+    if (a.accumulate) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            int64_t row = q0 + wq * 64 + er + 4 * i;
+            if (row > a.Qrows - 1) row = a.Qrows - 1;
+            old[i] = *reinterpret_cast<const f32x4*>(outb + (row * a.ldo + col_c) * 4);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) old[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int64_t row = q0 + wq * 64 + er + 4 * i;
-        f32x4 v = *reinterpret_cast<const f32x4*>(ep + (er + 4 * i) * EP_LD + ec * 16);
-        if (row >= a.Qrows || col + 4 > a.Prows) continue;
-        f32x4* dst = reinterpret_cast<f32x4*>(outb + (row * a.ldo + col) * 4);
-        if (a.accumulate) { const f32x4 old = *dst; v = (f32x4){old.x + v.x, old.y + v.y, old.z + v.z, old.w + v.w}; }
-        *dst = v;
+        const f32x4 v = *reinterpret_cast<const f32x4*>(ep + (er + 4 * i) * EP_LD + ec * 16);
+        const f32x4 o = (f32x4){old[i].x + v.x, old[i].y + v.y, old[i].z + v.z, old[i].w + v.w};
+        if (row < a.Qrows && col_ok) *reinterpret_cast<f32x4*>(outb + (row * a.ldo + col) * 4) = o;
     }
 #undef PF8_DMA
 #undef PF8_LOAD_S
