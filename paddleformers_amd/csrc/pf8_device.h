@@ -130,20 +130,76 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 // Quantise 8 values of one tile: bytes == e4m3_rne(v / s) with v / s the correctly rounded fp32
 // quotient.  Fast path: the quotient is bracketed by v*r_lo and v*r_hi (the reciprocal is good to
 // 1 ulp, the nudges are 2^-20, so the bracket holds with a wide margin); rounding is monotone, so
-// when both ends convert to the same e4m3 codes those are the codes of the exact quotient.  Only
-// when an end pair differs (a rounding boundary lies inside the 2^-19-wide bracket, about 3e-5 per
-// element) does the lane redo its 8 elements with the IEEE division.
+// where both ends convert to the same e4m3 code that is the code of the exact quotient.  Where they
+// differ a rounding boundary lies inside the 2^-19-wide bracket and that ELEMENT is redone with the
+// IEEE division.  This is not rare: s = amax/448 carries an fp32 rounding error, so every element
+// for which 448 v / amax is an exact e4m3 tie in real arithmetic (bf16 inputs make these common,
+// about one element in a thousand) sits 2^-24 from a boundary.  Most wavefronts therefore visit
+// the fallback for one or two elements, and it is written to cost one division, not eight.
+__device__ __forceinline__ uint32_t nonzero_bytes(uint32_t d) {   // 0x80 in every byte of d that is not zero
+    return (((d & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | d) & 0x80808080u;
+}
+__device__ __forceinline__ void quant8_fix(const float (&v)[8], float s, uint2& lo, const uint2 hi) {
+    const uint32_t dx = lo.x ^ hi.x, dy = lo.y ^ hi.y;
+    if (__builtin_expect((dx | dy) != 0u, 0)) {
+        const uint32_t zx = nonzero_bytes(dx), zy = nonzero_bytes(dy);
+        if (__builtin_popcount(zx) + __builtin_popcount(zy) == 1) {
+            // the usual case, one element: pick it without branching on its index
+            const int idx = zx ? (__builtin_ctz(zx) >> 3) : 4 + (__builtin_ctz(zy) >> 3);
+            const float a = (idx & 1) ? v[1] : v[0], b = (idx & 1) ? v[3] : v[2];
+            const float c = (idx & 1) ? v[5] : v[4], d = (idx & 1) ? v[7] : v[6];
+            const float e = (idx & 2) ? b : a, f = (idx & 2) ? d : c;
+            const float qv = ((idx & 4) ? f : e) / s;
+            const uint32_t code = cvt_e4m3_lo(qv, qv, 0u) & 0xFFu;
+            const int sh = 8 * (idx & 3);
+            const uint32_t keep = ~(0xFFu << sh), put = code << sh;
+            if (idx & 4) lo.y = (lo.y & keep) | put;
+            else lo.x = (lo.x & keep) | put;
+        } else {
+            // a tile whose amax makes exact ties common (e.g. amax = 448 * 2^k: one value in eight)
+            lo.x = pack4_e4m3(v[0] / s, v[1] / s, v[2] / s, v[3] / s);
+            lo.y = pack4_e4m3(v[4] / s, v[5] / s, v[6] / s, v[7] / s);
+        }
+    }
+}
 __device__ __forceinline__ uint2 quant8(const float (&v)[8], const TileScale& t) {
     uint2 lo, hi;
-    lo.x = pack4_e4m3(v[0] * t.r_lo, v[1] * t.r_lo, v[2] * t.r_lo, v[3] * t.r_lo);
-    lo.y = pack4_e4m3(v[4] * t.r_lo, v[5] * t.r_lo, v[6] * t.r_lo, v[7] * t.r_lo);
-    hi.x = pack4_e4m3(v[0] * t.r_hi, v[1] * t.r_hi, v[2] * t.r_hi, v[3] * t.r_hi);
-    hi.y = pack4_e4m3(v[4] * t.r_hi, v[5] * t.r_hi, v[6] * t.r_hi, v[7] * t.r_hi);
-    const bool redo = t.slow | (lo.x != hi.x) | (lo.y != hi.y);
-    if (__builtin_expect(redo, 0)) {
-        lo.x = pack4_e4m3(v[0] / t.s, v[1] / t.s, v[2] / t.s, v[3] / t.s);
-        lo.y = pack4_e4m3(v[4] / t.s, v[5] / t.s, v[6] / t.s, v[7] / t.s);
-    }
+    const float r_lo = t.slow ? 0.0f : t.r_lo, r_hi = t.slow ? __builtin_inff() : t.r_hi;   // slow: every element differs
+    lo.x = pack4_e4m3(v[0] * r_lo, v[1] * r_lo, v[2] * r_lo, v[3] * r_lo);
+    lo.y = pack4_e4m3(v[4] * r_lo, v[5] * r_lo, v[6] * r_lo, v[7] * r_lo);
+    hi.x = pack4_e4m3(v[0] * r_hi, v[1] * r_hi, v[2] * r_hi, v[3] * r_hi);
+    hi.y = pack4_e4m3(v[4] * r_hi, v[5] * r_hi, v[6] * r_hi, v[7] * r_hi);
+    quant8_fix(v, t.s, lo, hi);
+    return lo;
+}
+
+// ---- quantizers that hold several tiles per lane: scales for up to four tiles in one pass ----
+// value of lane Q of every quad, for all four lanes of the quad (folds into the consuming VALU op)
+template <int Q>
+__device__ __forceinline__ float quad_bcast(float v) {
+    return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v), Q * 0x55, 0xF, 0xF, false));
+}
+// Reciprocal pair of a scale; a scale too small for a finite reciprocal gets (0, inf), which makes
+// the two conversions of any element disagree and sends the tile down the division path.
+__device__ __forceinline__ void scale_recips(float s, float& r_lo, float& r_hi) {
+    const float r = __builtin_amdgcn_rcpf(s);
+    const bool ok = s >= 1.0e-30f;
+    r_lo = ok ? r * 0.99999904632568359375f : 0.0f;          // 1 - 2^-20
+    r_hi = ok ? r * 1.00000095367431640625f : __builtin_inff();   // 1 + 2^-20
+}
+__device__ __forceinline__ float scale_of(uint32_t amax_bits, bool pow2) {
+    float s = u2f(amax_bits) / 448.0f;
+    if (pow2) s = u2f((f2u(s) + 0x007FFFFFu) & 0x7F800000u);
+    return amax_bits == 0u ? 1.0f : s;
+}
+// 8 values against a reciprocal pair; elements whose two conversions differ are redone by division
+__device__ __forceinline__ uint2 quant8_r(const float (&v)[8], float r_lo, float r_hi, float s) {
+    uint2 lo, hi;
+    lo.x = pack4_e4m3(v[0] * r_lo, v[1] * r_lo, v[2] * r_lo, v[3] * r_lo);
+    lo.y = pack4_e4m3(v[4] * r_lo, v[5] * r_lo, v[6] * r_lo, v[7] * r_lo);
+    hi.x = pack4_e4m3(v[0] * r_hi, v[1] * r_hi, v[2] * r_hi, v[3] * r_hi);
+    hi.y = pack4_e4m3(v[4] * r_hi, v[5] * r_hi, v[6] * r_hi, v[7] * r_hi);
+    quant8_fix(v, s, lo, hi);
     return lo;
 }
 

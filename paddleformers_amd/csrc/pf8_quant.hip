@@ -16,39 +16,60 @@ namespace pf8 {
 // 1x128 quantizer: one wavefront per row, four tiles per load instruction
 // ---------------------------------------------------------------------------------------------
 
-// grid.x = column chunks of 4*U tiles, grid.y = groups of 4 rows; every lane issues its U 16-byte
-// loads before any arithmetic, so a wavefront is one load phase, one compute phase, one store phase
+// grid.x = column chunks of 16 tiles, grid.y = groups of 4 rows; every lane issues its four 16-byte
+// loads before any arithmetic, so a wavefront is one load phase, one compute phase, one store phase.
+// The kernel is bound by the vector ALU, not by memory (the bracketing quantizer costs about 20
+// ALU cycles per element), so the bookkeeping around it is kept off the vector pipe:
+//   * the row is wave-uniform: every address is a scalar base plus one 32-bit lane offset;
+//   * the scales of a lane group's four tiles are computed in ONE pass (lane q of every quad takes
+//     tile q; the IEEE divide and the reciprocal run once, not four times) and come back through
+//     quad-broadcast DPP operands.
 template <int LAYOUT, int U>
 __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict__ x, int64_t M, int64_t m0, int KB, int64_t ldx,
                                                      uint8_t* __restrict__ q, float* __restrict__ s, int pow2) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, l = lane & 15;
+    static_assert(U == 4, "one quad lane per tile");
+    const int lane = threadIdx.x & 63, g = lane >> 4, l = lane & 15;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t r = m0 + (int64_t)blockIdx.y * 4 + wave;   // m0: first row of this launch's slab
     if (r >= M) return;
-    const int kb0 = blockIdx.x * (4 * U);
-    const uint4* xr = reinterpret_cast<const uint4*>(x + r * ldx);
-    uint2* qr = reinterpret_cast<uint2*>(q + r * (int64_t)KB * 128);
-    uint4 w[U];
+    const int kb0 = blockIdx.x * 16;
+    const uint8_t* xr = reinterpret_cast<const uint8_t*>(x + r * ldx);
+    uint8_t* qr = q + r * (int64_t)KB * 128;
+    const uint32_t in_off = (uint32_t)((kb0 + g) * 256 + l * 16);    // tile u adds u * 1024
+    const uint32_t out_off = (uint32_t)((kb0 + g) * 128 + l * 8);    // tile u adds u * 512
+    uint4 w[4];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        int kb = kb0 + 4 * u + g;
+    for (int u = 0; u < 4; ++u) {
         w[u] = make_uint4(0, 0, 0, 0);
-        if (kb < KB) w[u] = ld16(xr + kb * 16 + l);
+        if (kb0 + 4 * u + g < KB) w[u] = ld16(xr + in_off + u * 1024);
     }
+    uint32_t am[4];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        int kb = kb0 + 4 * u + g;
+    for (int u = 0; u < 4; ++u) am[u] = row16_max(amax_bits8(w[u]));
+    const int ql = l & 3;
+    const uint32_t am_sel = ql == 0 ? am[0] : ql == 1 ? am[1] : ql == 2 ? am[2] : am[3];
+    const float sc = scale_of(am_sel, pow2 != 0);       // lane q of a quad: scale of tile q
+    float r_lo, r_hi;
+    scale_recips(sc, r_lo, r_hi);
+    if (l < 4) {
+        const int kb = kb0 + 4 * l + g;
         if (kb < KB) {
-            TileScale t = make_scale(row16_max(amax_bits8(w[u])), pow2 != 0);
-            float v[8];
-            unpack8(w[u], v);
-            uint2 o = quant8(v, t);
-            st8(qr + kb * 16 + l, o);
-            if (l == 0) {
-                if (LAYOUT == 0) s[r * KB + kb] = t.s;
-                else s[(int64_t)kb * M + r] = t.s;
-            }
+            if (LAYOUT == 0) s[r * KB + kb] = sc;
+            else s[(int64_t)kb * M + r] = sc;
         }
     }
+    // cross-lane reads see only active lanes: every broadcast happens while the wavefront is whole
+    uint2 o[4];
+    {
+        float v[8];
+        unpack8(w[0], v); o[0] = quant8_r(v, quad_bcast<0>(r_lo), quad_bcast<0>(r_hi), quad_bcast<0>(sc));
+        unpack8(w[1], v); o[1] = quant8_r(v, quad_bcast<1>(r_lo), quad_bcast<1>(r_hi), quad_bcast<1>(sc));
+        unpack8(w[2], v); o[2] = quant8_r(v, quad_bcast<2>(r_lo), quad_bcast<2>(r_hi), quad_bcast<2>(sc));
+        unpack8(w[3], v); o[3] = quant8_r(v, quad_bcast<3>(r_lo), quad_bcast<3>(r_hi), quad_bcast<3>(sc));
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (kb0 + 4 * u + g < KB) st8(qr + out_off + u * 512, o[u]);
 }
 
 // ---------------------------------------------------------------------------------------------
