@@ -180,6 +180,16 @@ def bench_other_gemms(iters=10, warmup=3):
     g = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
     ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True), [()], 5, 2)
     out["grouped_wgrad_config5_dw1"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms}
+    del a_t, sa_t, b_t, sb_t, g
+    torch.cuda.empty_cache()
+    # per-step weight requantization of config 3's up+gate experts: both orientations from one read
+    Ew, Hw, Iw = 32, 7168, 2048
+    ws = [(torch.randn((Hw, 2 * Iw), device="cuda") * 0.02).to(torch.bfloat16) for _ in range(Ew)]
+    ms = time_kernel(lambda: F8.fused_stack_quant_both(ws), [()], 5, 2)
+    out["stack_quant_both_config3_w1"] = {"bytes": Ew * Hw * 2 * Iw * 4 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4, "ms": ms}
+    ms = time_kernel(lambda: (F8.fused_stack_transpose_quant(ws, False), F8.fused_stack_transpose_quant(ws, True)), [()], 5, 2)
+    out["stack_quant_two_calls_config3_w1"] = {"bytes": Ew * Hw * 2 * Iw * 6 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4, "ms": ms}
+    del ws
     for v in out.values():
         if "flop" in v:
             v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)

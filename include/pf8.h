@@ -73,6 +73,14 @@ int pf8_quant_transpose(const uint16_t* x, int64_t M, int64_t K, uint8_t* q, flo
 int pf8_stack_transpose_quant(const uint16_t* const* w_list, int E, int64_t R, int64_t C,
                               int transpose, uint8_t* q, float* s, int pow2, pf8_stream_t stream);
 
+/* Both orientations of fused_stack_transpose_quant from ONE read of the weights: what
+ * DeepseekV2MoE.fp8_quant_weight(quant_transpose=None) asks for with two calls per weight list
+ * (cli/train/deepseek_v3_pretrain/modeling.py:506-567, driven once per optimizer step by
+ * FP8QuantWeightCallback, trainer/trainer_callback.py:727-765).  q [E*R, C] + s [E*R/128, C/128]
+ * and q_t [E*C, R] + s_t [E*C/128, R/128]; byte-identical to the two separate calls. */
+int pf8_stack_quant_both(const uint16_t* const* w_list, int E, int64_t R, int64_t C, uint8_t* q,
+                         float* s, uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream);
+
 /* fused_weighted_swiglu_act_quant(o1, probs, using_pow2_scaling) -- transformers/fp8_utils.py:981-987;
  * un-fused definition ernie token_dispatcher/fp8_utils.py:996-1004.  o1 bf16 [M,2I] (gate first),
  * probs fp32 [M] or NULL -> q [M,I], s per scale_layout.  o2 (bf16 [M,I]) optionally receives the

@@ -631,6 +631,29 @@ extern "C" int pf8_stack_transpose_quant(const uint16_t* const* w_list, int E, i
     return PF8_OK;
 }
 
+extern "C" int pf8_stack_quant_both(const uint16_t* const* w_list, int E, int64_t R, int64_t C, uint8_t* q, float* s,
+                                    uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(E >= 0 && R >= 0 && C >= 0, "negative shape");
+    PF8_REQUIRE(R % 128 == 0 && C % 128 == 0, "R and C must be multiples of 128");
+    if (E == 0 || R == 0 || C == 0) return PF8_OK;
+    PF8_REQUIRE(w_list && q && s && q_t && s_t, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(q) && PF8_ALIGNED16(q_t), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(R / 128 <= 65535, "shape too large");
+    for (int e = 0; e < E; ++e) PF8_REQUIRE(w_list[e] && PF8_ALIGNED16(w_list[e]), "null or misaligned weight pointer");
+    const int64_t per_q = R * C, per_s = (R / 128) * (C / 128);
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        const int n = E - e0 < 256 ? E - e0 : 256;
+        StackArgs a = {};
+        for (int i = 0; i < n; ++i) a.w[i] = w_list[e0 + i];
+        dim3 grid((unsigned)(C / 128), (unsigned)(R / 128), (unsigned)n), block(256);
+        hipLaunchKernelGGL(k_quant_128x128<true>, grid, block, 0, (hipStream_t)stream, nullptr, a, R, C,
+                           q + (int64_t)e0 * per_q, s + (int64_t)e0 * per_s, q_t + (int64_t)e0 * per_q, s_t + (int64_t)e0 * per_s, pow2);
+        int rc = pf8_check_launch(__func__);
+        if (rc) return rc;
+    }
+    return PF8_OK;
+}
+
 extern "C" int pf8_quant_transpose(const uint16_t* x, int64_t M, int64_t K, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
                                    int scale_layout, int pow2, pf8_stream_t stream) {
     PF8_REQUIRE(M >= 0 && K >= 0, "negative shape");

@@ -131,6 +131,45 @@ def cache_fp8_weight(weight, quant_transpose=None):
         raise ValueError("quant_transpose must be either True, False or None.")
 
 
+def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_transpose=None):
+    """DeepseekV2MoE.fp8_quant_weight (cli/train/deepseek_v3_pretrain/modeling.py:506-567), the body
+    FP8QuantWeightCallback.on_step_begin runs once per optimizer step: attach the stacked FP8 copies
+    of the expert weights to the first weight of each list (batch mode) or to every weight.
+
+    quant_transpose None caches both orientations; here they come from one read of the weights
+    (`fused_stack_quant_both`) instead of two passes.  Weights that already carry a cache are left
+    alone, as in the reference."""
+
+    def quantize_weights(weight_list, weight_obj=None):
+        if weight_obj is None:
+            weight_obj = weight_list[0]
+        if hasattr(weight_obj, "fp8_weight_stacked") or hasattr(weight_obj, "fp8_weight_stacked_transpose"):
+            return
+        if quant_transpose is None:
+            q, s, qt, st = F8.fused_stack_quant_both(weight_list)
+            weight_obj.fp8_weight_stacked, weight_obj.fp8_scale_stacked = q, s
+            weight_obj.fp8_weight_stacked_transpose, weight_obj.fp8_scale_stacked_transpose = qt, st
+        elif quant_transpose is False:
+            weight_obj.fp8_weight_stacked, weight_obj.fp8_scale_stacked = F8.fused_stack_transpose_quant(weight_list, transpose=False)
+        elif quant_transpose is True:
+            weight_obj.fp8_weight_stacked_transpose, weight_obj.fp8_scale_stacked_transpose = F8.fused_stack_transpose_quant(
+                weight_list, transpose=True)
+        else:
+            raise ValueError("Invalid value for `quant_transpose`.")
+
+    w1s = [w for w in expert_w1_list if w is not None]
+    w2s = [w for w in expert_w2_list if w is not None]
+    if batch_mode:
+        if w1s:
+            quantize_weights(w1s, w1s[0])
+        if w2s:
+            quantize_weights(w2s, w2s[0])
+    else:
+        for w1, w2 in zip(w1s, w2s):
+            quantize_weights([w1])
+            quantize_weights([w2])
+
+
 def split_group_gemm(x_fp8, x_scale, w_fp8, w_scale, tokens_per_expert, gemm_out):
     """fp8_utils.py:853-870: the grouped GEMM as a loop of dense GEMMs, empty experts skipped."""
     start_idx = 0

@@ -160,6 +160,35 @@ def fused_stack_transpose_quant(weight_list: Sequence[torch.Tensor], transpose: 
     return q, s
 
 
+def fused_stack_quant_both(weight_list: Sequence[torch.Tensor], using_pow2_scale: bool = False):
+    """Both orientations of `fused_stack_transpose_quant` from one read of the weights.
+
+    Returns (q, s, q_t, s_t) equal to `fused_stack_transpose_quant(ws, False)` +
+    `fused_stack_transpose_quant(ws, True)`: the pair DeepseekV2MoE.fp8_quant_weight builds with two
+    calls when quant_transpose is None (cli/train/deepseek_v3_pretrain/modeling.py:521-534).
+    """
+    if len(weight_list) == 0:
+        raise ValueError("weight_list is empty")
+    R, Cc = weight_list[0].shape
+    ws = []
+    for w in weight_list:
+        _dev(w, "weight")
+        if w.dtype != torch.bfloat16 or tuple(w.shape) != (R, Cc):
+            raise ValueError("all weights must be bfloat16 with the same 2-D shape")
+        ws.append(w if w.is_contiguous() else w.contiguous())
+    if R % 128 != 0 or Cc % 128 != 0:
+        raise ValueError(f"weight dimensions must be divisible by 128, got [{R}, {Cc}]")
+    E = len(ws)
+    dev = ws[0].device
+    q = torch.empty((E * R, Cc), dtype=FP8, device=dev)
+    s = torch.empty((E * R // 128, Cc // 128), dtype=torch.float32, device=dev)
+    qt = torch.empty((E * Cc, R), dtype=FP8, device=dev)
+    st = torch.empty((E * Cc // 128, R // 128), dtype=torch.float32, device=dev)
+    ptrs = (C.c_void_p * E)(*[w.data_ptr() for w in ws])
+    _lib.call("pf8_stack_quant_both", ptrs, E, R, Cc, _p(q), _p(s), _p(qt), _p(st), int(bool(using_pow2_scale)), _stream())
+    return q, s, qt, st
+
+
 # ---------------------------------------------------------------------------------------------
 # fused_weighted_swiglu_act_quant
 # ---------------------------------------------------------------------------------------------
