@@ -190,6 +190,16 @@ def bench_other_gemms(iters=10, warmup=3):
     ms = time_kernel(lambda: (F8.fused_stack_transpose_quant(ws, False), F8.fused_stack_transpose_quant(ws, True)), [()], 5, 2)
     out["stack_quant_two_calls_config3_w1"] = {"bytes": Ew * Hw * 2 * Iw * 6 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4, "ms": ms}
     del ws
+    torch.cuda.empty_cache()
+    # checkpoint load: block-FP8 [32, 4096, 7168] (128x128 blocks, UE8M0 scales) -> bf16
+    from paddleformers_amd import checkpoint_dequant as CD
+
+    dq = CD.get_checkpoint_dequantizer("fp8_block").configure_formats("e4m3", "ue8m0").configure_geometry((1, 2), (128, 128))
+    qw = torch.randint(0, 120, (Ew, 2 * Iw, Hw), dtype=torch.uint8, device="cuda")
+    sc = torch.randint(110, 130, (Ew, 2 * Iw // 128, Hw // 128), dtype=torch.uint8, device="cuda")
+    ms = time_kernel(lambda: dq.dequantize({"qweight": qw, "scale": sc}, torch.bfloat16), [()], 5, 2)
+    out["block_dequant_config3_w1"] = {"bytes": Ew * 2 * Iw * Hw * 3 + sc.numel(), "ms": ms}
+    del qw, sc
     for v in out.values():
         if "flop" in v:
             v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)

@@ -110,6 +110,15 @@ int pf8_act_dequant(const uint8_t* q, const float* s, int scale_layout, int64_t 
 int pf8_weight_dequant(const uint8_t* q, const float* s, int64_t R, int64_t C, uint16_t* out,
                        pf8_stream_t stream);
 
+/* FP8BlockCheckpointDequantizer.dequantize -- quantization/checkpoint_dequant.py:277-292 with
+ * _decode_e4m3 / _decode_ue8m0 / _expand_scale_grid (:76-176): out = cast(e4m3(q) * scale), q raw
+ * e4m3 bytes viewed as [B, R, C], scale [B, ceil(R/block_r), ceil(C/block_c)] (an axis that is not
+ * blocked has block size 1), partial trailing blocks cropped.  scale_format 0 = fp32, 1 = UE8M0
+ * exponent bytes (2^(e-127), 255 -> inf), 2 = bf16, 3 = fp16.  out is bf16 (out_f32 = 0) or fp32. */
+int pf8_block_dequant(const uint8_t* q, const void* scale, int scale_format, int64_t B, int64_t R,
+                      int64_t C, int64_t block_r, int64_t block_c, void* out, int out_f32,
+                      pf8_stream_t stream);
+
 /* fused_swiglu_weighted_bwd(o1, do2_s, probs) -- transformers/fp8_utils.py:1049-1052; un-fused
  * definition ernie token_dispatcher/fp8_utils.py:1088-1092.  -> do1 bf16 [M,2I], probs_grad fp32 [M],
  * o2_s bf16 [M,I]. */

@@ -331,3 +331,50 @@ def grouped_gemm_nt_masked(a, sa, b, sb, masked_m, out=None):
     out = np.zeros((E, Mmax, N), np.uint16) if out is None else out
     lib().pf8o_grouped_gemm_nt_masked(_p(a), _p(sa), _p(b), _p(sb), int(E), I64(Mmax), I64(N), I64(K), _p(masked_m), _p(out))
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# block-FP8 checkpoint dequantization (numpy restatement; pinned by the reference's own known-answer
+# tests, tests/coverage_test/quantization/test_coverage_hf_checkpoint_dequant.py:210-289)
+# ---------------------------------------------------------------------------------------------
+
+
+def ue8m0_table() -> np.ndarray:
+    """quantization/checkpoint_dequant.py:93: 2^(code-127), code 255 -> inf."""
+    t = np.array([2.0 ** (e - 127) for e in range(256)], dtype=np.float64)
+    t[255] = np.inf
+    return t.astype(np.float32)
+
+
+def decode_scales(scale: np.ndarray, scale_format: str) -> np.ndarray:
+    """checkpoint_dequant.py:177-183 (_decode_scales): UE8M0 codes through the table (int8 storage is
+    reinterpreted as unsigned, :100-108), float formats widened to fp32; bf16 comes as uint16 bits."""
+    fmt = scale_format.strip().lower()
+    if fmt in ("ue8m0", "e8m0", "float8_e8m0"):
+        assert scale.dtype in (np.uint8, np.int8)
+        return ue8m0_table()[scale.view(np.uint8)]
+    if fmt in ("bf16", "bfloat16"):
+        return bf16_bits_to_f32(scale)
+    return scale.astype(np.float32)
+
+
+def block_dequant(q: np.ndarray, scale: np.ndarray, scale_format: str, block_axes, block_shape, out: str = "f32") -> np.ndarray:
+    """FP8BlockCheckpointDequantizer.dequantize (checkpoint_dequant.py:277-292): decode the e4m3 codes
+    (:76-90, :111-118), expand the scale grid by repeating it block_size times along every blocked
+    axis and cropping to the weight's shape (:145-176), multiply in fp32, cast.  Returns fp32 values
+    or bf16 bit patterns."""
+    assert q.dtype in (np.uint8, np.int8)
+    vals = e4m3_decode_np(q.view(np.uint8))
+    sc = decode_scales(scale, scale_format)
+    if sc.ndim != vals.ndim:
+        raise ValueError("Scale rank must match logical weight rank")
+    axis_to_block = dict(zip([a + vals.ndim if a < 0 else a for a in block_axes], block_shape))
+    expected = tuple(-(-d // axis_to_block[ax]) if ax in axis_to_block else d for ax, d in enumerate(vals.shape))
+    if tuple(sc.shape) != expected:
+        raise ValueError(f"Invalid scale grid shape: expected {expected}, got {tuple(sc.shape)}")
+    for ax, bs in sorted(axis_to_block.items()):
+        sc = np.repeat(sc, bs, axis=ax)
+    sc = sc[tuple(slice(0, d) for d in vals.shape)]
+    with np.errstate(invalid="ignore", over="ignore"):
+        prod = (vals * sc).astype(np.float32)
+    return prod if out == "f32" else f32_to_bf16_bits(prod)

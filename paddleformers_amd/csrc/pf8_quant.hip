@@ -524,6 +524,76 @@ __global__ __launch_bounds__(256) void k_weight_dequant(const uint8_t* __restric
 }
 
 // ---------------------------------------------------------------------------------------------
+// Block-FP8 checkpoint dequantization: out = cast(e4m3(q) * scale(block)), any block geometry on the
+// last two axes, partial trailing blocks cropped, scales as UE8M0 exponent bytes or fp32/bf16/fp16.
+// One thread per 16 consecutive bytes of a row; HBM-bound (1 B in, 2 or 4 B out).  IDX is the
+// integer type of the index arithmetic: 32-bit whenever the tensor allows it (64-bit divisions are
+// emulated and would cost more than the data movement).
+// ---------------------------------------------------------------------------------------------
+enum { SCALE_F32 = 0, SCALE_UE8M0 = 1, SCALE_BF16 = 2, SCALE_F16 = 3 };
+
+__device__ __forceinline__ float load_block_scale(const void* s, int fmt, int64_t i) {
+    if (fmt == SCALE_F32) return reinterpret_cast<const float*>(s)[i];
+    if (fmt == SCALE_UE8M0) {
+        const uint32_t e = reinterpret_cast<const uint8_t*>(s)[i];
+        // 2^(e-127): exponent field e, e == 0 is the subnormal 2^-127, e == 255 decodes to +inf
+        return e == 0u ? u2f(0x00400000u) : u2f(e << 23);
+    }
+    if (fmt == SCALE_BF16) return u2f((uint32_t)reinterpret_cast<const uint16_t*>(s)[i] << 16);
+    return (float)reinterpret_cast<const _Float16*>(s)[i];
+}
+
+template <int OUT_F32, typename IDX>
+__global__ __launch_bounds__(256) void k_block_dequant(const uint8_t* __restrict__ q, const void* __restrict__ s, int fmt, int64_t B,
+                                                       int64_t R, int64_t C, int64_t br, int64_t bc, void* __restrict__ out) {
+    const IDX chunks = (IDX)((C + 15) / 16);
+    const IDX idx = (IDX)blockIdx.x * 256 + threadIdx.x;
+    if ((int64_t)idx >= B * R * (int64_t)chunks) return;
+    const IDX ch = idx % chunks, row = idx / chunks;               // row runs over B * R
+    const IDX b = row / (IDX)R, r = row % (IDX)R;
+    const IDX gr = (IDX)((R + br - 1) / br), gc = (IDX)((C + bc - 1) / bc);
+    const IDX c0 = ch * 16;
+    const int n = (IDX)C - c0 < 16 ? (int)((IDX)C - c0) : 16;
+    const int64_t srow = ((int64_t)b * gr + r / (IDX)br) * gc;
+    const IDX cb0 = c0 / (IDX)bc, cb1 = (c0 + n - 1) / (IDX)bc;
+    const uint8_t* qp = q + (int64_t)row * C + c0;
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    const bool vec = n == 16 && ((reinterpret_cast<uintptr_t>(qp) & 15u) == 0);
+    if (vec) {
+        const uint4 v = *reinterpret_cast<const uint4*>(qp);
+        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    } else {
+        for (int i = 0; i < n; ++i) w[i >> 2] |= (uint32_t)qp[i] << (8 * (i & 3));
+    }
+    float f[16];
+    const bool one_scale = cb0 == cb1;
+    const float s0 = load_block_scale(s, fmt, srow + cb0);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        float sc = s0;
+        if (!one_scale && i < n) sc = load_block_scale(s, fmt, srow + (c0 + i) / (IDX)bc);
+        f[i] = e4m3_to_f32((w[i >> 2] >> (8 * (i & 3))) & 0xFFu) * sc;
+    }
+    if (OUT_F32) {
+        float* op = reinterpret_cast<float*>(out) + (int64_t)row * C + c0;
+        if (vec && (reinterpret_cast<uintptr_t>(op) & 15u) == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) reinterpret_cast<f32x4*>(op)[i] = (f32x4){f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]};
+        } else {
+            for (int i = 0; i < n; ++i) op[i] = f[i];
+        }
+    } else {
+        uint16_t* op = reinterpret_cast<uint16_t*>(out) + (int64_t)row * C + c0;
+        if (vec && (reinterpret_cast<uintptr_t>(op) & 15u) == 0) {
+            st16(op, make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7])));
+            st16(op + 8, make_uint4(pack_bf16(f[8], f[9]), pack_bf16(f[10], f[11]), pack_bf16(f[12], f[13]), pack_bf16(f[14], f[15])));
+        } else {
+            for (int i = 0; i < n; ++i) op[i] = (uint16_t)(pack_bf16(f[i], 0.0f) & 0xFFFFu);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // self-test kernels
 // ---------------------------------------------------------------------------------------------
 
@@ -768,6 +838,26 @@ extern "C" int pf8_weight_dequant(const uint8_t* q, const float* s, int64_t R, i
     const int64_t n = R * C;
     dim3 grid((unsigned)((n + 255) / 256)), block(256);
     hipLaunchKernelGGL(k_weight_dequant, grid, block, 0, (hipStream_t)stream, q, s, R, C, out);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_block_dequant(const uint8_t* q, const void* scale, int scale_format, int64_t B, int64_t R, int64_t C,
+                                 int64_t block_r, int64_t block_c, void* out, int out_f32, pf8_stream_t stream) {
+    PF8_REQUIRE(B >= 0 && R >= 0 && C >= 0, "negative shape");
+    PF8_REQUIRE(block_r > 0 && block_c > 0, "block sizes must be positive");
+    PF8_REQUIRE(scale_format >= 0 && scale_format <= 3, "scale_format must be 0 (fp32), 1 (ue8m0), 2 (bf16) or 3 (fp16)");
+    if (B == 0 || R == 0 || C == 0) return PF8_OK;
+    PF8_REQUIRE(q && scale && out, "null pointer");
+    PF8_REQUIRE(B * R < (1LL << 40) && C < (1LL << 40), "tensor too large");
+    const int64_t threads = B * R * ((C + 15) / 16);
+    PF8_REQUIRE((threads + 255) / 256 <= 0x7FFFFFFF, "tensor too large for one launch");
+    dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+    const bool small = threads + 256 < (1LL << 31) && C + 16 < (1LL << 31) && block_r < (1LL << 31) && block_c < (1LL << 31);
+    hipStream_t st = (hipStream_t)stream;
+    if (out_f32 && small) hipLaunchKernelGGL((k_block_dequant<1, uint32_t>), grid, block, 0, st, q, scale, scale_format, B, R, C, block_r, block_c, out);
+    else if (out_f32) hipLaunchKernelGGL((k_block_dequant<1, int64_t>), grid, block, 0, st, q, scale, scale_format, B, R, C, block_r, block_c, out);
+    else if (small) hipLaunchKernelGGL((k_block_dequant<0, uint32_t>), grid, block, 0, st, q, scale, scale_format, B, R, C, block_r, block_c, out);
+    else hipLaunchKernelGGL((k_block_dequant<0, int64_t>), grid, block, 0, st, q, scale, scale_format, B, R, C, block_r, block_c, out);
     return pf8_check_launch(__func__);
 }
 
