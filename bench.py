@@ -200,6 +200,21 @@ def bench_other_gemms(iters=10, warmup=3):
     ms = time_kernel(lambda: dq.dequantize({"qweight": qw, "scale": sc}, torch.bfloat16), [()], 5, 2)
     out["block_dequant_config3_w1"] = {"bytes": Ew * 2 * Iw * Hw * 3 + sc.numel(), "ms": ms}
     del qw, sc
+    torch.cuda.empty_cache()
+    # config 5 token reordering either side of the expert MLP: 16384 tokens x top-8 over 128 experts
+    Tt, Ht, tk, Et = 16384, 4096, 8, 128
+    rng = np.random.default_rng(5)
+    rm_np = np.stack([rng.permutation(Et)[:tk] for _ in range(Tt)]).astype(np.int32)
+    cnts = [int((rm_np == e).sum()) for e in range(Et)]
+    rm_t = torch.from_numpy(rm_np).cuda()
+    pr_t = torch.rand((Tt, tk), device="cuda")
+    xt = torch.randn((Tt, Ht), device="cuda").to(torch.bfloat16)
+    ms = time_kernel(lambda: F8.moe_permute(xt, None, rm_t, pr_t, Et, cnts, 128, validate=False), [()], 5, 2)
+    ux, rowmap, up, _ = F8.moe_permute(xt, None, rm_t, pr_t, Et, cnts, 128)
+    out["moe_permute_config5"] = {"bytes": Tt * Ht * 2 + ux.numel() * 2, "ms": ms}
+    ms = time_kernel(lambda: F8.moe_unpermute(ux, rowmap, rm_t, up, Tt, Et), [()], 5, 2)
+    out["moe_unpermute_config5"] = {"bytes": Tt * tk * Ht * 2 + Tt * Ht * 2, "ms": ms}
+    del xt, ux
     for v in out.values():
         if "flop" in v:
             v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)

@@ -119,6 +119,32 @@ int pf8_block_dequant(const uint8_t* q, const void* scale, int scale_format, int
                       int64_t C, int64_t block_r, int64_t block_c, void* out, int out_f32,
                       pf8_stream_t stream);
 
+/* paddle.nn.functional.moe_permute(hidden_states, scale, expert_routemap_topk, expert_prob_topk,
+ * num_experts, tokens_per_expert, padding_alignment) as UnZipNode.forward / ZipNode.backward call it
+ * (cli/train/deepseek_v3_pretrain/moe_utils.py:141-186, 217-261; ernie twin
+ * models/moe/token_dispatcher/moe_utils.py:222, 349).  x [T,H] bf16 (x_is_fp8 = 0) or e4m3 bytes with
+ * xs fp32 [T,H/128]; routemap int32 [T,topk] (expert id, negative = unused slot), probs fp32 [T,topk]
+ * or NULL; tokens_per_expert: HOST array of E routed-row counts.  Outputs: out_x [Mpad,H] with every
+ * expert's segment padded to a multiple of padding_alignment (zero rows), rowmap int32 [T,E] (row of
+ * token t in expert e's segment, -1 = not routed; tokens keep their order inside a segment),
+ * out_probs fp32 [Mpad] (0 on padding rows; NULL to skip), out_xs fp32 [Mpad,H/128] (with xs).
+ * *overflow (device int32, cleared by the caller) is set when a token is routed to an expert whose
+ * tokens_per_expert count is already used up; such copies are dropped. */
+int pf8_moe_permute(const void* x, int x_is_fp8, const float* xs, const int32_t* routemap,
+                    const float* probs, int64_t T, int64_t H, int topk, int E,
+                    const int64_t* tokens_per_expert, int padding_alignment, void* out_x,
+                    int32_t* rowmap, float* out_probs, float* out_xs, int32_t* overflow,
+                    pf8_stream_t stream);
+
+/* paddle.nn.functional.moe_unpermute(hidden_states_unzipped, zipped_expertwise_rowmap,
+ * expert_routemap_topk, token_prob_unzipped, total_zipped_tokens, num_experts) as ZipNode.forward /
+ * UnZipNode.backward call it (moe_utils.py:188-215): out[t] = bf16(sum over the token's used slots,
+ * in slot order, fp32) of unzipped[rowmap[t, routemap[t,k]]]; out_probs[t,k] = probs_unzipped of
+ * that row (0 for an unused slot; NULL to skip). */
+int pf8_moe_unpermute(const uint16_t* unzipped, const int32_t* rowmap, const int32_t* routemap,
+                      const float* probs_unzipped, int64_t T, int64_t H, int topk, int E,
+                      uint16_t* out, float* out_probs, pf8_stream_t stream);
+
 /* fused_swiglu_weighted_bwd(o1, do2_s, probs) -- transformers/fp8_utils.py:1049-1052; un-fused
  * definition ernie token_dispatcher/fp8_utils.py:1088-1092.  -> do1 bf16 [M,2I], probs_grad fp32 [M],
  * o2_s bf16 [M,I]. */

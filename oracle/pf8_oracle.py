@@ -5,6 +5,13 @@ benchmark.  The product package never imports it.
 
 bf16 tensors are numpy uint16 bit patterns, e4m3 tensors are numpy uint8 codes, scales float32.
 Each wrapper names the C function it calls; the reference citations live in pf8_oracle.c.
+
+Two restatements at the end of this file are plain numpy, not C:
+  block_dequant              pinned by the reference's own known-answer vectors
+                             (tests/test_oracle_dequant.py)
+  moe_permute / moe_unpermute  PARITY UNPINNED: no test, fixture or importable implementation of
+                             the operators exists in the reference; checked only against the
+                             invariants their call sites rely on (tests/test_oracle_ops.py)
 """
 from __future__ import annotations
 
@@ -378,3 +385,60 @@ def block_dequant(q: np.ndarray, scale: np.ndarray, scale_format: str, block_axe
     with np.errstate(invalid="ignore", over="ignore"):
         prod = (vals * sc).astype(np.float32)
     return prod if out == "f32" else f32_to_bf16_bits(prod)
+
+
+# ---------------------------------------------------------------------------------------------
+# moe_permute / moe_unpermute (numpy restatement).  PARITY UNPINNED: the operators live in the
+# paddlepaddle-gpu binary, the reference holds no test or fixture for them; the semantics below are
+# what its call sites rely on (cli/train/deepseek_v3_pretrain/moe_utils.py:141-261): expert-sorted
+# rows, token order kept inside an expert, zero rows up to a multiple of padding_alignment, a
+# [T, num_experts] row map with -1 for "not routed", fp32 summation in slot order on the way back.
+# ---------------------------------------------------------------------------------------------
+
+
+def moe_permute(x, xs, routemap, probs, num_experts, tokens_per_expert, padding_alignment):
+    """x: uint16 bf16 bits or uint8 e4m3 codes [T, H]; xs fp32 [T, H/128] or None."""
+    T, H = x.shape
+    a = padding_alignment
+    padded = [(int(c) + a - 1) // a * a for c in tokens_per_expert]
+    starts = np.concatenate([[0], np.cumsum(padded)]).astype(np.int64)
+    mpad = int(starts[-1])
+    out_x = np.zeros((mpad, H), dtype=x.dtype)
+    out_p = np.zeros((mpad, 1), dtype=np.float32)
+    out_s = None if xs is None else np.zeros((mpad, xs.shape[1]), dtype=np.float32)
+    rowmap = np.full((T, num_experts), -1, dtype=np.int32)
+    fill = np.zeros(num_experts, dtype=np.int64)
+    for t in range(T):
+        for e in sorted(set(int(v) for v in routemap[t] if 0 <= v < num_experts)):
+            rowmap[t, e] = starts[e] + fill[e]
+            fill[e] += 1
+    assert (fill <= np.asarray(tokens_per_expert)).all()
+    for t in range(T):
+        for k in range(routemap.shape[1]):
+            e = int(routemap[t, k])
+            if e < 0 or e >= num_experts:
+                continue
+            r = rowmap[t, e]
+            out_x[r] = x[t]
+            if probs is not None:
+                out_p[r, 0] = probs[t, k]
+            if xs is not None:
+                out_s[r] = xs[t]
+    return out_x, rowmap, out_p, out_s
+
+
+def moe_unpermute(unzipped_bits, rowmap, routemap, probs_unzipped, total_tokens, num_experts):
+    T, topk = total_tokens, routemap.shape[1]
+    H = unzipped_bits.shape[1]
+    u = bf16_bits_to_f32(unzipped_bits)
+    acc = np.zeros((T, H), dtype=np.float32)
+    out_p = np.zeros((T, topk), dtype=np.float32)
+    for t in range(T):
+        for k in range(topk):
+            e = int(routemap[t, k])
+            if e < 0 or e >= num_experts or rowmap[t, e] < 0:
+                continue
+            acc[t] = (acc[t] + u[rowmap[t, e]]).astype(np.float32)
+            if probs_unzipped is not None:
+                out_p[t, k] = probs_unzipped.reshape(-1)[rowmap[t, e]]
+    return f32_to_bf16_bits(acc), out_p

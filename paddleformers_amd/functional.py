@@ -448,3 +448,86 @@ def swiglu(x: torch.Tensor, y: Optional[torch.Tensor] = None) -> torch.Tensor:
     o2 = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
     _lib.call("pf8_swiglu_weighted_quant", _p(x2), None, M, I, _p(q), _p(s), _p(o2), 0, 0, _stream())
     return o2.reshape(*x.shape[:-1], I)
+
+
+# ---------------------------------------------------------------------------------------------
+# moe_permute / moe_unpermute (paddle.nn.functional in the reference)
+# ---------------------------------------------------------------------------------------------
+
+
+def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expert_routemap_topk: torch.Tensor,
+                expert_prob_topk: Optional[torch.Tensor], num_experts: int, tokens_per_expert: Sequence[int],
+                padding_alignment: int, do_gather: bool = True, validate: bool = True):
+    """Gather the routed copies of every token into expert-sorted order, every expert's segment
+    padded with zero rows to a multiple of `padding_alignment`.
+
+    cli/train/deepseek_v3_pretrain/moe_utils.py:152-186 (UnZipNode.forward), :217-261 (ZipNode.backward).
+    hidden_states bf16 [T, H], or float8_e4m3fn [T, H] with `scale` fp32 [T, H/128];
+    expert_routemap_topk int32 [T, topk] (negative = unused slot); expert_prob_topk fp32 [T, topk].
+    Returns (hidden_states_unzipped [Mpad, H], zipped_expertwise_rowmap int32 [T, num_experts],
+    token_prob_unzipped fp32 [Mpad, 1], scale_unzipped fp32 [Mpad, H/128] or None).
+    A token routed to an expert beyond its `tokens_per_expert` count raises ValueError; that check
+    reads a flag back from the device (one synchronisation), `validate=False` skips it.
+    """
+    if not do_gather:
+        raise ValueError("do_gather=False is not supported")
+    _dev(hidden_states, "hidden_states")
+    _dev(expert_routemap_topk, "expert_routemap_topk")
+    if hidden_states.dim() != 2 or expert_routemap_topk.dim() != 2 or expert_routemap_topk.shape[0] != hidden_states.shape[0]:
+        raise ValueError("hidden_states must be [T, H] and expert_routemap_topk [T, topk]")
+    is_fp8 = hidden_states.dtype == FP8
+    if not is_fp8 and hidden_states.dtype != torch.bfloat16:
+        raise ValueError("hidden_states must be bfloat16 or float8_e4m3fn")
+    if is_fp8 != (scale is not None):
+        raise ValueError("float8 hidden_states come with a scale, bfloat16 hidden_states without")
+    T, H = hidden_states.shape
+    topk = expert_routemap_topk.shape[1]
+    counts = [int(c) for c in tokens_per_expert]
+    if len(counts) != num_experts:
+        raise ValueError("tokens_per_expert must hold num_experts counts")
+    a = int(padding_alignment)
+    mpad = sum((c + a - 1) // a * a for c in counts)
+    x = hidden_states.contiguous()
+    rm = expert_routemap_topk.to(torch.int32).contiguous()
+    pr = None if expert_prob_topk is None else expert_prob_topk.to(torch.float32).contiguous()
+    dev = x.device
+    out_x = torch.empty((mpad, H), dtype=hidden_states.dtype, device=dev)
+    rowmap = torch.empty((T, num_experts), dtype=torch.int32, device=dev)
+    out_p = torch.empty((mpad, 1), dtype=torch.float32, device=dev)
+    out_s = None
+    xs = None
+    if is_fp8:
+        if tuple(scale.shape) != (T, H // 128) or scale.dtype != torch.float32:
+            raise ValueError("scale must be float32 [T, H/128]")
+        xs = scale.contiguous()
+        out_s = torch.empty((mpad, H // 128), dtype=torch.float32, device=dev)
+    overflow = torch.zeros(1, dtype=torch.int32, device=dev)
+    cnt = (C.c_int64 * num_experts)(*counts)
+    _lib.call("pf8_moe_permute", _p(x), int(is_fp8), _p(xs), _p(rm), _p(pr), T, H, topk, num_experts, cnt, a, _p(out_x), _p(rowmap),
+              _p(out_p), _p(out_s), _p(overflow), _stream())
+    if validate and int(overflow.item()):
+        raise ValueError("expert_routemap_topk routes more tokens to an expert than tokens_per_expert allows")
+    return out_x, rowmap, out_p, out_s
+
+
+def moe_unpermute(hidden_states_unzipped: torch.Tensor, zipped_expertwise_rowmap: torch.Tensor, expert_routemap_topk: torch.Tensor,
+                  token_prob_unzipped: Optional[torch.Tensor], total_zipped_tokens: int, num_experts: int):
+    """Sum the routed copies of every token back (fp32 sum in slot order, bf16 out) and return the
+    probabilities in [T, topk] order.  moe_utils.py:188-215 (UnZipNode.backward, ZipNode.forward).
+    Returns (hidden_states [T, H] bf16, expert_prob_topk fp32 [T, topk])."""
+    _dev(hidden_states_unzipped, "hidden_states_unzipped")
+    if hidden_states_unzipped.dtype != torch.bfloat16 or hidden_states_unzipped.dim() != 2:
+        raise ValueError("hidden_states_unzipped must be bfloat16 [Mpad, H]")
+    T = int(total_zipped_tokens)
+    H = hidden_states_unzipped.shape[1]
+    topk = expert_routemap_topk.shape[1]
+    if tuple(zipped_expertwise_rowmap.shape) != (T, num_experts) or expert_routemap_topk.shape[0] != T:
+        raise ValueError("zipped_expertwise_rowmap must be [T, num_experts] and expert_routemap_topk [T, topk]")
+    u = hidden_states_unzipped.contiguous()
+    rowmap = zipped_expertwise_rowmap.to(torch.int32).contiguous()
+    rm = expert_routemap_topk.to(torch.int32).contiguous()
+    pu = None if token_prob_unzipped is None else token_prob_unzipped.to(torch.float32).contiguous()
+    out = torch.empty((T, H), dtype=torch.bfloat16, device=u.device)
+    out_p = torch.empty((T, topk), dtype=torch.float32, device=u.device)
+    _lib.call("pf8_moe_unpermute", _p(u), _p(rowmap), _p(rm), _p(pu), T, H, topk, num_experts, _p(out), _p(out_p), _stream())
+    return out, out_p

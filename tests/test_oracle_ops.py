@@ -304,3 +304,32 @@ def test_wgrad_is_dequant_matmul_with_accumulate():
     # it approximates dW = x^T . dout
     full = O.bf16_bits_to_f32(x).astype(np.float64).T @ O.bf16_bits_to_f32(d).astype(np.float64)
     assert G.rel_fro(out, full) < 0.06
+
+
+def test_moe_permute_unpermute_invariants():
+    """The numpy restatement of moe_permute / moe_unpermute (parity unpinned): segments start at the
+    padded prefix sums, rows of an expert keep token order, padding rows are zero, the way back sums
+    the copies (exact for small integers) and returns the probabilities to their slots."""
+    rng = np.random.default_rng(0)
+    T, H, topk, E = 50, 16, 3, 5
+    rm = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    rm[rng.random(rm.shape) < 0.2] = -1
+    counts = [int((rm == e).sum()) for e in range(E)]
+    probs = rng.random(rm.shape).astype(np.float32)
+    xv = rng.integers(-4, 5, size=(T, H)).astype(np.float32)
+    x = O.f32_to_bf16_bits(xv)
+    ox, rowmap, op, _ = O.moe_permute(x, None, rm, probs, E, counts, 8)
+    padded = [(c + 7) // 8 * 8 for c in counts]
+    starts = np.concatenate([[0], np.cumsum(padded)])
+    assert ox.shape[0] == starts[-1]
+    for e in range(E):
+        col = rowmap[:, e][rowmap[:, e] >= 0]
+        assert len(col) == counts[e] and (col == starts[e] + np.arange(counts[e])).all()
+        assert not ox[starts[e] + counts[e]:starts[e + 1]].any() and not op[starts[e] + counts[e]:starts[e + 1]].any()
+    for t in range(T):
+        for k in range(topk):
+            if rm[t, k] >= 0:
+                assert (ox[rowmap[t, rm[t, k]]] == x[t]).all() and op[rowmap[t, rm[t, k]], 0] == probs[t, k]
+    back, pb = O.moe_unpermute(ox, rowmap, rm, op, T, E)
+    assert (O.bf16_bits_to_f32(back) == xv * (rm >= 0).sum(axis=1, keepdims=True)).all()
+    assert (pb == np.where(rm >= 0, probs, 0)).all()
