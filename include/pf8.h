@@ -145,6 +145,16 @@ int pf8_moe_unpermute(const uint16_t* unzipped, const int32_t* rowmap, const int
                       const float* probs_unzipped, int64_t T, int64_t H, int topk, int E,
                       uint16_t* out, float* out_probs, pf8_stream_t stream);
 
+/* paddle.incubate.nn.functional.fused_rms_norm_ext(x, norm_w, eps) -> (y, invvar) and its gradient
+ * paddle._C_ops.fused_rms_norm_ext_grad(x, norm_w, invvar, dy, eps) -> (dx, dw), the norm that
+ * FusedNormFP8MLPFunction recomputes (transformers/fp8_utils.py:470-475, 520-541, 687-741).
+ * x, dy, y, dx bf16 [M,H], w bf16 [H], invar fp32 [M] = 1/sqrt(mean(x^2)+eps); y = bf16(x*invar*w).
+ * dw fp32 [H] is ADDED to (the caller zeroes it), with atomics: its rounding depends on the order. */
+int pf8_rms_norm_fwd(const uint16_t* x, const uint16_t* w, float eps, int64_t M, int64_t H,
+                     uint16_t* y, float* invar, pf8_stream_t stream);
+int pf8_rms_norm_bwd(const uint16_t* x, const uint16_t* w, const float* invar, const uint16_t* dy,
+                     int64_t M, int64_t H, uint16_t* dx, float* dw, pf8_stream_t stream);
+
 /* fused_swiglu_weighted_bwd(o1, do2_s, probs) -- transformers/fp8_utils.py:1049-1052; un-fused
  * definition ernie token_dispatcher/fp8_utils.py:1088-1092.  -> do1 bf16 [M,2I], probs_grad fp32 [M],
  * o2_s bf16 [M,I]. */

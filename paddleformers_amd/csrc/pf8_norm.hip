@@ -1,0 +1,149 @@
+// pf8_norm.hip -- RMSNorm forward and backward for the FP8 MLP with norm recompute
+// (FusedNormFP8MLPFunction): y = bf16(x * invar * w), invar = 1/sqrt(mean(x^2) + eps) per row.
+// HBM-bound row kernels: one workgroup per row forward, one per block of rows backward (the weight
+// gradient is accumulated per workgroup in registers and added to the fp32 output once).
+#include "pf8_device.h"
+#include "pf8_host.h"
+#include "../../include/pf8.h"
+
+namespace pf8 {
+
+__device__ __forceinline__ float block_sum(float v, float* lds4) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();                       // lds4 may still be read from the previous call
+    if ((threadIdx.x & 63) == 0) lds4[wave] = v;
+    __syncthreads();
+    return (lds4[0] + lds4[1]) + (lds4[2] + lds4[3]);
+}
+
+__global__ __launch_bounds__(256) void k_rms_norm_fwd(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float eps, int64_t M,
+                                                      int64_t H, uint16_t* __restrict__ y, float* __restrict__ invar) {
+    __shared__ float lds4[4];
+    const int64_t r = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int64_t chunks = H / 8;
+    const uint4* xr = reinterpret_cast<const uint4*>(x + r * H);
+    float ss = 0.0f;
+    for (int64_t c = tid; c < chunks; c += 256) {
+        float v[8];
+        unpack8(xr[c], v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss = __builtin_fmaf(v[i], v[i], ss);
+    }
+    ss = block_sum(ss, lds4);
+    const float iv = 1.0f / __builtin_sqrtf(ss / (float)H + eps);
+    if (tid == 0) invar[r] = iv;
+    uint4* yr = reinterpret_cast<uint4*>(y + r * H);
+    const uint4* wr = reinterpret_cast<const uint4*>(w);
+    for (int64_t c = tid; c < chunks; c += 256) {
+        float v[8], g[8];
+        unpack8(xr[c], v);
+        unpack8(wr[c], g);
+        uint4 o;
+        o.x = pack_bf16(v[0] * iv * g[0], v[1] * iv * g[1]);
+        o.y = pack_bf16(v[2] * iv * g[2], v[3] * iv * g[3]);
+        o.z = pack_bf16(v[4] * iv * g[4], v[5] * iv * g[5]);
+        o.w = pack_bf16(v[6] * iv * g[6], v[7] * iv * g[7]);
+        yr[c] = o;
+    }
+}
+
+// dx = invar * (g - x * invar^2 * mean(g * x)),  g = dy * w;   dw += sum_rows dy * x * invar
+template <int MAXC>   // column chunks (of 8) per thread whose weight gradient lives in registers
+__global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                      const float* __restrict__ invar, const uint16_t* __restrict__ dy, int64_t M, int64_t H,
+                                                      int rows_per_wg, uint16_t* __restrict__ dx, float* __restrict__ dw) {
+    __shared__ float lds4[4];
+    const int tid = threadIdx.x;
+    const int64_t chunks = H / 8;
+    const uint4* wr = reinterpret_cast<const uint4*>(w);
+    float dwa[MAXC][8];
+#pragma unroll
+    for (int j = 0; j < MAXC; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dwa[j][i] = 0.0f;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
+    for (int64_t r = r0; r < r0 + rows_per_wg && r < M; ++r) {
+        const uint4* xr = reinterpret_cast<const uint4*>(x + r * H);
+        const uint4* dr = reinterpret_cast<const uint4*>(dy + r * H);
+        const float iv = invar[r];
+        float s1 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < MAXC; ++j) {
+            const int64_t c = tid + 256 * j;
+            if (c < chunks) {
+                float xv[8], dv[8], gv[8];
+                unpack8(xr[c], xv);
+                unpack8(dr[c], dv);
+                unpack8(wr[c], gv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    s1 = __builtin_fmaf(dv[i] * gv[i], xv[i], s1);
+                    dwa[j][i] = __builtin_fmaf(dv[i] * xv[i], iv, dwa[j][i]);
+                }
+            }
+        }
+        s1 = block_sum(s1, lds4);
+        const float k = iv * iv * iv * (s1 / (float)H);
+        uint4* oxr = reinterpret_cast<uint4*>(dx + r * H);
+#pragma unroll
+        for (int j = 0; j < MAXC; ++j) {
+            const int64_t c = tid + 256 * j;
+            if (c < chunks) {
+                float xv[8], dv[8], gv[8], o[8];
+                unpack8(xr[c], xv);
+                unpack8(dr[c], dv);
+                unpack8(wr[c], gv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o[i] = dv[i] * gv[i] * iv - xv[i] * k;
+                oxr[c] = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < MAXC; ++j) {
+        const int64_t c = tid + 256 * j;
+        if (c < chunks)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) atomicAdd(dw + c * 8 + i, dwa[j][i]);
+    }
+}
+
+}  // namespace pf8
+
+using namespace pf8;
+
+#define PF8_REQUIRE(cond, msg) do { if (!(cond)) return pf8_fail(PF8_EINVAL, __func__, msg); } while (0)
+#define PF8_ALIGNED16(p) ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)
+
+extern "C" int pf8_rms_norm_fwd(const uint16_t* x, const uint16_t* w, float eps, int64_t M, int64_t H, uint16_t* y, float* invar,
+                                pf8_stream_t stream) {
+    PF8_REQUIRE(M >= 0 && H > 0 && H % 8 == 0, "H must be a positive multiple of 8");
+    if (M == 0) return PF8_OK;
+    PF8_REQUIRE(M <= 0x7FFFFFFF, "too many rows");
+    PF8_REQUIRE(x && w && y && invar, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(w) && PF8_ALIGNED16(y), "pointers must be 16-byte aligned");
+    hipLaunchKernelGGL(k_rms_norm_fwd, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, x, w, eps, M, H, y, invar);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_rms_norm_bwd(const uint16_t* x, const uint16_t* w, const float* invar, const uint16_t* dy, int64_t M, int64_t H,
+                                uint16_t* dx, float* dw, pf8_stream_t stream) {
+    PF8_REQUIRE(M >= 0 && H > 0 && H % 8 == 0, "H must be a positive multiple of 8");
+    PF8_REQUIRE(H <= 8 * 256 * 8, "H larger than 16384 is not supported");
+    if (M == 0) return PF8_OK;
+    PF8_REQUIRE(x && w && invar && dy && dx && dw, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(w) && PF8_ALIGNED16(dy) && PF8_ALIGNED16(dx), "pointers must be 16-byte aligned");
+    // enough workgroups to fill the device, few enough that the atomics on dw stay a small share
+    int rows = (int)((M + 2047) / 2048);
+    if (rows < 1) rows = 1;
+    const int64_t wgs = (M + rows - 1) / rows;
+    const int64_t chunks = H / 8;
+    hipStream_t st = (hipStream_t)stream;
+    if (chunks <= 256 * 2) hipLaunchKernelGGL(k_rms_norm_bwd<2>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, rows, dx, dw);
+    else if (chunks <= 256 * 4) hipLaunchKernelGGL(k_rms_norm_bwd<4>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, rows, dx, dw);
+    else hipLaunchKernelGGL(k_rms_norm_bwd<8>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, rows, dx, dw);
+    return pf8_check_launch(__func__);
+}

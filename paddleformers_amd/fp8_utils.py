@@ -25,6 +25,11 @@ __all__ = [
     "FP8LinearFunctionBase",
     "FP8GroupGemmMlpFunctionNode",
     "FP8Mlp",
+    "FP8Linear",
+    "FP8KeepXLinear",
+    "FP8LinearFunction",
+    "FP8MlpFunction",
+    "FusedNormFP8MLPFunction",
     "WeightGradStore",
     "weight_quant",
     "fused_stack_quant",
@@ -315,21 +320,217 @@ class FP8LinearFunctionBase:
         return o1, x_fp8, x_scale, o3
 
 
-class FP8Mlp(torch.nn.Module):
-    """fp8_utils.py:806-850: SwiGLU MLP with w1 [H, 2I] and w2 [I, H] in bf16, FP8 forward."""
+    @staticmethod
+    def common_fp8_mlp_bwd(do3, x_t_fp8, x_t_scale, w1, w2, o1=None, x_fp8=None, x_scale=None, apply_backward_hook=False):
+        """fp8_utils.py:352-446: backward of the dense SwiGLU MLP.  Either o1 is given, or the
+        quantised input from which it is recomputed.  With apply_backward_hook the weight gradients
+        go into w.main_grad / w.grad (possibly deferred) and only dx is returned."""
+        if o1 is not None and (x_fp8 is not None or x_scale is not None):
+            raise ValueError("When o1 is provided, both x_fp8 and x_scale must be None.")
+        if o1 is None:
+            if x_fp8 is None or x_scale is None:
+                raise ValueError("When o1 is None, both x_fp8 and x_scale must be provided.")
+            w1_fp8, w1_scale = weight_quant(w1, True)
+            o1 = torch.empty([x_fp8.shape[0], w1_fp8.shape[0]], dtype=do3.dtype, device=do3.device)
+            deep_gemm.fp8_gemm_nt((x_fp8, x_scale.T), (w1_fp8, w1_scale), o1)
+        o2 = swiglu(o1)
+        do2, do3_t_fp8, do3_t_scale = FP8LinearFunctionBase.compute_fp8_linear(do3, w2, return_mode="with_input_transpose_quant")
+        o2 = FP8LinearFunctionBase.padding(o2, 0)
+        o2_t_fp8, o2_t_scale = F8.fp8_quant_blockwise(o2, output_scale_transpose=True, quant_method="1x128", input_transpose=True,
+                                                      return_transpose_only=True)
+        dw1 = dw2 = None
+        if apply_backward_hook:
+            FP8LinearFunctionBase.compute_expert_w_grad(o2_t_fp8, o2_t_scale, do3_t_fp8, do3_t_scale, True, True, w2,
+                                                        rtn_dtype=torch.float32)
+        else:
+            dw2 = FP8LinearFunctionBase.kitchen_gemm(o2_t_fp8, o2_t_scale, do3_t_fp8, do3_t_scale, True, True, rtn_dtype=torch.float32)
+        do1, _ = F8.swiglu_grad(o1, None, do2)
+        dx, do1_t_fp8, do1_t_scale = FP8LinearFunctionBase.compute_fp8_linear(do1, w1, return_mode="with_input_transpose_quant")
+        if apply_backward_hook:
+            FP8LinearFunctionBase.compute_expert_w_grad(x_t_fp8, x_t_scale, do1_t_fp8, do1_t_scale, True, True, w1,
+                                                        rtn_dtype=torch.float32)
+            return dx
+        dw1 = FP8LinearFunctionBase.kitchen_gemm(x_t_fp8, x_t_scale, do1_t_fp8, do1_t_scale, True, True, rtn_dtype=torch.float32)
+        assert dw1 is not None and dw2 is not None
+        return dx, dw1, dw2
 
-    def __init__(self, hidden_size, intermediate_size, device=None):
+    @staticmethod
+    def fp8_mlp_fwd_norm_rc(x, norm_w, norm_eps, w1, w2):
+        """fp8_utils.py:469-475."""
+        norm_output, _ = F8.fused_rms_norm_ext(x, norm_w, norm_eps)
+        return FP8LinearFunctionBase.fp8_mlp_fwd(norm_output, w1, w2)[3]
+
+    @staticmethod
+    def fp8_mlp_bwd(do3, x, w1, w2, apply_backward_hook=False):
+        """fp8_utils.py:477-517: quantise x both ways, recompute o1, run the common backward."""
+        do3 = do3.reshape([-1, do3.shape[-1]])
+        x_orig_shape = x.shape
+        x = x.reshape([-1, x_orig_shape[-1]])
+        x_fp8, x_scale, x_t_fp8, x_t_scale = FP8LinearFunctionBase.padding_and_quant_input(x)
+        res = FP8LinearFunctionBase.common_fp8_mlp_bwd(do3, x_t_fp8, x_t_scale, w1, w2, o1=None, x_fp8=x_fp8, x_scale=x_scale,
+                                                       apply_backward_hook=apply_backward_hook)
+        dx = res if apply_backward_hook else res[0]
+        if len(x_orig_shape) > 2:
+            dx = dx.reshape([x_orig_shape[0], -1, dx.shape[-1]])
+        return dx if apply_backward_hook else (dx, res[1], res[2])
+
+    @staticmethod
+    def fp8_mlp_bwd_norm_rc(do3, x, norm_w, norm_eps, w1, w2):
+        """fp8_utils.py:519-541: recompute the norm, backward through the MLP (weight gradients go
+        to main_grad / grad), then through the norm; the norm weight's gradient is accumulated."""
+        norm_output, invar = F8.fused_rms_norm_ext(x, norm_w, norm_eps)
+        d_norm_output = FP8LinearFunctionBase.fp8_mlp_bwd(do3, norm_output, w1, w2, True)
+        dx, d_rms_norm_weight = F8.fused_rms_norm_ext_grad(x, norm_w, invar, d_norm_output, norm_eps)
+        slot = "main_grad" if hasattr(norm_w, "main_grad") else "grad"
+        if getattr(norm_w, slot, None) is None:
+            setattr(norm_w, slot, torch.zeros(norm_w.shape, dtype=torch.float32, device=norm_w.device))
+        getattr(norm_w, slot).add_(d_rms_norm_weight.reshape(norm_w.shape))
+        if hasattr(norm_w, "_apply_backward_hook"):
+            norm_w._apply_backward_hook()
+        return dx, norm_output, invar
+
+
+class FP8LinearFunction(torch.autograd.Function):
+    """fp8_utils.py:544-610.  custom_map carries `.weight` ([in, out] bf16).  keep_x saves the bf16
+    input and quantises it in backward; otherwise the transposed FP8 copy is saved.  The weight
+    gradient is accumulated into weight.main_grad / weight.grad, not returned."""
+
+    @staticmethod
+    def forward(ctx, x, custom_map, keep_x=False):
+        weight = custom_map.weight
+        x_orig_shape = x.shape
+        x = x.reshape([-1, x_orig_shape[-1]]).contiguous()
+        ctx.keep_x, ctx.weight, ctx.x_orig_shape = keep_x, weight, x_orig_shape
+        if keep_x:
+            out = FP8LinearFunctionBase.compute_fp8_linear(x, weight, weight_transpose=True, return_transpose_only=True)
+            ctx.saved = (x,)
+        else:
+            out, x_t_fp8, x_t_scale = FP8LinearFunctionBase.compute_fp8_linear(x, weight, weight_transpose=True, return_transpose_only=True,
+                                                                              return_mode="with_input_transpose_quant")
+            ctx.saved = (x_t_fp8, x_t_scale)
+        return out.reshape(*x_orig_shape[:-1], weight.shape[-1])
+
+    @staticmethod
+    def backward(ctx, dout):
+        weight = ctx.weight
+        dout_2d = dout.reshape([-1, dout.shape[-1]]).contiguous()
+        if ctx.keep_x:
+            x = FP8LinearFunctionBase.padding(ctx.saved[0], 0)
+            x_t_fp8, x_t_scale = F8.fp8_quant_blockwise(x, output_scale_transpose=True, quant_method="1x128", input_transpose=True,
+                                                        return_transpose_only=True)
+        else:
+            x_t_fp8, x_t_scale = ctx.saved
+        dx, dout_t_fp8, dout_t_scale = FP8LinearFunctionBase.compute_fp8_linear(dout_2d, weight, weight_transpose=False,
+                                                                                return_mode="with_input_transpose_quant")
+        FP8LinearFunctionBase.compute_expert_w_grad(x_t_fp8, x_t_scale, dout_t_fp8, dout_t_scale, True, True, weight, torch.float32)
+        return dx.reshape(ctx.x_orig_shape), None, None
+
+
+class FP8Linear(torch.nn.Module):
+    """fp8_utils.py:613-625: bias-free linear layer, weight [in, out] bf16, FP8 forward and backward."""
+
+    def __init__(self, in_features, out_features, bias_attr=False, device=None):
         super().__init__()
+        self.weight = torch.nn.Parameter(torch.empty(in_features, out_features, dtype=torch.bfloat16, device=device))
+        self.weight.main_grad = None   # fp32 accumulator of the weight gradient, created on first use
+
+    def forward(self, x):
+        return FP8LinearFunction.apply(x, self, False)
+
+
+class FP8KeepXLinear(FP8Linear):
+    """fp8_utils.py:668-684: same layer, keeps the bf16 input for backward; caches its FP8 weight."""
+
+    def fp8_quant_weight(self, quant_transpose=None):
+        cache_fp8_weight(self.weight, quant_transpose=quant_transpose)
+
+    def forward(self, x):
+        return FP8LinearFunction.apply(x, self, True)
+
+
+class FusedNormFP8MLPFunction(torch.autograd.Function):
+    """fp8_utils.py:687-741: RMSNorm + FP8 MLP; the norm output is kept, o1 is recomputed."""
+
+    @staticmethod
+    def forward(ctx, x, norm_w, w1, w2, norm_eps):
+        norm_output, invar = F8.fused_rms_norm_ext(x, norm_w, norm_eps)
+        x_orig_shape = norm_output.shape
+        norm_output = norm_output.reshape([-1, x_orig_shape[-1]])
+        o3 = FP8LinearFunctionBase.fp8_mlp_fwd(norm_output, w1, w2)[3]
+        if len(x_orig_shape) > 2:
+            o3 = o3.reshape([x_orig_shape[0], -1, o3.shape[-1]])
+        ctx.saved = (norm_output, invar, x, norm_w, w1, w2, norm_eps, x_orig_shape)
+        return o3
+
+    @staticmethod
+    def backward(ctx, do3):
+        do3 = do3.reshape([-1, do3.shape[-1]]).contiguous()
+        norm_output, invar, x, norm_w, w1, w2, norm_eps, x_orig_shape = ctx.saved
+        x_fp8, x_scale, x_t_fp8, x_t_scale = FP8LinearFunctionBase.padding_and_quant_input(norm_output)
+        d_norm_output, dw1, dw2 = FP8LinearFunctionBase.common_fp8_mlp_bwd(do3, x_t_fp8, x_t_scale, w1, w2, o1=None, x_fp8=x_fp8,
+                                                                           x_scale=x_scale)
+        d_norm_output = d_norm_output.reshape(x_orig_shape)
+        dx, d_rms_norm_weight = F8.fused_rms_norm_ext_grad(x, norm_w, invar, d_norm_output, norm_eps)
+        return dx, d_rms_norm_weight.to(norm_w.dtype), dw1.to(w1.dtype), dw2.to(w2.dtype), None
+
+
+class FP8MlpFunction(torch.autograd.Function):
+    """fp8_utils.py:744-803: FP8 MLP that saves the quantised input (and o1 unless it is to be
+    recomputed); weight gradients are accumulated into main_grad / grad, not returned."""
+
+    @staticmethod
+    def forward(ctx, x, w1, w2, recompute_fwd_gate_up):
+        x_orig_shape = x.shape
+        x = x.reshape([-1, x_orig_shape[-1]])
+        o1, x_fp8, x_scale, o3 = FP8LinearFunctionBase.fp8_mlp_fwd(x, w1, w2)
+        if len(x_orig_shape) > 2:
+            o3 = o3.reshape([x_orig_shape[0], -1, o3.shape[-1]])
+        ctx.saved = (None if recompute_fwd_gate_up else o1, x_fp8, x_scale, w1, w2, x_orig_shape)
+        return o3
+
+    @staticmethod
+    def backward(ctx, do3):
+        do3 = do3.reshape([-1, do3.shape[-1]]).contiguous()
+        o1, x_fp8, x_scale, w1, w2, x_orig_shape = ctx.saved
+        x_dequant = F8.fused_act_dequant(x_fp8, x_scale.T.contiguous())
+        x_dequant = FP8LinearFunctionBase.padding(x_dequant, 0)
+        x_t_fp8, x_t_scale = F8.fp8_quant_blockwise(x_dequant, output_scale_transpose=True, quant_method="1x128", input_transpose=True,
+                                                    return_transpose_only=True)
+        if o1 is None:
+            dx = FP8LinearFunctionBase.common_fp8_mlp_bwd(do3, x_t_fp8, x_t_scale, w1, w2, o1=None, x_fp8=x_fp8, x_scale=x_scale,
+                                                          apply_backward_hook=True)
+        else:
+            dx = FP8LinearFunctionBase.common_fp8_mlp_bwd(do3, x_t_fp8, x_t_scale, w1, w2, o1=o1, x_fp8=None, x_scale=None,
+                                                          apply_backward_hook=True)
+        return dx.reshape(x_orig_shape), None, None, None
+
+
+class FP8Mlp(torch.nn.Module):
+    """fp8_utils.py:806-850: SwiGLU MLP with w1 [H, 2I] and w2 [I, H] in bf16, FP8 forward and
+    backward; optionally fused with the preceding RMSNorm (using_post_norm_recompute)."""
+
+    def __init__(self, hidden_size, intermediate_size, device=None, using_post_norm_recompute=False, norm_weight=None, norm_eps=None,
+                 recompute_fwd_gate_up=False):
+        super().__init__()
+        self.using_post_norm_recompute = using_post_norm_recompute
+        if using_post_norm_recompute:
+            assert norm_weight is not None and norm_eps is not None
+            self.norm_weight, self.norm_eps = norm_weight, norm_eps
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.recompute_fwd_gate_up = recompute_fwd_gate_up
         self.w1 = torch.nn.Parameter(torch.empty(hidden_size, intermediate_size * 2, dtype=torch.bfloat16, device=device))
         self.w2 = torch.nn.Parameter(torch.empty(intermediate_size, hidden_size, dtype=torch.bfloat16, device=device))
+        self.w1.main_grad = None       # fp32 accumulators of the weight gradients, created on first use
+        self.w2.main_grad = None
 
     def fp8_quant_weight(self, quant_transpose=None):
         cache_fp8_weight(self.w1, quant_transpose)
         cache_fp8_weight(self.w2, quant_transpose)
 
-    @torch.no_grad()
     def forward(self, x):
-        return FP8LinearFunctionBase.fp8_mlp_fwd(x, self.w1, self.w2)[3]
+        if self.using_post_norm_recompute:
+            return FusedNormFP8MLPFunction.apply(x, self.norm_weight, self.w1, self.w2, self.norm_eps)
+        return FP8MlpFunction.apply(x, self.w1, self.w2, self.recompute_fwd_gate_up)
 
 
 class FP8GroupGemmMlpFunctionNode:

@@ -451,6 +451,63 @@ def swiglu(x: torch.Tensor, y: Optional[torch.Tensor] = None) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------------------------
+# swiglu_grad, fused_rms_norm_ext(+grad): the remaining operators of the dense FP8 MLP backward
+# ---------------------------------------------------------------------------------------------
+
+
+def swiglu_grad(o1: torch.Tensor, y, do2: torch.Tensor):
+    """paddle._C_ops.swiglu_grad(o1, None, do2) as the dense MLP backward calls it
+    (transformers/fp8_utils.py:407): gradient of swiglu(o1) with the two halves packed in o1.
+    Returns (do1, None).  Runs the weighted kernel with unit probabilities (bf16(do2 * 1) == do2)."""
+    if y is not None:
+        raise ValueError("swiglu_grad supports the packed form only (y must be None)")
+    o2d = _as2d(o1)
+    ones = torch.ones((o2d.shape[0],), dtype=torch.float32, device=o1.device)
+    do1, _, _ = fused_swiglu_weighted_bwd(o2d, _as2d(do2), ones)
+    return do1.reshape(o1.shape), None
+
+
+def fused_rms_norm_ext(x: torch.Tensor, norm_weight: torch.Tensor, epsilon: float):
+    """paddle.incubate.nn.functional.fused_rms_norm_ext(x, norm_w, eps) -> (y, invvar)
+    (transformers/fp8_utils.py:472, 522, 691).  x bf16 [..., H], norm_weight bf16 [H];
+    y = bf16(x * invvar * w) with invvar fp32 [rows] = 1/sqrt(mean(x^2) + eps)."""
+    _dev(x, "x")
+    _dev(norm_weight, "norm_weight")
+    if x.dtype != torch.bfloat16 or norm_weight.dtype != torch.bfloat16:
+        raise ValueError("x and norm_weight must be bfloat16")
+    H = x.shape[-1]
+    if norm_weight.numel() != H or H % 8 != 0:
+        raise ValueError("norm_weight must have one entry per column and the width must be a multiple of 8")
+    x2 = _as2d(x).contiguous()
+    M = x2.shape[0]
+    y = torch.empty_like(x2)
+    invar = torch.empty((M,), dtype=torch.float32, device=x.device)
+    _lib.call("pf8_rms_norm_fwd", _p(x2), _p(norm_weight.contiguous()), C.c_float(float(epsilon)), M, H, _p(y), _p(invar), _stream())
+    return y.reshape(x.shape), invar.reshape(x.shape[:-1])
+
+
+def fused_rms_norm_ext_grad(x: torch.Tensor, norm_weight: torch.Tensor, invvar: torch.Tensor, dy: torch.Tensor, epsilon: float):
+    """paddle._C_ops.fused_rms_norm_ext_grad(x, norm_w, invvar, dy, eps) -> (dx bf16, dw fp32 [H])
+    (transformers/fp8_utils.py:528, 739)."""
+    for t, n in ((x, "x"), (norm_weight, "norm_weight"), (invvar, "invvar"), (dy, "dy")):
+        _dev(t, n)
+    if x.dtype != torch.bfloat16 or dy.dtype != torch.bfloat16 or norm_weight.dtype != torch.bfloat16:
+        raise ValueError("x, dy and norm_weight must be bfloat16")
+    H = x.shape[-1]
+    x2, d2 = _as2d(x).contiguous(), _as2d(dy).contiguous()
+    if x2.shape != d2.shape:
+        raise ValueError("x and dy must have the same shape")
+    M = x2.shape[0]
+    iv = invvar.reshape(-1).float().contiguous()
+    if iv.numel() != M:
+        raise ValueError("invvar must have one entry per row")
+    dx = torch.empty_like(x2)
+    dw = torch.zeros((H,), dtype=torch.float32, device=x.device)
+    _lib.call("pf8_rms_norm_bwd", _p(x2), _p(norm_weight.contiguous()), _p(iv), _p(d2), M, H, _p(dx), _p(dw), _stream())
+    return dx.reshape(x.shape), dw
+
+
+# ---------------------------------------------------------------------------------------------
 # moe_permute / moe_unpermute (paddle.nn.functional in the reference)
 # ---------------------------------------------------------------------------------------------
 
