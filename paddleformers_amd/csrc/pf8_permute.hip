@@ -16,35 +16,39 @@ struct PermuteArgs {
 
 // One workgroup per expert: rank the tokens routed to it (stable in token order) with wave ballots
 // and a running offset, fill its column of the row map, clear its padding rows' probabilities.
-__global__ __launch_bounds__(256) void k_permute_rowmap(const int32_t* __restrict__ routemap, int64_t T, int topk, PermuteArgs pa,
+__global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restrict__ routemap, int64_t T, int topk, PermuteArgs pa,
                                                         int32_t* __restrict__ rowmap, float* __restrict__ out_probs,
                                                         int32_t* __restrict__ overflow) {
-    __shared__ int wave_cnt[4];
+    __shared__ int wave_cnt[2][16];    // double-buffered: one barrier per step
     const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int E = pa.E;
     int64_t base = pa.row_start[e];
     const int64_t limit = base + pa.count[e];
-    for (int64_t t0 = 0; t0 < T; t0 += 256) {
+    int buf = 0;
+    for (int64_t t0 = 0; t0 < T; t0 += 1024, buf ^= 1) {
         const int64_t t = t0 + tid;
         bool hit = false;
         if (t < T)
             for (int k = 0; k < topk; ++k) hit |= routemap[t * topk + k] == e;
         const uint64_t m = __ballot(hit);
-        if (lane == 0) wave_cnt[wave] = __popcll(m);
+        if (lane == 0) wave_cnt[buf][wave] = __popcll(m);
         __syncthreads();
-        int before = __popcll(m & ((1ull << lane) - 1ull));
-        for (int w = 0; w < wave; ++w) before += wave_cnt[w];
-        const int total = wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
+        int before = __popcll(m & ((1ull << lane) - 1ull)), total = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            const int c = wave_cnt[buf][w];
+            before += w < wave ? c : 0;
+            total += c;
+        }
         if (t < T) {
             int64_t row = hit ? base + before : -1;
             if (row >= limit) { row = -1; *overflow = 1; }      // more routed rows than tokens_per_expert says
             rowmap[t * E + e] = (int32_t)row;
         }
         base += total;
-        __syncthreads();
     }
     if (out_probs)
-        for (int64_t r = limit + tid; r < pa.row_start[e + 1]; r += 256) out_probs[r] = 0.0f;
+        for (int64_t r = limit + tid; r < pa.row_start[e + 1]; r += 1024) out_probs[r] = 0.0f;
 }
 
 // One workgroup per padding row: zero the row of tokens (and of scales).
@@ -165,7 +169,7 @@ extern "C" int pf8_moe_permute(const void* x, int x_is_fp8, const float* xs, con
     PF8_REQUIRE(T == 0 || (x && routemap && PF8_ALIGNED16(x)), "null or misaligned input");
     hipStream_t st = (hipStream_t)stream;
     const int64_t scale_cols = xs ? H / 128 : 0;
-    hipLaunchKernelGGL(k_permute_rowmap, dim3(E), dim3(256), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
+    hipLaunchKernelGGL(k_permute_rowmap, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
     int rc = pf8_check_launch(__func__);
     if (rc) return rc;
     if (max_pad > 0 && row_bytes > 0) {
