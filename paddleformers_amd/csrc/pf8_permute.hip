@@ -19,33 +19,48 @@ struct PermuteArgs {
 __global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restrict__ routemap, int64_t T, int topk, PermuteArgs pa,
                                                         int32_t* __restrict__ rowmap, float* __restrict__ out_probs,
                                                         int32_t* __restrict__ overflow) {
-    __shared__ int wave_cnt[2][16];    // double-buffered: one barrier per step
+    // every thread ranks J tokens per step (token = step base + j * 1024 + tid, so rank order is
+    // j-major): the J x topk loads of a step are in flight together and a step costs one barrier
+    constexpr int J = 4;
+    __shared__ int wave_cnt[2][J][16];    // double-buffered: one barrier per step
     const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int E = pa.E;
     int64_t base = pa.row_start[e];
     const int64_t limit = base + pa.count[e];
     int buf = 0;
-    for (int64_t t0 = 0; t0 < T; t0 += 1024, buf ^= 1) {
-        const int64_t t = t0 + tid;
-        bool hit = false;
-        if (t < T)
-            for (int k = 0; k < topk; ++k) hit |= routemap[t * topk + k] == e;
-        const uint64_t m = __ballot(hit);
-        if (lane == 0) wave_cnt[buf][wave] = __popcll(m);
-        __syncthreads();
-        int before = __popcll(m & ((1ull << lane) - 1ull)), total = 0;
+    for (int64_t t0 = 0; t0 < T; t0 += 1024 * J, buf ^= 1) {
+        bool hit[J];
+        uint64_t m[J];
 #pragma unroll
-        for (int w = 0; w < 16; ++w) {
-            const int c = wave_cnt[buf][w];
-            before += w < wave ? c : 0;
-            total += c;
+        for (int j = 0; j < J; ++j) {
+            const int64_t t = t0 + j * 1024 + tid;
+            hit[j] = false;
+            if (t < T)
+                for (int k = 0; k < topk; ++k) hit[j] |= routemap[t * topk + k] == e;
         }
-        if (t < T) {
-            int64_t row = hit ? base + before : -1;
-            if (row >= limit) { row = -1; *overflow = 1; }      // more routed rows than tokens_per_expert says
-            rowmap[t * E + e] = (int32_t)row;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            m[j] = __ballot(hit[j]);
+            if (lane == 0) wave_cnt[buf][j][wave] = __popcll(m[j]);
         }
-        base += total;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            int before = __popcll(m[j] & ((1ull << lane) - 1ull)), total = 0;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) {
+                const int c = wave_cnt[buf][j][w];
+                before += w < wave ? c : 0;
+                total += c;
+            }
+            const int64_t t = t0 + j * 1024 + tid;
+            if (t < T) {
+                int64_t row = hit[j] ? base + before : -1;
+                if (row >= limit) { row = -1; *overflow = 1; }      // more routed rows than tokens_per_expert says
+                rowmap[t * E + e] = (int32_t)row;
+            }
+            base += total;
+        }
     }
     if (out_probs)
         for (int64_t r = limit + tid; r < pa.row_start[e + 1]; r += 1024) out_probs[r] = 0.0f;
