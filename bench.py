@@ -214,7 +214,42 @@ def bench_other_gemms(iters=10, warmup=3):
     out["moe_permute_config5"] = {"bytes": Tt * Ht * 2 + ux.numel() * 2, "ms": ms}
     ms = time_kernel(lambda: F8.moe_unpermute(ux, rowmap, rm_t, up, Tt, Et), [()], 5, 2)
     out["moe_unpermute_config5"] = {"bytes": Tt * tk * Ht * 2 + Tt * Ht * 2, "ms": ms}
-    del xt, ux
+    del xt, ux, rowmap, up
+    torch.cuda.empty_cache()
+    # the fused FP8 MoE node end to end at config 5: forward + backward (dgrad and wgrad, both GEMMs),
+    # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers
+    from paddleformers_amd import fp8_utils as U8
+
+    class _Ex:
+        pass
+
+    class _Mp:
+        pass
+
+    g1 = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
+    g2 = torch.zeros((E, I, H), dtype=torch.float32, device="cuda")
+    exps = []
+    for e in range(E):
+        ex = _Ex()
+        ex.w1 = (torch.randn((H, 2 * I), device="cuda") * 0.02).to(torch.bfloat16)
+        ex.w2 = (torch.randn((I, H), device="cuda") * 0.02).to(torch.bfloat16)
+        ex.w1.main_grad, ex.w2.main_grad = g1[e], g2[e]
+        exps.append(ex)
+    U8.fp8_quant_weight([ex.w1 for ex in exps], [ex.w2 for ex in exps], batch_mode=True)
+    mp = _Mp()
+    mp.experts = exps
+    node = U8.FP8GroupGemmMlpFunctionNode(mp)
+    xin = torch.randn((Mp, H), device="cuda").to(torch.bfloat16)
+    dout = (torch.randn((Mp, H), device="cuda") * 1e-3).to(torch.bfloat16)
+    pr = torch.rand((Mp, 1), device="cuda")
+
+    def fwd_bwd():
+        node.forward(xin, pr, rows)
+        node.backward(dout, pr, rows, reset_status=True)
+
+    ms = time_kernel(fwd_bwd, [()], 3, 2)
+    out["moe_node_config5_fwd_bwd"] = {"flop": 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H), "ms": ms}
+    del node, exps, g1, g2, xin, dout
     for v in out.values():
         if "flop" in v:
             v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)

@@ -679,9 +679,35 @@ class FP8GroupGemmMlpFunctionNode:
         return F8.fused_transpose_split_quant(x, scale, tokens_per_expert, pow_2_scales)
 
     @staticmethod
+    def _stacked_main_grad(expert_w):
+        """The experts' fp32 main_grad tensors as one [E, K, N] tensor when they sit back to back in
+        memory (slices of one buffer), else None."""
+        grads = [getattr(w, "main_grad", None) for w in expert_w]
+        g0 = grads[0]
+        if g0 is None or g0.dtype != torch.float32 or not g0.is_contiguous() or g0.dim() != 2:
+            return None
+        step = g0.numel() * 4
+        for e, g in enumerate(grads):
+            if g is None or g.shape != g0.shape or g.dtype != torch.float32 or not g.is_contiguous() or \
+                    g.data_ptr() != g0.data_ptr() + e * step:
+                return None
+        if g0.untyped_storage().nbytes() - g0.storage_offset() * 4 < len(grads) * step:
+            return None
+        K, N = g0.shape
+        return torch.as_strided(g0, (len(grads), K, N), (K * N, N, 1))
+
+    @staticmethod
     def _expert_wgrads(a_t, sa_t, b_t, sb_t, expert_w):
-        """Per-expert loop of fp8_utils.py:1117-1129 / :1170-1182."""
+        """The per-expert loop of fp8_utils.py:1117-1129 / :1170-1182.  When the experts' main_grad
+        tensors are slices of one [E, K, N] buffer, all experts run in one grouped launch."""
         with torch.no_grad():
+            stacked = FP8GroupGemmMlpFunctionNode._stacked_main_grad(expert_w) if len(expert_w) > 1 else None
+            if stacked is not None:
+                F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, stacked, accumulate=True)
+                for w in expert_w:
+                    if hasattr(w, "_apply_backward_hook"):
+                        w._apply_backward_hook()
+                return
             for i in range(len(expert_w)):
                 FP8LinearFunctionBase.compute_expert_w_grad(a_t[i], sa_t[i], b_t[i], sb_t[i], True, True, expert_w[i], torch.float32)
 

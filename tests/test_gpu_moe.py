@@ -180,3 +180,38 @@ def test_moe_backward_stages_against_oracle():
     e = 1
     exp = O.gemm_nt_1d1d_f32(G.from_torch_fp8(a_t[e]), sa_t[e].cpu().numpy(), G.from_torch_fp8(b_t[e]), sb_t[e].cpu().numpy())
     assert G.rel_fro(experts[e].w2.main_grad.cpu().numpy(), exp) <= 5e-5
+
+
+def test_moe_backward_grouped_wgrad_when_main_grads_are_stacked():
+    """Experts whose main_grad tensors are slices of one buffer get their weight gradients from one
+    grouped launch; the result equals the per-expert loop."""
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 4, 512, 256
+    rows = [256, 0, 128, 384]
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=21)
+    dout = G.bf16_normal((sum(rows), H), seed=22, std=1e-3)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    # reference: separate main_grad tensors (allocated on first use), per-expert loop
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts))
+    node.forward(G.to_torch_bf16(x), tp, rows)
+    dx_ref, pg_ref = node.backward(G.to_torch_bf16(dout), tp, rows)
+    ref1 = [e.w1.main_grad for e in experts]
+    ref2 = [e.w2.main_grad for e in experts]
+    # stacked buffers
+    g1 = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
+    g2 = torch.zeros((E, I, H), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        experts[e].w1.main_grad, experts[e].w2.main_grad = g1[e], g2[e]
+    assert FP8GroupGemmMlpFunctionNode._stacked_main_grad([e.w1 for e in experts]) is not None
+    node.forward(G.to_torch_bf16(x), tp, rows)
+    dx, pg = node.backward(G.to_torch_bf16(dout), tp, rows)
+    assert torch.equal(dx, dx_ref) and torch.equal(pg, pg_ref)
+    for e in range(E):
+        if rows[e] == 0:
+            assert ref1[e] is None and not g1[e].any() and not g2[e].any()
+        else:
+            assert torch.equal(g1[e], ref1[e]) and torch.equal(g2[e], ref2[e])
+    # not stacked: one expert's gradient lives elsewhere
+    experts[2].w1.main_grad = torch.zeros((H, 2 * I), dtype=torch.float32, device="cuda")
+    assert FP8GroupGemmMlpFunctionNode._stacked_main_grad([e.w1 for e in experts]) is None
