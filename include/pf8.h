@@ -185,6 +185,27 @@ int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_lay
                                    const float* sb, int E, int64_t Mtot, int64_t N, int64_t K,
                                    const int32_t* m_indices, uint16_t* out, pf8_stream_t stream);
 
+/* The same two GEMMs with power-of-two scales held as UE8M0 exponent bytes (scale = 2^(byte-127)),
+ * the form `use_ue8m0` selects for deep_gemm (transformers/configuration_utils.py:454-459; byte
+ * format quantization/checkpoint_dequant.py:121-131).  Both operands must have been quantized with
+ * pow2 scales (using_pow2_scale=True).  sa u8 [K/128, ldsa] (1x128 scales, K-block major, ldsa >= M
+ * and a multiple of 8); sb u8 [N/128, K/128] ([E, N/128, K/128] grouped), read as whole aligned
+ * dwords.  M (Mtot) multiple of 128, N multiple of 256, K multiple of 128 and >= 384, ldo multiple
+ * of 8; other shapes return PF8_EINVAL (decode the scales and use the fp32-scale entry points). */
+int pf8_gemm_nt_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b,
+                      const uint8_t* sb, int64_t M, int64_t N, int64_t K, uint16_t* out, int64_t ldo,
+                      pf8_stream_t stream);
+int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa,
+                                         const uint8_t* b, const uint8_t* sb, int E, int64_t Mtot,
+                                         int64_t N, int64_t K, const int32_t* m_indices, uint16_t* out,
+                                         pf8_stream_t stream);
+
+/* fp32 scales that are powers of two -> UE8M0 exponent bytes, elementwise (any layout).  not_pow2,
+ * when non-null, is a DEVICE int the kernel adds the number of scales to that are negative, zero,
+ * non-finite or not a power of two (the caller zeroes it).  Scale side of `use_ue8m0`
+ * (transformers/configuration_utils.py:454-459). */
+int pf8_scales_to_ue8m0(const float* s, int64_t n, uint8_t* out, int* not_pow2, pf8_stream_t stream);
+
 /* deep_gemm.m_grouped_fp8_gemm_nt_masked((a, sa), (b, sb), out, masked_m, expected_m) --
  * ernie token_dispatcher/fp8_utils.py:227-233.  a [E,Mmax,K], sa [E,Mmax,K/128] row-major,
  * b [E,N,K], sb [E,ceil(N/128),K/128], masked_m DEVICE int32 [E] valid rows -> out [E,Mmax,N];

@@ -6,9 +6,11 @@ benchmark.  The product package never imports it.
 bf16 tensors are numpy uint16 bit patterns, e4m3 tensors are numpy uint8 codes, scales float32.
 Each wrapper names the C function it calls; the reference citations live in pf8_oracle.c.
 
-Two restatements at the end of this file are plain numpy, not C:
+A few restatements at the end of this file are plain numpy, not C:
   block_dequant              pinned by the reference's own known-answer vectors
                              (tests/test_oracle_dequant.py)
+  scales_to_ue8m0            pinned as the inverse of the UE8M0 decode table above, itself pinned by
+                             those vectors (tests/test_oracle_dequant.py)
   moe_permute / moe_unpermute  PARITY UNPINNED: no test, fixture or importable implementation of
                              the operators exists in the reference; checked only against the
                              invariants their call sites rely on (tests/test_oracle_ops.py)
@@ -363,6 +365,16 @@ def decode_scales(scale: np.ndarray, scale_format: str) -> np.ndarray:
     if fmt in ("bf16", "bfloat16"):
         return bf16_bits_to_f32(scale)
     return scale.astype(np.float32)
+
+
+def scales_to_ue8m0(scale: np.ndarray) -> np.ndarray:
+    """fp32 powers of two -> UE8M0 exponent bytes (the biased exponent field of the float).  Inverse
+    of decode_scales(..., "ue8m0"), whose table follows quantization/checkpoint_dequant.py:121-131;
+    the CPU tests pin it by that round trip over every finite exponent."""
+    bits = np.ascontiguousarray(scale, dtype=np.float32).view(np.uint32)
+    if np.any(bits & np.uint32(0x807FFFFF)):
+        raise ValueError("scale is not a positive power of two")
+    return (bits >> np.uint32(23)).astype(np.uint8)
 
 
 def block_dequant(q: np.ndarray, scale: np.ndarray, scale_format: str, block_axes, block_shape, out: str = "f32") -> np.ndarray:

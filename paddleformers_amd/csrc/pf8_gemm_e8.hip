@@ -1,0 +1,416 @@
+// pf8_gemm_e8.hip -- FP8 GEMMs whose block scales are powers of two, stored as UE8M0 exponent bytes
+// (scale = 2^(byte - 127)): the forward / dgrad GEMM of the path when every operand was quantized
+// with pow2 scales.  gfx950's block-scaled MFMA (v_mfma_scale_f32_16x16x128_f8f6f4) applies both
+// operands' scales inside the instruction, so a K block's product is accumulated by the matrix pipe
+// itself instead of being folded in by vector FMAs.  That removes the product registers and the
+// VALU work of the fp32-scale kernels and lets the accumulator tile fill the whole AGPR file.
+//
+// Geometry: 256(Q, output rows) x 256(P, output columns) x 128(K) blocks, 256 threads = 4 wavefronts
+// (2 along Q x 2 along P), each owning 128 x 128 = 8 x 8 MFMA tiles = 256 accumulator registers.
+// Per K block a compute unit moves 64 KB L2 -> LDS and reads 128 KB of fragments for 256 MFMAs:
+// two thirds of the LDS traffic per MFMA of the 128 x 256 fp32-scale kernels.
+//   * One persistent workgroup per compute unit; 128 KB of LDS is two slots of [P 32 KB | Q 32 KB].
+//     The P fragments of a block (64 registers) are read once, behind the previous block's barrier,
+//     and held; the Q fragments stream through a ring of four, three ahead of their MFMAs.
+//   * One barrier per block, before MFMA 44 of 64: by then every fragment read of the block has
+//     been issued, so the slot is free, and the wavefront's copies of the next block have landed.
+//     Behind it the copies of the block after next go into the freed slot, one between every other
+//     MFMA, running on into the next block; the ring runs on across tile boundaries.
+//   * The accumulator tile IS the AGPR file: element (i, j) lives in a[4(8i+j) .. +3], named
+//     literally in every instruction that touches it, so the register allocator never sees it
+//     (left to the allocator, the tile gets split between both register files and copied back and
+//     forth).  One empty statement that clobbers a255 makes the kernel descriptor reserve all 256.
+//   * Q row r of a wavefront's fragment j is row 8 (r) + j of its 128, so the eight scale bytes a lane
+//     needs per block are contiguous (one 8-byte load) and op_sel picks the byte per MFMA.
+//   * A 256-row tile of the contiguous grouped layout may hold two experts (segments are padded to
+//     128 rows): such a tile is walked twice, once per expert, each pass storing its own half.
+#include <type_traits>
+
+#include "pf8_device.h"
+#include "pf8_host.h"
+
+namespace pf8 {
+
+struct E8Args {
+    const uint8_t* p;      // [E][Prows, red]  weights: output columns
+    const uint8_t* q;      // [Qrows, red]     activations: output rows
+    const uint8_t* sp8;    // [E][Prows/128, KB] exponent bytes
+    const uint8_t* sq8;    // [KB, ldsq] exponent bytes (1x128 scales, K-block major)
+    void* out;             // bf16 [Qrows, ldo]
+    int64_t Prows, Qrows, red, ldo, ldsq;
+    int grouped;
+    const int32_t* m_indices;
+};
+
+__device__ __forceinline__ int e8_keyp(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// 16 bytes per lane global -> LDS, scalar base + 32-bit lane offset; tracked by vmcnt only
+__device__ __forceinline__ void e8_dma16(uint32_t voff, const uint8_t* sbase, uint32_t lds_dst) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase), "s"(lds_dst) : "memory");
+}
+__device__ __forceinline__ i32x8 e8_frag(const uint8_t* p0, const uint8_t* p1) {
+    i32x4 lo = *reinterpret_cast<const i32x4*>(p0);
+    i32x4 hi = *reinterpret_cast<const i32x4*>(p1);
+    return (i32x8){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+}
+
+// acc[IDX] += (2^(sa-127) A) (2^(sb.byte[OB]-127) B): A = P fragment (one scale per block), B = Q fragment
+template <int IDX, int OB>
+__device__ __forceinline__ void e8_mfma(const i32x8& a, const i32x8& b, int sa, int sb) {
+    if constexpr (OB == 0) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel_hi:[0,0,0]" : : "v"(a), "v"(b), "v"(sa), "v"(sb), "n"(4 * IDX), "n"(4 * IDX + 3));
+    if constexpr (OB == 1) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel:[0,1,0] op_sel_hi:[0,0,0]" : : "v"(a), "v"(b), "v"(sa), "v"(sb), "n"(4 * IDX), "n"(4 * IDX + 3));
+    if constexpr (OB == 2) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel_hi:[0,1,0]" : : "v"(a), "v"(b), "v"(sa), "v"(sb), "n"(4 * IDX), "n"(4 * IDX + 3));
+    if constexpr (OB == 3) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel:[0,1,0] op_sel_hi:[0,1,0]" : : "v"(a), "v"(b), "v"(sa), "v"(sb), "n"(4 * IDX), "n"(4 * IDX + 3));
+}
+template <int IDX>
+__device__ __forceinline__ void e8_acc_zero4() {
+    asm volatile("v_accvgpr_write_b32 a[%0], 0\n\tv_accvgpr_write_b32 a[%1], 0\n\tv_accvgpr_write_b32 a[%2], 0\n\tv_accvgpr_write_b32 a[%3], 0"
+                 : : "n"(4 * IDX), "n"(4 * IDX + 1), "n"(4 * IDX + 2), "n"(4 * IDX + 3));
+}
+template <int R>
+__device__ __forceinline__ float e8_acc_get() {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v) : "n"(R));
+    return v;
+}
+template <int N, typename F>
+__device__ __forceinline__ void e8_static_for(F&& f) {
+    if constexpr (N > 0) {
+        e8_static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+__global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
+    constexpr int SLOT = 65536, Q_OFS = 32768, EP_OFS = 131072, EP_LD = 272;
+    constexpr int BAR = 44, CSTEP = 2;     // barrier position; MFMAs between two copies
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    asm volatile("" ::: "a255");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wq = wave >> 1, wp = wave & 1;
+    const int li = lane & 15, kg = lane >> 4;
+
+    const int64_t p_tiles = a.Prows / 256, q_tiles = (a.Qrows + 255) / 256;
+    const int64_t T = p_tiles * q_tiles;
+    // consecutive workgroups go round-robin to the 8 XCDs: every XCD owns a contiguous run of
+    // logical tiles (groups of 8 q-tiles x all p-tiles), walked W tiles at a time by its W workgroups
+    const int64_t per_xcd = (T + 7) / 8;
+    const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, W = gridDim.x >> 3;
+    const int64_t KB = a.red / 128, PB = a.Prows / 128;
+
+    auto tile_coords = [&](int64_t n, int64_t& q_tile, int64_t& p_tile) -> bool {
+        constexpr int G = 8;
+        const int64_t loc = slot + n * W, logical = xcd * per_xcd + loc;
+        if (loc >= per_xcd || logical >= T) return false;
+        const int64_t grp = logical / (G * p_tiles), rem = logical % (G * p_tiles);
+        const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;
+        q_tile = grp * G + rem % gq;
+        p_tile = rem / gq;
+        return true;
+    };
+    // which expert's weights a tile multiplies and which 128-row halves it stores.  A half of padding
+    // rows (index < 0) or past the end stores nothing; two different experts need a second pass.
+    auto classify = [&](int e0, int e1, int& e, int& mask, int& second_e) {
+        second_e = -1;
+        if (e0 < 0 && e1 < 0) { e = 0; mask = 0; }
+        else if (e0 < 0) { e = e1; mask = 2; }
+        else if (e1 < 0 || e0 == e1) { e = e0; mask = e1 < 0 ? 1 : 3; }
+        else { e = e0; mask = 1; second_e = e1; }
+    };
+    auto has_tail = [&](int64_t qt) -> bool { return qt * 256 + 128 >= a.Qrows; };
+
+    // work item = (tile, expert, halves to store); c_* current, n_* next; all wave-uniform
+    int64_t cq = 0, cp = 0, nq = 0, np = 0, tn = 0;
+    if (!tile_coords(0, cq, cp)) return;
+    int c_e, c_mask, c_second, n_mask = 0, n_second = -1;
+    {
+        int e0 = 0, e1 = has_tail(cq) ? -1 : 0;
+        if (a.grouped) {
+            e0 = a.m_indices[cq * 256];
+            if (!has_tail(cq)) e1 = a.m_indices[cq * 256 + 128];
+        }
+        classify(e0, e1, c_e, c_mask, c_second);
+    }
+    int ld_e0 = 0, ld_e1 = 0;      // expert ids of the next tile's halves, loaded one block before they are used
+    const uint8_t *c_ptile, *c_qtile, *c_qtile2, *c_sq, *c_sp;
+    auto setup = [&](int64_t qt, int64_t pt, int e, const uint8_t*& ptile, const uint8_t*& qtile, const uint8_t*& qtile2,
+                     const uint8_t*& sq, const uint8_t*& sp) {
+        const bool tail = has_tail(qt);
+        ptile = a.p + ((int64_t)e * a.Prows + pt * 256) * a.red;
+        qtile = a.q + qt * 256 * a.red;
+        qtile2 = tail ? qtile : qtile + 128 * a.red;     // a missing second half re-reads the first
+        sq = a.sq8 + qt * 256 + ((wq && !tail) ? 128 : 0);
+        sp = a.sp8 + ((int64_t)e * PB + pt * 2 + wp) * KB;
+    };
+    setup(cq, cp, c_e, c_ptile, c_qtile, c_qtile2, c_sq, c_sp);
+    const uint8_t *n_ptile = c_ptile, *n_qtile = c_qtile, *n_qtile2 = c_qtile2, *n_sq = c_sq, *n_sp = c_sp;
+    bool n_valid = false;
+
+    // copy c of a wavefront fills rows (4 c + wave) * 8 + (lane >> 3) of the stacked [P; Q] block.  P rows
+    // are swizzled by e8_keyp(row), Q rows by (row >> 3) & 7: a Q fragment's 16 lanes read rows 8 apart
+    const int crow = lane >> 3, cpos = lane & 7;
+    const uint32_t c_off_p = (uint32_t)((wave * 8 + crow) * a.red + ((cpos ^ e8_keyp(wave * 8 + crow)) << 4));
+    uint32_t c_off_q[2];
+#pragma unroll
+    for (int par = 0; par < 2; ++par) c_off_q[par] = (uint32_t)((wave * 8 + crow) * a.red + ((cpos ^ (4 * par + wave)) << 4));
+    const int64_t copy_step = 32 * a.red;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+    int fp_ofs[2], fq_ofs[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int prow = wp * 128 + li;
+        fp_ofs[h] = prow * 128 + (((2 * kg + h) ^ e8_keyp(prow)) << 4);
+        fq_ofs[h] = Q_OFS + (wq * 128 + li * 8) * 128 + (((2 * kg + h) ^ (li & 7)) << 4);
+    }
+    const uint32_t s_off = (uint32_t)(li * 8);
+
+#define E8_COPY(c_, pt_, qt_, qt2_, slot_)                                                             \
+    do {                                                                                               \
+        if ((c_) < 8) e8_dma16(c_off_p, (pt_) + (c_) * copy_step, lds_base + (slot_) * SLOT + ((c_) * 4 + wave) * 1024); \
+        else if ((c_) < 12) e8_dma16(c_off_q[(c_) & 1], (qt_) + ((c_) - 8) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
+        else e8_dma16(c_off_q[(c_) & 1], (qt2_) + ((c_) - 12) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
+    } while (0)
+    // the scale bytes of a block: eight Q exponents per lane, and the aligned dword that holds the P
+    // block's exponent (extracted when the block starts)
+#define E8_LOAD_S(sq_, sp_)                                                                            \
+    do {                                                                                               \
+        asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(sq_nxt) : "v"(s_off), "s"(sq_) : "memory"); \
+        const uintptr_t spa_ = reinterpret_cast<uintptr_t>(sp_);                                       \
+        asm volatile("s_load_dword %0, %1, 0x0" : "=s"(sp_nxt) : "s"(spa_ & ~(uintptr_t)3) : "memory"); \
+        sp_sh_nxt = (uint32_t)(spa_ & 3) * 8;                                                          \
+    } while (0)
+
+    i32x8 pf[2][8], qf[4];
+    u32x2 sq_nxt = {0, 0};
+    uint32_t sp_nxt = 0, sp_sh_nxt = 0;
+
+    e8_static_for<64>([&](auto ix) { e8_acc_zero4<decltype(ix)::value>(); });
+    {
+        E8_LOAD_S(c_sq, c_sp);
+#pragma unroll
+        for (int c = 0; c < 16; ++c) E8_COPY(c, c_ptile, c_qtile, c_qtile2, 0);
+#pragma unroll
+        for (int c = 0; c < 16; ++c)
+            if (c * CSTEP < 64 - BAR) E8_COPY(c, c_ptile + 128, c_qtile + 128, c_qtile2 + 128, 1);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(sq_nxt), "+s"(sp_nxt) : : "memory");
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pf[0][i] = e8_frag(lds + fp_ofs[0] + i * 2048, lds + fp_ofs[1] + i * 2048);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) qf[j] = e8_frag(lds + fq_ofs[0] + j * 128, lds + fq_ofs[1] + j * 128);
+    }
+    int64_t kb = 0;
+
+    // one K block; PAR = parity of the block in this workgroup's stream of blocks = its LDS slot and
+    // the half of pf[] that holds its P fragments.  Returns true after the last work item.
+    auto blk = [&](auto par_c) -> bool {
+        constexpr int PAR = decltype(par_c)::value;
+        if (kb == 0) {
+            // the item after this one: the same tile again for its second expert, or the next tile, whose
+            // expert ids are fetched by scalar loads that this block's barrier wait covers
+            n_valid = c_second >= 0 ? true : tile_coords(tn + 1, nq, np);
+            if (c_second < 0 && n_valid && a.grouped) {
+                asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ld_e0) : "s"(a.m_indices + nq * 256) : "memory");
+                if (!has_tail(nq)) asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ld_e1) : "s"(a.m_indices + nq * 256 + 128) : "memory");
+            }
+        }
+        if (kb == 1) {
+            if (c_second >= 0) {
+                nq = cq; np = cp; n_mask = 2; n_second = -1;
+                setup(nq, np, c_second, n_ptile, n_qtile, n_qtile2, n_sq, n_sp);
+            } else if (n_valid) {
+                const int e0 = a.grouped ? ld_e0 : 0, e1 = has_tail(nq) ? -1 : (a.grouped ? ld_e1 : 0);
+                int ne;
+                classify(e0, e1, ne, n_mask, n_second);
+                setup(nq, np, ne, n_ptile, n_qtile, n_qtile2, n_sq, n_sp);
+            } else {
+                // past the last item the copies and scale loads re-read this item's first blocks
+                n_ptile = c_ptile; n_qtile = c_qtile; n_qtile2 = c_qtile2; n_sq = c_sq; n_sp = c_sp;
+            }
+        }
+        const u32x2 sq_cur = sq_nxt;
+        const uint32_t sp_cur = (sp_nxt >> sp_sh_nxt) & 0xFFu;
+        const bool in1 = kb + 1 < KB, in2 = kb + 2 < KB;
+        const int64_t o1 = (in1 ? kb + 1 : kb + 1 - KB) * 128, o2 = (in2 ? kb + 2 : kb + 2 - KB) * 128;
+        const uint8_t* s_sq = in1 ? c_sq + (kb + 1) * a.ldsq : n_sq;
+        const uint8_t* s_sp = in1 ? c_sp + (kb + 1) : n_sp;
+        const uint8_t* cp1_p = (in1 ? c_ptile : n_ptile) + o1;
+        const uint8_t* cp1_q = (in1 ? c_qtile : n_qtile) + o1;
+        const uint8_t* cp1_q2 = (in1 ? c_qtile2 : n_qtile2) + o1;
+        const uint8_t* cp2_p = (in2 ? c_ptile : n_ptile) + o2;
+        const uint8_t* cp2_q = (in2 ? c_qtile : n_qtile) + o2;
+        const uint8_t* cp2_q2 = (in2 ? c_qtile2 : n_qtile2) + o2;
+        E8_LOAD_S(s_sq, s_sp);
+        const uint8_t* pbase = lds + PAR * SLOT;
+        const uint8_t* nbase = lds + (PAR ^ 1) * SLOT;
+        __builtin_amdgcn_sched_barrier(0);
+        e8_static_for<64>([&](auto mc) {
+            constexpr int m = decltype(mc)::value;
+            constexpr int j = m >> 3, i = m & 7;
+            if constexpr (m == BAR) {
+                // every fragment read of this block has been issued (the last at MFMA 32) and the next
+                // block's copies were all issued by MFMA 12: once both have returned, meet the others
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(sq_nxt), "+s"(sp_nxt), "+s"(ld_e0), "+s"(ld_e1) : : "memory");
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (i == 0 && j + 3 < 8) {
+                qf[(j + 3) % 4] = e8_frag(pbase + fq_ofs[0] + (j + 3) * 128, pbase + fq_ofs[1] + (j + 3) * 128);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            e8_mfma<8 * i + j, (j & 3)>(pf[PAR][i], qf[j % 4], (int)sp_cur, (int)(j < 4 ? sq_cur.x : sq_cur.y));
+            __builtin_amdgcn_sched_barrier(0);
+            // copies: the block after next into the slot this block has just left, continued in the
+            // next block before its barrier
+            if constexpr (m >= BAR && (m - BAR) % CSTEP == 0 && (m - BAR) / CSTEP < 16) {
+                E8_COPY((m - BAR) / CSTEP, cp2_p, cp2_q, cp2_q2, PAR);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (m < BAR && (m + 64 - BAR) % CSTEP == 0 && (m + 64 - BAR) / CSTEP < 16) {
+                E8_COPY((m + 64 - BAR) / CSTEP, cp1_p, cp1_q, cp1_q2, PAR ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // the next block's P fragments and first Q fragments, from the slot just declared landed
+            if constexpr (m >= 48 && m < 56) {
+                pf[PAR ^ 1][m - 48] = e8_frag(nbase + fp_ofs[0] + (m - 48) * 2048, nbase + fp_ofs[1] + (m - 48) * 2048);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (m == 57 || m == 59 || m == 61) {
+                constexpr int jj = (m - 57) / 2;
+                qf[jj] = e8_frag(nbase + fq_ofs[0] + jj * 128, nbase + fq_ofs[1] + jj * 128);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        });
+        ++kb;
+        if (kb < KB) return false;
+
+        // ---- item finished: the wavefronts whose half is stored write it out through a private LDS
+        // slice, one Q fragment (16 rows x 128 columns) at a time, as whole 256-byte rows
+        if ((c_mask >> wq) & 1) {
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written back before they are read
+            uint8_t* ep = lds + EP_OFS + wave * (16 * EP_LD);
+            const int er = lane >> 4, ec = lane & 15;
+            const uint32_t vo = (uint32_t)((er * 8 * a.ldo + ec * 8) * 2);
+            const uint32_t vo_step = (uint32_t)(32 * a.ldo * 2);
+            uint8_t* tile_out = reinterpret_cast<uint8_t*>(a.out) + ((cq * 256 + wq * 128) * a.ldo + cp * 256 + wp * 128) * 2;
+            e8_static_for<8>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                e8_static_for<8>([&](auto icn) {
+                    constexpr int i = decltype(icn)::value;
+                    constexpr int R = 4 * (8 * i + j);
+                    uint2 o;
+                    o.x = pack_bf16(e8_acc_get<R>(), e8_acc_get<R + 1>());
+                    o.y = pack_bf16(e8_acc_get<R + 2>(), e8_acc_get<R + 3>());
+                    *reinterpret_cast<uint2*>(ep + li * EP_LD + (i * 16 + 4 * kg) * 2) = o;
+                });
+                uint8_t* row_out = tile_out + j * a.ldo * 2;
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int rl = er + 4 * it;                        // staged row = li of the producer
+                    const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
+                    *reinterpret_cast<uint4*>(row_out + vo + it * vo_step) = v;
+                }
+            });
+        }
+        if (!n_valid) return true;
+        e8_static_for<64>([&](auto ix) { e8_acc_zero4<decltype(ix)::value>(); });
+        if (c_second < 0) ++tn;
+        cq = nq; cp = np; c_mask = n_mask; c_second = n_second;
+        c_ptile = n_ptile; c_qtile = n_qtile; c_qtile2 = n_qtile2; c_sq = n_sq; c_sp = n_sp;
+        kb = 0;
+        return false;
+    };
+    for (;;) {
+        if (blk(std::integral_constant<int, 0>{})) break;
+        if (blk(std::integral_constant<int, 1>{})) break;
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // the copies issued past the end must land before the LDS is released
+#undef E8_COPY
+#undef E8_LOAD_S
+}
+
+// fp32 scales that are powers of two -> exponent bytes; *bad counts the scales that are not
+__global__ void k_scales_to_ue8m0(const float* __restrict__ s, int64_t n, uint8_t* __restrict__ out, int* bad) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t b = f2u(s[i]);
+    out[i] = (uint8_t)(b >> 23);
+    if (bad && ((b & 0x807FFFFFu) != 0 || (b >> 23) == 0xFF || (b >> 23) == 0)) atomicAdd(bad, 1);
+}
+
+}  // namespace pf8
+
+using namespace pf8;
+
+#define PF8_REQUIRE(cond, msg) do { if (!(cond)) return pf8_fail(PF8_EINVAL, __func__, msg); } while (0)
+#define PF8_ALIGNED16(p) ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)
+
+static constexpr int E8_LDS_BYTES = 131072 + 4 * 16 * 272;
+
+static int launch_e8(const E8Args& a, hipStream_t st, const char* where) {
+    static int attr_done = 0;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_e8), hipFuncAttributeMaxDynamicSharedMemorySize, E8_LDS_BYTES);
+        if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, where, hipGetErrorString(e));
+        attr_done = 1;
+    }
+    const int64_t T = (a.Prows / 256) * ((a.Qrows + 255) / 256), per_xcd = (T + 7) / 8;
+    int64_t w = pf8_effective_cus() / 8;
+    if (w < 1) w = 1;
+    if (w > per_xcd) w = per_xcd;
+    hipLaunchKernelGGL(k_gemm_e8, dim3((unsigned)(8 * w)), dim3(256), E8_LDS_BYTES, st, a);
+    return pf8_check_launch(where);
+}
+
+static int check_e8_shapes(const char* where, int64_t M, int64_t N, int64_t K, int64_t ldsa) {
+    if (M % 128 != 0) return pf8_fail(PF8_EINVAL, where, "M must be a multiple of 128");
+    if (N % 256 != 0) return pf8_fail(PF8_EINVAL, where, "N must be a multiple of 256");
+    if (K % 128 != 0 || K < 384) return pf8_fail(PF8_EINVAL, where, "K must be a multiple of 128 and at least 384");
+    if (ldsa < M || ldsa % 8 != 0) return pf8_fail(PF8_EINVAL, where, "ldsa must be >= M and a multiple of 8");
+    if (K > (1ll << 24)) return pf8_fail(PF8_EINVAL, where, "K too large");
+    return PF8_OK;
+}
+
+extern "C" int pf8_gemm_nt_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b, const uint8_t* sb, int64_t M,
+                                 int64_t N, int64_t K, uint16_t* out, int64_t ldo, pf8_stream_t stream) {
+    PF8_REQUIRE(M >= 0 && N >= 0 && K >= 0, "negative shape");
+    int rc = check_e8_shapes(__func__, M, N, K, ldsa);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return PF8_OK;
+    PF8_REQUIRE(a && sa && b && sb && out, "null pointer");
+    PF8_REQUIRE(ldo >= N && ldo % 8 == 0, "ldo must be >= N and a multiple of 8");
+    PF8_REQUIRE(PF8_ALIGNED16(a) && PF8_ALIGNED16(b) && PF8_ALIGNED16(out) && (reinterpret_cast<uintptr_t>(sa) & 7u) == 0,
+                "a, b, out must be 16-byte aligned and sa 8-byte aligned");
+    PF8_REQUIRE(ldo * 2 * 128 <= 0x7FFFFFFFll, "ldo too large");
+    E8Args g = {};
+    g.p = b; g.q = a; g.sp8 = sb; g.sq8 = sa; g.out = out;
+    g.Prows = N; g.Qrows = M; g.red = K; g.ldo = ldo; g.ldsq = ldsa; g.grouped = 0;
+    return launch_e8(g, (hipStream_t)stream, __func__);
+}
+
+extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b,
+                                                    const uint8_t* sb, int E, int64_t Mtot, int64_t N, int64_t K,
+                                                    const int32_t* m_indices, uint16_t* out, pf8_stream_t stream) {
+    PF8_REQUIRE(E >= 0 && Mtot >= 0 && N >= 0 && K >= 0, "negative shape");
+    int rc = check_e8_shapes(__func__, Mtot, N, K, ldsa);
+    if (rc) return rc;
+    if (Mtot == 0 || N == 0 || E == 0) return PF8_OK;
+    PF8_REQUIRE(a && sa && b && sb && out && m_indices, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(a) && PF8_ALIGNED16(b) && PF8_ALIGNED16(out) && (reinterpret_cast<uintptr_t>(sa) & 7u) == 0,
+                "a, b, out must be 16-byte aligned and sa 8-byte aligned");
+    PF8_REQUIRE(N * 2 * 128 <= 0x7FFFFFFFll, "N too large");
+    E8Args g = {};
+    g.p = b; g.q = a; g.sp8 = sb; g.sq8 = sa; g.out = out;
+    g.Prows = N; g.Qrows = Mtot; g.red = K; g.ldo = N; g.ldsq = ldsa; g.grouped = 1; g.m_indices = m_indices;
+    return launch_e8(g, (hipStream_t)stream, __func__);
+}
+
+extern "C" int pf8_scales_to_ue8m0(const float* s, int64_t n, uint8_t* out, int* not_pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(n >= 0, "negative length");
+    if (n == 0) return PF8_OK;
+    PF8_REQUIRE(s && out, "null pointer");
+    PF8_REQUIRE((n + 255) / 256 <= 0x7FFFFFFFll, "too many scales");
+    hipLaunchKernelGGL(k_scales_to_ue8m0, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, s, n, out, not_pow2);
+    return pf8_check_launch(__func__);
+}

@@ -37,12 +37,39 @@ def _check_pair(pair, what) -> Tuple[torch.Tensor, torch.Tensor]:
     return t, s
 
 
+def _is_ue8m0(s: torch.Tensor) -> bool:
+    return s.dtype == torch.uint8 or s.dtype == getattr(torch, "float8_e8m0fnu", None)
+
+
+def _ue8m0_kmajor(s: torch.Tensor, rows: int, kb: int, what: str) -> torch.Tensor:
+    """Exponent bytes logically [rows, K/128] -> the K-block-major [K/128, ld] storage the kernel reads
+    (ld a multiple of 8).  The `.T` view of such a tensor is consumed without a copy."""
+    s = s.view(torch.uint8)
+    if tuple(s.shape) != (rows, kb):
+        raise ValueError(f"{what} must be [{rows}, {kb}]")
+    if s.stride(0) == 1 and s.stride(1) >= rows and s.stride(1) % 8 == 0 and s.data_ptr() % 8 == 0:
+        return s.t()
+    ld = (rows + 7) // 8 * 8
+    buf = torch.empty((kb, ld), dtype=torch.uint8, device=s.device)
+    buf[:, :rows].copy_(s.t())
+    return buf[:, :rows]
+
+
+def _decode_ue8m0(s: torch.Tensor) -> torch.Tensor:
+    return torch.exp2(s.view(torch.uint8).to(torch.float32) - 127.0)
+
+
+def _ue8m0_kernel_shape(M: int, N: int, K: int) -> bool:
+    return M % 128 == 0 and N % 256 == 0 and K % 128 == 0 and K >= 384
+
+
 def fp8_gemm_nt(a, b, out: torch.Tensor, c: Optional[torch.Tensor] = None, recipe=None, compiled_dims: str = "nk"):
     """out[M, N] = a[M, K] . b[N, K]^T with block scales, fp32 accumulation.
 
     Default recipe (transformers/fp8_utils.py:278): a is 1x128-scaled with sa logically [M, K/128]
     (any strides; the M-contiguous `.T` view of a [K/128, M] tensor is consumed without a copy),
-    b is 128x128-scaled with sb [ceil(N/128), K/128]; out is bf16.
+    b is 128x128-scaled with sb [ceil(N/128), K/128]; out is bf16.  Scales of dtype uint8 (or
+    float8_e8m0fnu) are UE8M0 exponent bytes, scale = 2^(byte - 127), in the same logical shapes.
     recipe=(1, 1, 128) (transformers/fp8_utils.py:187-194): both operands 1x128-scaled along K with
     scales logically [rows, K/128]; out is fp32 and `c is out` means accumulate.
     """
@@ -76,6 +103,19 @@ def fp8_gemm_nt(a, b, out: torch.Tensor, c: Optional[torch.Tensor] = None, recip
         raise ValueError("accumulation needs recipe=(1, 1, 128)")
     if out.dtype != torch.bfloat16 or out.stride(-1) != 1:
         raise ValueError("out must be bfloat16 with a unit inner stride")
+    if _is_ue8m0(sa) != _is_ue8m0(sb):
+        raise ValueError("UE8M0 scales must be given for both operands or for neither")
+    if _is_ue8m0(sa):
+        # power-of-two scales as exponent bytes (`use_ue8m0`, transformers/configuration_utils.py:454-459):
+        # the block-scaled MFMA kernel where its tile shape fits, else the fp32-scale kernel on decoded scales
+        if tuple(sb.shape) != ((N + 127) // 128, K // 128):
+            raise ValueError(f"b scale must be [{(N + 127) // 128}, {K // 128}]")
+        if _ue8m0_kernel_shape(M, N, K) and out.stride(0) % 8 == 0 and out.data_ptr() % 16 == 0:
+            sa_k = _ue8m0_kmajor(sa, M, K // 128, "a scale")
+            sb_k = sb.view(torch.uint8).contiguous()
+            _lib.call("pf8_gemm_nt_ue8m0", _p(ta), _p(sa_k), sa_k.stride(0), _p(tb), _p(sb_k), M, N, K, _p(out), out.stride(0), _stream())
+            return out
+        sa, sb = _decode_ue8m0(sa), _decode_ue8m0(sb)
     sa, lay = _scale_layout_of(sa, M, K // 128, "a scale")
     if tuple(sb.shape) != ((N + 127) // 128, K // 128) or sb.dtype != torch.float32:
         raise ValueError(f"b scale must be float32 [{(N + 127) // 128}, {K // 128}]")
@@ -109,11 +149,23 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
         return out
     ta = ta if ta.is_contiguous() else ta.contiguous()
     tb = tb if tb.is_contiguous() else tb.contiguous()
+    m_indices = m_indices if m_indices.is_contiguous() else m_indices.contiguous()
+    if _is_ue8m0(sa) != _is_ue8m0(sb):
+        raise ValueError("UE8M0 scales must be given for both operands or for neither")
+    if _is_ue8m0(sa):
+        if tuple(sb.shape) != (E, (N + 127) // 128, K // 128):
+            raise ValueError(f"b scale must be [{E}, {(N + 127) // 128}, {K // 128}]")
+        if _ue8m0_kernel_shape(Mtot, N, K):
+            sa_k = _ue8m0_kmajor(sa, Mtot, K // 128, "a scale")
+            sb_k = sb.view(torch.uint8).contiguous()
+            _lib.call("pf8_grouped_gemm_nt_contiguous_ue8m0", _p(ta), _p(sa_k), sa_k.stride(0), _p(tb), _p(sb_k), E, Mtot, N, K,
+                      _p(m_indices), _p(out), _stream())
+            return out
+        sa, sb = _decode_ue8m0(sa), _decode_ue8m0(sb)
     sa, lay = _scale_layout_of(sa, Mtot, K // 128, "a scale")
     if tuple(sb.shape) != (E, (N + 127) // 128, K // 128) or sb.dtype != torch.float32:
         raise ValueError(f"b scale must be float32 [{E}, {(N + 127) // 128}, {K // 128}]")
     sb = sb if sb.is_contiguous() else sb.contiguous()
-    m_indices = m_indices if m_indices.is_contiguous() else m_indices.contiguous()
     _lib.call("pf8_grouped_gemm_nt_contiguous", _p(ta), _p(sa), lay, _p(tb), _p(sb), E, Mtot, N, K, _p(m_indices), _p(out), _stream())
     return out
 

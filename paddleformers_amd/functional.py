@@ -295,6 +295,26 @@ def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], 
 # ---------------------------------------------------------------------------------------------
 
 
+def scales_to_ue8m0(scale: torch.Tensor, check: bool = True) -> torch.Tensor:
+    """fp32 power-of-two scales (what the quantizers emit with using_pow2_scale=True) -> UE8M0
+    exponent bytes of the same shape and strides order, scale = 2^(byte - 127): the scale format
+    `use_ue8m0` hands to deep_gemm (transformers/configuration_utils.py:454-459).  With `check` the
+    call synchronizes and raises if a scale is not a positive finite power of two."""
+    _dev(scale, "scale")
+    if scale.dtype != torch.float32:
+        raise ValueError("scale must be float32")
+    dense = scale if scale.is_contiguous() or scale.t().is_contiguous() else scale.contiguous()
+    out = torch.empty_like(dense, dtype=torch.uint8)      # preserves the strides of a dense tensor
+    if out.stride() != dense.stride():
+        dense = dense.contiguous()
+        out = torch.empty_like(dense, dtype=torch.uint8)
+    bad = torch.zeros(1, dtype=torch.int32, device=scale.device) if check else None
+    _lib.call("pf8_scales_to_ue8m0", _p(dense), dense.numel(), _p(out), _p(bad), _stream())
+    if check and int(bad.item()) != 0:
+        raise ValueError(f"{int(bad.item())} scales are not positive powers of two")
+    return out
+
+
 def fused_act_dequant(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     """1x128 dequantization to bf16: bf16(float(q) * s).  transformers/fp8_utils.py:136-138, :779."""
     _dev(q, "q")

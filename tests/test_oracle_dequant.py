@@ -62,3 +62,22 @@ def test_float_scales_and_bf16_output_match_the_128x128_weight_dequant():
     q[(q & 0x7F) == 0x7F] = 0x10
     s = rng.uniform(1e-3, 2.0, size=(2, 3)).astype(np.float32)
     np.testing.assert_array_equal(O.block_dequant(q, s, "float32", (0, 1), (128, 128), out="bf16"), O.weight_dequant(q, s))
+
+
+def test_scales_to_ue8m0_inverts_the_decode_table_over_every_finite_exponent():
+    # the table is pinned by the reference's vectors above (code 126 -> 0.5, 127 -> 1, 128 -> 2, 255 -> inf)
+    codes = np.arange(1, 255, dtype=np.uint8)
+    scales = O.decode_scales(codes, "ue8m0")
+    assert np.array_equal(O.scales_to_ue8m0(scales), codes)
+    assert O.scales_to_ue8m0(np.array([1.0, 0.5, 2.0 ** -20], np.float32)).tolist() == [127, 126, 107]
+    for bad in (0.75, -1.0, 3.0):
+        with pytest.raises(ValueError):
+            O.scales_to_ue8m0(np.array([bad], np.float32))
+
+
+def test_pow2_quantizer_scales_are_exact_ue8m0_codes():
+    # what the GEMM with exponent-byte scales relies on: a pow2 scale survives the byte round trip
+    rng = np.random.default_rng(3)
+    x = O.f32_to_bf16_bits(rng.standard_normal((4, 256)).astype(np.float32) * 3.0)
+    _, s = O.quant_1x128(x, 0, pow2=True)
+    assert np.array_equal(O.decode_scales(O.scales_to_ue8m0(s), "ue8m0"), s)
