@@ -22,8 +22,11 @@
 //     forth).  One empty statement that clobbers a255 makes the kernel descriptor reserve all 256.
 //   * Q row r of a wavefront's fragment j is row 8 (r) + j of its 128, so the eight scale bytes a lane
 //     needs per block are contiguous (one 8-byte load) and op_sel picks the byte per MFMA.
-//   * A 256-row tile of the contiguous grouped layout may hold two experts (segments are padded to
-//     128 rows): such a tile is walked twice, once per expert, each pass storing its own half.
+//   * Grouped layout: expert segments are padded to 128 rows, so a 256-row tile is made of two
+//     128-row blocks of the SAME expert that need not be neighbours.  A one-workgroup pre-pass pairs
+//     the blocks of every expert (an odd one out gets a half-empty tile, padding blocks get none) and
+//     writes the list the GEMM walks.  Without a list the kernel walks aligned 256-row tiles and
+//     visits a tile that holds two experts twice, once per expert, each pass storing its own half.
 #include <type_traits>
 
 #include "pf8_device.h"
@@ -40,6 +43,7 @@ struct E8Args {
     int64_t Prows, Qrows, red, ldo, ldsq;
     int grouped;
     const int32_t* m_indices;
+    const int32_t* items;   // grouped: {n, -, -, -} then {block0, block1 or -1, expert, -} per item; may be null
 };
 
 __device__ __forceinline__ int e8_keyp(int row) { return (row & 7) ^ ((row >> 3) & 1); }
@@ -91,7 +95,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     const int wq = wave >> 1, wp = wave & 1;
     const int li = lane & 15, kg = lane >> 4;
 
-    const int64_t p_tiles = a.Prows / 256, q_tiles = (a.Qrows + 255) / 256;
+    const int64_t p_tiles = a.Prows / 256, q_tiles = a.items ? (int64_t)__builtin_amdgcn_readfirstlane(a.items[0]) : (a.Qrows + 255) / 256;
     const int64_t T = p_tiles * q_tiles;
     // consecutive workgroups go round-robin to the 8 XCDs: every XCD owns a contiguous run of
     // logical tiles (groups of 8 q-tiles x all p-tiles), walked W tiles at a time by its W workgroups
@@ -123,27 +127,46 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     // work item = (tile, expert, halves to store); c_* current, n_* next; all wave-uniform
     int64_t cq = 0, cp = 0, nq = 0, np = 0, tn = 0;
     if (!tile_coords(0, cq, cp)) return;
-    int c_e, c_mask, c_second, n_mask = 0, n_second = -1;
-    {
-        int e0 = 0, e1 = has_tail(cq) ? -1 : 0;
-        if (a.grouped) {
-            e0 = a.m_indices[cq * 256];
-            if (!has_tail(cq)) e1 = a.m_indices[cq * 256 + 128];
-        }
-        classify(e0, e1, c_e, c_mask, c_second);
-    }
-    int ld_e0 = 0, ld_e1 = 0;      // expert ids of the next tile's halves, loaded one block before they are used
+    int c_mask, c_second = -1, n_mask = 0, n_second = -1;
+    int64_t c_orow, n_orow = 0;                 // first output row of this wavefront's half
     const uint8_t *c_ptile, *c_qtile, *c_qtile2, *c_sq, *c_sp;
+    // aligned tile qt of expert e
     auto setup = [&](int64_t qt, int64_t pt, int e, const uint8_t*& ptile, const uint8_t*& qtile, const uint8_t*& qtile2,
-                     const uint8_t*& sq, const uint8_t*& sp) {
+                     const uint8_t*& sq, const uint8_t*& sp, int64_t& orow) {
         const bool tail = has_tail(qt);
         ptile = a.p + ((int64_t)e * a.Prows + pt * 256) * a.red;
         qtile = a.q + qt * 256 * a.red;
         qtile2 = tail ? qtile : qtile + 128 * a.red;     // a missing second half re-reads the first
         sq = a.sq8 + qt * 256 + ((wq && !tail) ? 128 : 0);
         sp = a.sp8 + ((int64_t)e * PB + pt * 2 + wp) * KB;
+        orow = qt * 256 + wq * 128;
     };
-    setup(cq, cp, c_e, c_ptile, c_qtile, c_qtile2, c_sq, c_sp);
+    // listed item {block0, block1 or -1, expert}
+    auto setup_item = [&](i32x4 it, int64_t pt, int& mask, const uint8_t*& ptile, const uint8_t*& qtile, const uint8_t*& qtile2,
+                          const uint8_t*& sq, const uint8_t*& sp, int64_t& orow) {
+        const int64_t b0 = it.x, b1 = it.y < 0 ? it.x : it.y;
+        mask = it.y < 0 ? 1 : 3;
+        ptile = a.p + ((int64_t)it.z * a.Prows + pt * 256) * a.red;
+        qtile = a.q + b0 * 128 * a.red;
+        qtile2 = a.q + b1 * 128 * a.red;
+        sq = a.sq8 + (wq ? b1 : b0) * 128;
+        sp = a.sp8 + ((int64_t)it.z * PB + pt * 2 + wp) * KB;
+        orow = (wq ? b1 : b0) * 128;
+    };
+    if (a.items) {
+        const int32_t* ip = a.items + 4 + 4 * cq;
+        setup_item((i32x4){__builtin_amdgcn_readfirstlane(ip[0]), __builtin_amdgcn_readfirstlane(ip[1]), __builtin_amdgcn_readfirstlane(ip[2]), 0}, cp, c_mask, c_ptile, c_qtile, c_qtile2, c_sq, c_sp, c_orow);
+    } else {
+        int e0 = 0, e1 = has_tail(cq) ? -1 : 0, c_e;
+        if (a.grouped) {
+            e0 = __builtin_amdgcn_readfirstlane(a.m_indices[cq * 256]);
+            if (!has_tail(cq)) e1 = __builtin_amdgcn_readfirstlane(a.m_indices[cq * 256 + 128]);
+        }
+        classify(e0, e1, c_e, c_mask, c_second);
+        setup(cq, cp, c_e, c_ptile, c_qtile, c_qtile2, c_sq, c_sp, c_orow);
+    }
+    int ld_e0 = 0, ld_e1 = 0;      // expert ids of the next tile's halves
+    i32x4 ld_item = {0, 0, 0, 0};  // or its list entry
     const uint8_t *n_ptile = c_ptile, *n_qtile = c_qtile, *n_qtile2 = c_qtile2, *n_sq = c_sq, *n_sp = c_sp;
     bool n_valid = false;
 
@@ -164,6 +187,8 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
         fq_ofs[h] = Q_OFS + (wq * 128 + li * 8) * 128 + (((2 * kg + h) ^ (li & 7)) << 4);
     }
     const uint32_t s_off = (uint32_t)(li * 8);
+    uint32_t zero_off = 0;
+    asm volatile("" : "+v"(zero_off));     // a VGPR holding 0 (the address form needs one)
 
 #define E8_COPY(c_, pt_, qt_, qt2_, slot_)                                                             \
     do {                                                                                               \
@@ -171,19 +196,19 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
         else if ((c_) < 12) e8_dma16(c_off_q[(c_) & 1], (qt_) + ((c_) - 8) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
         else e8_dma16(c_off_q[(c_) & 1], (qt2_) + ((c_) - 12) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
     } while (0)
-    // the scale bytes of a block: eight Q exponents per lane, and the aligned dword that holds the P
-    // block's exponent (extracted when the block starts)
+    // the scale bytes of a block, straight into the VGPRs the MFMAs take them from: eight Q exponents per
+    // lane and the P block's exponent (every lane the same byte).  Vector loads on purpose: the value of
+    // an asynchronous load may not be touched before its wait, and the compiler, which cannot know that,
+    // is free to copy or spill a scalar register at any point, but leaves these VGPRs alone.
 #define E8_LOAD_S(sq_, sp_)                                                                            \
     do {                                                                                               \
         asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(sq_nxt) : "v"(s_off), "s"(sq_) : "memory"); \
-        const uintptr_t spa_ = reinterpret_cast<uintptr_t>(sp_);                                       \
-        asm volatile("s_load_dword %0, %1, 0x0" : "=s"(sp_nxt) : "s"(spa_ & ~(uintptr_t)3) : "memory"); \
-        sp_sh_nxt = (uint32_t)(spa_ & 3) * 8;                                                          \
+        asm volatile("global_load_ubyte %0, %1, %2" : "=v"(sp_nxt) : "v"(zero_off), "s"(sp_) : "memory"); \
     } while (0)
 
     i32x8 pf[2][8], qf[4];
     u32x2 sq_nxt = {0, 0};
-    uint32_t sp_nxt = 0, sp_sh_nxt = 0;
+    uint32_t sp_nxt = 0;
 
     e8_static_for<64>([&](auto ix) { e8_acc_zero4<decltype(ix)::value>(); });
     {
@@ -193,7 +218,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
 #pragma unroll
         for (int c = 0; c < 16; ++c)
             if (c * CSTEP < 64 - BAR) E8_COPY(c, c_ptile + 128, c_qtile + 128, c_qtile2 + 128, 1);
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(sq_nxt), "+s"(sp_nxt) : : "memory");
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(sq_nxt), "+v"(sp_nxt) : : "memory");
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < 8; ++i) pf[0][i] = e8_frag(lds + fp_ofs[0] + i * 2048, lds + fp_ofs[1] + i * 2048);
@@ -208,29 +233,36 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
         constexpr int PAR = decltype(par_c)::value;
         if (kb == 0) {
             // the item after this one: the same tile again for its second expert, or the next tile, whose
-            // expert ids are fetched by scalar loads that this block's barrier wait covers
+            // list entry / expert ids are fetched here (scalar loads, waited for on the spot: once per item)
             n_valid = c_second >= 0 ? true : tile_coords(tn + 1, nq, np);
-            if (c_second < 0 && n_valid && a.grouped) {
-                asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ld_e0) : "s"(a.m_indices + nq * 256) : "memory");
-                if (!has_tail(nq)) asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ld_e1) : "s"(a.m_indices + nq * 256 + 128) : "memory");
+            if (c_second < 0 && n_valid) {
+                if (a.items) {
+                    asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ld_item) : "s"(a.items + 4 + 4 * nq) : "memory");
+                } else if (a.grouped) {
+                    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ld_e0) : "s"(a.m_indices + nq * 256) : "memory");
+                    if (!has_tail(nq))
+                        asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ld_e1) : "s"(a.m_indices + nq * 256 + 128) : "memory");
+                }
             }
         }
         if (kb == 1) {
             if (c_second >= 0) {
                 nq = cq; np = cp; n_mask = 2; n_second = -1;
-                setup(nq, np, c_second, n_ptile, n_qtile, n_qtile2, n_sq, n_sp);
+                setup(nq, np, c_second, n_ptile, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
+            } else if (n_valid && a.items) {
+                setup_item(ld_item, np, n_mask, n_ptile, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
             } else if (n_valid) {
                 const int e0 = a.grouped ? ld_e0 : 0, e1 = has_tail(nq) ? -1 : (a.grouped ? ld_e1 : 0);
                 int ne;
                 classify(e0, e1, ne, n_mask, n_second);
-                setup(nq, np, ne, n_ptile, n_qtile, n_qtile2, n_sq, n_sp);
+                setup(nq, np, ne, n_ptile, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
             } else {
                 // past the last item the copies and scale loads re-read this item's first blocks
                 n_ptile = c_ptile; n_qtile = c_qtile; n_qtile2 = c_qtile2; n_sq = c_sq; n_sp = c_sp;
             }
         }
         const u32x2 sq_cur = sq_nxt;
-        const uint32_t sp_cur = (sp_nxt >> sp_sh_nxt) & 0xFFu;
+        const uint32_t sp_cur = sp_nxt;
         const bool in1 = kb + 1 < KB, in2 = kb + 2 < KB;
         const int64_t o1 = (in1 ? kb + 1 : kb + 1 - KB) * 128, o2 = (in2 ? kb + 2 : kb + 2 - KB) * 128;
         const uint8_t* s_sq = in1 ? c_sq + (kb + 1) * a.ldsq : n_sq;
@@ -251,7 +283,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
             if constexpr (m == BAR) {
                 // every fragment read of this block has been issued (the last at MFMA 32) and the next
                 // block's copies were all issued by MFMA 12: once both have returned, meet the others
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(sq_nxt), "+s"(sp_nxt), "+s"(ld_e0), "+s"(ld_e1) : : "memory");
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(sq_nxt), "+v"(sp_nxt) : : "memory");
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -293,7 +325,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
             const int er = lane >> 4, ec = lane & 15;
             const uint32_t vo = (uint32_t)((er * 8 * a.ldo + ec * 8) * 2);
             const uint32_t vo_step = (uint32_t)(32 * a.ldo * 2);
-            uint8_t* tile_out = reinterpret_cast<uint8_t*>(a.out) + ((cq * 256 + wq * 128) * a.ldo + cp * 256 + wp * 128) * 2;
+            uint8_t* tile_out = reinterpret_cast<uint8_t*>(a.out) + (c_orow * a.ldo + cp * 256 + wp * 128) * 2;
             e8_static_for<8>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 e8_static_for<8>([&](auto icn) {
@@ -316,7 +348,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
         if (!n_valid) return true;
         e8_static_for<64>([&](auto ix) { e8_acc_zero4<decltype(ix)::value>(); });
         if (c_second < 0) ++tn;
-        cq = nq; cp = np; c_mask = n_mask; c_second = n_second;
+        cq = nq; cp = np; c_mask = n_mask; c_second = n_second; c_orow = n_orow;
         c_ptile = n_ptile; c_qtile = n_qtile; c_qtile2 = n_qtile2; c_sq = n_sq; c_sp = n_sp;
         kb = 0;
         return false;
@@ -328,6 +360,75 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     __builtin_amdgcn_s_waitcnt(0);   // the copies issued past the end must land before the LDS is released
 #undef E8_COPY
 #undef E8_LOAD_S
+}
+
+// Pairs the 128-row blocks of every expert of a contiguous grouped layout into 256-row work items.
+// One workgroup of 1024 threads, each walking a contiguous run of blocks; two scans over the threads:
+// the parity of a block inside its expert's segment (a composition of {reset, flip} functions), then
+// the number of items opened before it (an item opens at every even block of a segment).
+// items = {n, 0, 0, 0} followed by {block0, block1 or -1, expert, 0} per item.
+__global__ __launch_bounds__(1024) void k_e8_build_items(const int32_t* __restrict__ m_indices, int64_t NB, int32_t* __restrict__ items) {
+    __shared__ int s_scan[2][1024];
+    const int tid = threadIdx.x;
+    const int64_t chunk = (NB + 1023) / 1024;
+    const int64_t lo = tid * chunk < NB ? tid * chunk : NB, hi = lo + chunk < NB ? lo + chunk : NB;
+    auto expert = [&](int64_t b) -> int { return (b < 0 || b >= NB) ? -2 : m_indices[b * 128]; };
+    // function codes: bit 1 = constant, bit 0 = its value (constant) or flip (otherwise); g after f:
+    auto then = [](int f, int g) -> int { return (g & 2) ? g : (f ^ (g & 1)); };
+    auto step_fn = [&](int prev_e, int e) -> int { return e < 0 ? 3 : (e != prev_e ? 2 : 1); };
+    int f = 0, pe = expert(lo - 1);
+    for (int64_t b = lo; b < hi; ++b) { const int e = expert(b); f = then(f, step_fn(pe, e)); pe = e; }
+    // inclusive scan of the function composition (Hillis-Steele)
+    int cur = 0;
+    s_scan[0][tid] = f;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int v = tid >= d ? then(s_scan[cur][tid - d], s_scan[cur][tid]) : s_scan[cur][tid];
+        s_scan[cur ^ 1][tid] = v;
+        cur ^= 1;
+        __syncthreads();
+    }
+    const int f_in = tid ? s_scan[cur][tid - 1] : 0;
+    int par = (f_in & 2) ? (f_in & 1) : (1 ^ (f_in & 1));     // parity of the block before `lo` (1 = none open)
+    __syncthreads();
+    // items opened in this run of blocks
+    int opened = 0, p = par;
+    pe = expert(lo - 1);
+    for (int64_t b = lo; b < hi; ++b) {
+        const int e = expert(b);
+        p = e < 0 ? 1 : (e != pe ? 0 : p ^ 1);
+        opened += (e >= 0 && p == 0);
+        pe = e;
+    }
+    cur = 0;
+    s_scan[0][tid] = opened;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int v = tid >= d ? s_scan[cur][tid - d] + s_scan[cur][tid] : s_scan[cur][tid];
+        s_scan[cur ^ 1][tid] = v;
+        cur ^= 1;
+        __syncthreads();
+    }
+    int t = (tid ? s_scan[cur][tid - 1] : 0) - 1;     // index of the item open before `lo`
+    if (tid == 1023) { items[0] = s_scan[cur][1023]; items[1] = 0; items[2] = 0; items[3] = 0; }
+    p = par;
+    pe = expert(lo - 1);
+    for (int64_t b = lo; b < hi; ++b) {
+        const int e = expert(b);
+        p = e < 0 ? 1 : (e != pe ? 0 : p ^ 1);
+        if (e >= 0) {
+            if (p == 0) {
+                ++t;
+                items[4 + 4 * t] = (int32_t)b;
+                items[4 + 4 * t + 2] = e;
+                items[4 + 4 * t + 3] = 0;
+                if (expert(b + 1) != e) items[4 + 4 * t + 1] = -1;
+            } else {
+                items[4 + 4 * t + 1] = (int32_t)b;
+            }
+        }
+        pe = e;
+    }
 }
 
 // fp32 scales that are powers of two -> exponent bytes; *bad counts the scales that are not
@@ -348,14 +449,14 @@ using namespace pf8;
 
 static constexpr int E8_LDS_BYTES = 131072 + 4 * 16 * 272;
 
-static int launch_e8(const E8Args& a, hipStream_t st, const char* where) {
+static int launch_e8(const E8Args& a, int64_t max_q_tiles, hipStream_t st, const char* where) {
     static int attr_done = 0;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_e8), hipFuncAttributeMaxDynamicSharedMemorySize, E8_LDS_BYTES);
         if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, where, hipGetErrorString(e));
         attr_done = 1;
     }
-    const int64_t T = (a.Prows / 256) * ((a.Qrows + 255) / 256), per_xcd = (T + 7) / 8;
+    const int64_t T = (a.Prows / 256) * max_q_tiles, per_xcd = (T + 7) / 8;
     int64_t w = pf8_effective_cus() / 8;
     if (w < 1) w = 1;
     if (w > per_xcd) w = per_xcd;
@@ -386,12 +487,13 @@ extern "C" int pf8_gemm_nt_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ld
     E8Args g = {};
     g.p = b; g.q = a; g.sp8 = sb; g.sq8 = sa; g.out = out;
     g.Prows = N; g.Qrows = M; g.red = K; g.ldo = ldo; g.ldsq = ldsa; g.grouped = 0;
-    return launch_e8(g, (hipStream_t)stream, __func__);
+    return launch_e8(g, (M + 255) / 256, (hipStream_t)stream, __func__);
 }
 
 extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b,
                                                     const uint8_t* sb, int E, int64_t Mtot, int64_t N, int64_t K,
-                                                    const int32_t* m_indices, uint16_t* out, pf8_stream_t stream) {
+                                                    const int32_t* m_indices, int32_t* items_ws, uint16_t* out,
+                                                    pf8_stream_t stream) {
     PF8_REQUIRE(E >= 0 && Mtot >= 0 && N >= 0 && K >= 0, "negative shape");
     int rc = check_e8_shapes(__func__, Mtot, N, K, ldsa);
     if (rc) return rc;
@@ -403,7 +505,15 @@ extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint
     E8Args g = {};
     g.p = b; g.q = a; g.sp8 = sb; g.sq8 = sa; g.out = out;
     g.Prows = N; g.Qrows = Mtot; g.red = K; g.ldo = N; g.ldsq = ldsa; g.grouped = 1; g.m_indices = m_indices;
-    return launch_e8(g, (hipStream_t)stream, __func__);
+    if (items_ws) {
+        PF8_REQUIRE((reinterpret_cast<uintptr_t>(items_ws) & 15u) == 0, "items_ws must be 16-byte aligned");
+        hipLaunchKernelGGL(k_e8_build_items, dim3(1), dim3(1024), 0, (hipStream_t)stream, m_indices, Mtot / 128, items_ws);
+        rc = pf8_check_launch(__func__);
+        if (rc) return rc;
+        g.items = items_ws;
+        return launch_e8(g, Mtot / 128, (hipStream_t)stream, __func__);
+    }
+    return launch_e8(g, (Mtot + 255) / 256, (hipStream_t)stream, __func__);
 }
 
 extern "C" int pf8_scales_to_ue8m0(const float* s, int64_t n, uint8_t* out, int* not_pow2, pf8_stream_t stream) {

@@ -158,8 +158,9 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
         if _ue8m0_kernel_shape(Mtot, N, K):
             sa_k = _ue8m0_kmajor(sa, Mtot, K // 128, "a scale")
             sb_k = sb.view(torch.uint8).contiguous()
+            items = torch.empty(4 + 4 * (Mtot // 128), dtype=torch.int32, device=ta.device)
             _lib.call("pf8_grouped_gemm_nt_contiguous_ue8m0", _p(ta), _p(sa_k), sa_k.stride(0), _p(tb), _p(sb_k), E, Mtot, N, K,
-                      _p(m_indices), _p(out), _stream())
+                      _p(m_indices), _p(items), _p(out), _stream())
             return out
         sa, sb = _decode_ue8m0(sa), _decode_ue8m0(sb)
     sa, lay = _scale_layout_of(sa, Mtot, K // 128, "a scale")

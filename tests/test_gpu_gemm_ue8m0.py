@@ -159,15 +159,34 @@ def _grouped_pow2_case(E, N, K, rows, seed):
     return a, sa, np.stack(bs), np.stack(sbs), np.repeat(np.arange(E, dtype=np.int32), rows)
 
 
-# segments that start in the middle of a 256-row tile (two experts in one tile), empty experts, a
-# half tile at the end
+def _grouped_call(dg, a, sa, b, sb, m_idx, out, paired):
+    """paired: through the mirror, which lets the library pair each expert's 128-row blocks into tiles;
+    otherwise the raw C ABI without a work-item list (aligned 256-row tiles, two passes over a tile
+    that holds two experts)."""
+    ta, tb, tm = G.to_torch_fp8(a), G.to_torch_fp8(b), torch.from_numpy(m_idx).cuda()
+    if paired:
+        dg.m_grouped_fp8_gemm_nt_contiguous((ta, _e8(sa)), (tb, _e8(sb)), out, tm)
+        return
+    from paddleformers_amd import _lib
+
+    E, N, K = b.shape
+    tsa = _e8(np.ascontiguousarray(sa.T))           # [K/128, Mtot]
+    tsb = _e8(sb)
+    _lib.call("pf8_grouped_gemm_nt_contiguous_ue8m0", ta.data_ptr(), tsa.data_ptr(), tsa.stride(0), tb.data_ptr(), tsb.data_ptr(),
+              E, a.shape[0], N, K, tm.data_ptr(), None, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+
+
+# segments that start in the middle of a 256-row tile (two experts in one aligned tile), segments of
+# an odd number of blocks, empty experts, a half tile at the end
 @pytest.mark.parametrize("rows", [[128, 256, 0, 128], [0, 0, 384], [128] * 6, [256, 512], [384, 128, 640, 128]])
-def test_grouped_contiguous_ue8m0_vs_oracle(dg, rows):
+@pytest.mark.parametrize("paired", [True, False])
+def test_grouped_contiguous_ue8m0_vs_oracle(dg, rows, paired):
     E, N, K = len(rows), 512, 512
     a, sa, b, sb, m_idx = _grouped_pow2_case(E, N, K, rows, seed=sum(rows) + E)
     Mtot = a.shape[0]
     out = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
-    dg.m_grouped_fp8_gemm_nt_contiguous((G.to_torch_fp8(a), _e8(sa)), (G.to_torch_fp8(b), _e8(sb)), out, torch.from_numpy(m_idx).cuda())
+    _grouped_call(dg, a, sa, b, sb, m_idx, out, paired)
     exp = O.grouped_gemm_nt_contiguous(a, sa, b, sb, m_idx)
     got = G.from_torch_bf16(out)
     assert G.rel_fro(_bf(got), _bf(exp)) <= BLOCK_FRO
@@ -178,7 +197,33 @@ def test_grouped_contiguous_ue8m0_vs_oracle(dg, rows):
         start += r
 
 
-def test_grouped_contiguous_ue8m0_negative_index_skips_rows(dg):
+def test_grouped_contiguous_ue8m0_many_small_experts(dg):
+    """40 experts of 0..5 blocks in Zipf-like disorder, some followed by padding blocks (index -1): every
+    routed row is computed with its own expert's weights and every padding row is left alone."""
+    rng = np.random.default_rng(12)
+    E, N, K = 40, 256, 384
+    rows = [int(128 * rng.integers(0, 6)) for _ in range(E)]
+    a, sa, b, sb, m_idx = _grouped_pow2_case(E, N, K, rows, seed=77)
+    pad = np.zeros(len(m_idx), bool)
+    start = 0
+    for e, r in enumerate(rows):
+        if r >= 256 and rng.random() < 0.4:
+            pad[start + r - 128:start + r] = True         # the expert's last block is padding
+        start += r
+    m_idx = m_idx.copy()
+    m_idx[pad] = -1
+    out = torch.full((len(m_idx), N), 7.0, dtype=torch.bfloat16, device="cuda")
+    _grouped_call(dg, a, sa, b, sb, m_idx, out, True)
+    got = G.from_torch_bf16(out)
+    seven = O.f32_to_bf16_bits(np.full((1,), 7.0, np.float32))[0]
+    assert (got[pad] == seven).all()
+    init = np.full(got.shape, seven, np.uint16)
+    exp = O.grouped_gemm_nt_contiguous(a, sa, b, sb, m_idx, out=init)
+    assert G.rel_fro(_bf(got[~pad]), _bf(exp[~pad])) <= BLOCK_FRO
+
+
+@pytest.mark.parametrize("paired", [True, False])
+def test_grouped_contiguous_ue8m0_negative_index_skips_rows(dg, paired):
     """Padding rows (index -1) are left untouched whichever half of a 256-row tile they fill."""
     E, N, K = 3, 256, 384
     rows = [256, 256, 256]
@@ -187,7 +232,7 @@ def test_grouped_contiguous_ue8m0_negative_index_skips_rows(dg):
     m_idx[256:384] = -1       # first half of tile 1
     m_idx[512:768] = -1       # all of tile 2
     out = torch.full((768, N), 7.0, dtype=torch.bfloat16, device="cuda")
-    dg.m_grouped_fp8_gemm_nt_contiguous((G.to_torch_fp8(a), _e8(sa)), (G.to_torch_fp8(b), _e8(sb)), out, torch.from_numpy(m_idx).cuda())
+    _grouped_call(dg, a, sa, b, sb, m_idx, out, paired)
     got = G.from_torch_bf16(out)
     seven = O.f32_to_bf16_bits(np.full((1,), 7.0, np.float32))[0]
     for lo, hi, e in [(0, 128, 0), (384, 512, 1)]:
