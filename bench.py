@@ -149,7 +149,32 @@ def bench_other_gemms(iters=10, warmup=3):
     o = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
     ms = time_kernel(lambda: deep_gemm.fp8_gemm_nt((a, sa.T), (b, sb), o), [()], iters, warmup)
     out["dense_config2_8192x4096x7168"] = {"flop": 2.0 * M * N * K, "ms": ms}
+
+    def e8(*shape):     # UE8M0 exponent bytes around 2^0
+        return torch.randint(120, 131, shape, dtype=torch.uint8, device="cuda")
+
+    # the same GEMM with power-of-two scales as exponent bytes: block-scaled MFMA kernel
+    ea, eb = e8(K // 128, M), e8(N // 128, K // 128)
+    ms = time_kernel(lambda: deep_gemm.fp8_gemm_nt((a, ea.T), (b, eb), o), [()], iters, warmup)
+    out["dense_config2_ue8m0"] = {"flop": 2.0 * M * N * K, "ms": ms}
     del a, b, o
+    # config 3 forward GEMMs (32 experts, 8192 routed rows, Zipf 1.1, segments padded to 128) with UE8M0 scales
+    E3, H3, I3 = 32, 7168, 2048
+    _, padded3 = zipf_counts(8192, E3, 1.1, seed=3)
+    M3 = int(padded3.sum())
+    mi3 = torch.from_numpy(np.repeat(np.arange(E3, dtype=np.int32), padded3)).cuda()
+    a3, w13 = rnd8(M3, H3), rnd8(E3, 2 * I3, H3)
+    o13 = torch.empty((M3, 2 * I3), dtype=torch.bfloat16, device="cuda")
+    ea3, ew13 = e8(H3 // 128, M3), e8(E3, 2 * I3 // 128, H3 // 128)
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a3, ea3.T), (w13, ew13), o13, mi3), [()], iters, warmup)
+    out["grouped_config3_up_gate_ue8m0"] = {"flop": 2.0 * 8192 * H3 * 2 * I3, "ms": ms, "padded_rows": M3}
+    del a3, w13, o13
+    a23, w23 = rnd8(M3, I3), rnd8(E3, H3, I3)
+    o33 = torch.empty((M3, H3), dtype=torch.bfloat16, device="cuda")
+    ea23, ew23 = e8(I3 // 128, M3), e8(E3, H3 // 128, I3 // 128)
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a23, ea23.T), (w23, ew23), o33, mi3), [()], iters, warmup)
+    out["grouped_config3_down_ue8m0"] = {"flop": 2.0 * 8192 * I3 * H3, "ms": ms, "padded_rows": M3}
+    del a23, w23, o33
     # config 5 forward: E=128, H=4096, I=1408, 131072 routed rows, Zipf(1.0)
     E, H, I, ROUTED = 128, 4096, 1408, 131072
     counts, padded = zipf_counts(ROUTED, E, 1.0, seed=5, n_empty=0)
@@ -161,13 +186,19 @@ def bench_other_gemms(iters=10, warmup=3):
     o1 = torch.empty((Mp, 2 * I), dtype=torch.bfloat16, device="cuda")
     ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa.T), (w1, s1), o1, mi), [()], iters, warmup)
     out["grouped_config5_up_gate"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms, "padded_rows": Mp}
-    del w1, o1
+    ea5, ew5 = e8(H // 128, Mp), e8(E, 2 * I // 128, H // 128)
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, ea5.T), (w1, ew5), o1, mi), [()], iters, warmup)
+    out["grouped_config5_up_gate_ue8m0"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms, "padded_rows": Mp}
+    del w1, o1, ea5, ew5
     a2, sa2 = rnd8(Mp, I), torch.rand((Mp, I // 128), device="cuda")
     w2, s2 = rnd8(E, H, I), torch.rand((E, H // 128, I // 128), device="cuda")
     o3 = torch.empty((Mp, H), dtype=torch.bfloat16, device="cuda")
     ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a2, sa2), (w2, s2), o3, mi), [()], iters, warmup)
     out["grouped_config5_down"] = {"flop": 2.0 * ROUTED * I * H, "ms": ms, "padded_rows": Mp}
-    del a2, w2, o3
+    ea5, ew5 = e8(I // 128, Mp), e8(E, H // 128, I // 128)
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a2, ea5.T), (w2, ew5), o3, mi), [()], iters, warmup)
+    out["grouped_config5_down_ue8m0"] = {"flop": 2.0 * ROUTED * I * H, "ms": ms, "padded_rows": Mp}
+    del a2, w2, o3, ea5, ew5
     # config 5 weight gradient dW1[e] [H, 2I] += x_e^T . do1_e, all experts in one launch
     rows = [int(r) for r in padded]
     x = torch.randn((Mp, H), device="cuda").to(torch.bfloat16)

@@ -321,9 +321,11 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
 //   * All global addresses are a scalar base plus one per-lane 32-bit offset (the swizzled chunk a
 //     lane fetches does not depend on the copy index): 224 registers, MFMA results stay in VGPRs.
 //   * Every memory instruction of the loop is inline assembly so that vmcnt is counted by hand: per
-//     block a wavefront issues 4 scale loads and then 12 copies, loads retire in issue order, and
+//     block a wavefront issues 5 scale loads and then 12 copies, loads retire in issue order, and
 //     the wait before the barrier leaves exactly the 12 youngest copies outstanding (the stores of a
-//     finished tile are older than those and simply retire with them).
+//     finished tile are older than those and simply retire with them).  The scales land in VGPRs,
+//     the P block's too (every lane loads the same word): a value in flight may not be touched
+//     before its wait, and the compiler, unaware of the load, copies scalar registers freely.
 //   * The epilogue stages bf16 rows in the LDS stage the tile's last block has just left, 32 rows
 //     per wavefront at a time, and writes whole 256-byte rows.
 // ---------------------------------------------------------------------------------------------
@@ -395,6 +397,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         fq_ofs[h] = Q_OFS + swz(wq * 64 + li, 2 * kg + h);
     }
     const uint32_t s_off = SQL == 0 ? (uint32_t)(li * KB * 4) : (uint32_t)(li * 4);
+    uint32_t zero_off = 0;
+    asm volatile("" : "+v"(zero_off));     // a VGPR holding 0 for the scalar-base address form
 
     f32x4 acc[NPS][4];
     float fq_nxt[4], fpb_nxt = 0.f;
@@ -407,7 +411,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
 #define PF8_LOAD_S(sq_, sp_)                                                                           \
     _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                      \
         asm volatile("global_load_dword %0, %1, %2" : "=v"(fq_nxt[t]) : "v"(s_off), "s"((sq_) + t * sq_t) : "memory"); \
-    asm volatile("s_load_dword %0, %1, 0x0" : "=s"(fpb_nxt) : "s"(sp_) : "memory");
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(fpb_nxt) : "v"(zero_off), "s"(sp_) : "memory");
 #define PF8_PFRAG(ps_) ld_frag_lds(pbase + fp_ofs[0] + (ps_) * 2048, pbase + fp_ofs[1] + (ps_) * 2048)
 #define PF8_QFRAG(qs_) ld_frag_lds(pbase + fq_ofs[0] + (qs_) * 2048, pbase + fq_ofs[1] + (qs_) * 2048)
 
@@ -420,7 +424,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
 #pragma unroll
         for (int i = 0; i < 12; ++i) PF8_COPY(i, c_ptile + 128, c_qtile + 128, 1);
         asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)"
-                     : "+v"(fq_nxt[0]), "+v"(fq_nxt[1]), "+v"(fq_nxt[2]), "+v"(fq_nxt[3]), "+s"(fpb_nxt) : : "memory");
+                     : "+v"(fq_nxt[0]), "+v"(fq_nxt[1]), "+v"(fq_nxt[2]), "+v"(fq_nxt[3]), "+v"(fpb_nxt) : : "memory");
         __syncthreads();
         const uint8_t* pbase = lds;
         pf[0] = PF8_PFRAG(0);
@@ -431,11 +435,11 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     }
     int cur = 0;
     for (int64_t n = 0;; ++n) {
-        // coordinates of the next tile; its expert id is fetched by a scalar load that the first
-        // barrier wait of this tile covers, and its addresses are formed at the head of block 1
+        // coordinates of the next tile; its expert id is fetched by a scalar load that is waited for on
+        // the spot (once per tile), and its addresses are formed at the head of block 1
         const bool n_valid = tile_coords(n + 1, nq, np);
         int ne = 0;
-        if (n_valid && grouped) asm volatile("s_load_dword %0, %1, 0x0" : "=s"(ne) : "s"(a.m_indices + nq * BQ) : "memory");
+        if (n_valid && grouped) asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ne) : "s"(a.m_indices + nq * BQ) : "memory");
 #pragma unroll
         for (int i = 0; i < NPS; ++i)
 #pragma unroll
@@ -444,7 +448,6 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         for (int64_t kb = 0; kb < KB; ++kb) {
             if (kb == 1) {
                 if (n_valid) {
-                    asm volatile("" : "+s"(ne));      // the load above has been waited for in block 0
                     n_rows = ne < 0 ? 0 : BQ;
                     const int e = ne < 0 ? 0 : ne;
                     n_ptile = a.p + ((int64_t)e * a.Prows + np * 256) * a.red;
@@ -482,7 +485,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                     // they have returned, and this wavefront's copies of the next block with them,
                     // meet the other wavefronts
                     asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)"
-                                 : "+v"(fq_nxt[0]), "+v"(fq_nxt[1]), "+v"(fq_nxt[2]), "+v"(fq_nxt[3]), "+s"(fpb_nxt), "+s"(ne) : : "memory");
+                                 : "+v"(fq_nxt[0]), "+v"(fq_nxt[1]), "+v"(fq_nxt[2]), "+v"(fq_nxt[3]), "+v"(fpb_nxt) : : "memory");
                     __syncthreads();
                     __builtin_amdgcn_sched_barrier(0);
                 }
