@@ -192,16 +192,24 @@ int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_lay
  * and a multiple of 8); sb u8 [N/128, K/128] ([E, N/128, K/128] grouped), read as whole aligned
  * dwords.  M (Mtot) multiple of 128, N multiple of 256, K multiple of 128 and >= 384, ldo multiple
  * of 8; other shapes return PF8_EINVAL (decode the scales and use the fp32-scale entry points).
- * items_ws: DEVICE scratch of 4 + 4 * Mtot/128 int32, 16-byte aligned, that the call fills with its
- * list of 256-row work items (two 128-row blocks of one expert each); NULL makes the call walk
- * aligned 256-row tiles instead and visit those that hold two experts twice. */
+ * items: the list pf8_grouped_items_build made for this m_indices (two 128-row blocks of one expert
+ * per 256-row work item); with it the call also weighs the expert load and hands a GEMM whose
+ * experts are too small for 256-row tiles to the 128-row-tile kernel.  NULL makes the call walk
+ * aligned 256-row tiles and visit those that hold two experts twice. */
 int pf8_gemm_nt_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b,
                       const uint8_t* sb, int64_t M, int64_t N, int64_t K, uint16_t* out, int64_t ldo,
                       pf8_stream_t stream);
 int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa,
                                          const uint8_t* b, const uint8_t* sb, int E, int64_t Mtot,
                                          int64_t N, int64_t K, const int32_t* m_indices,
-                                         int32_t* items_ws, uint16_t* out, pf8_stream_t stream);
+                                         const int32_t* items, uint16_t* out, pf8_stream_t stream);
+
+/* Work-item list of the call above for one m_indices (the same list serves every GEMM that shares
+ * it: up+gate, down and the dgrad GEMMs of an MoE step): pairs the 128-row blocks of each expert
+ * into 256-row tiles, skipping padding blocks.  items: DEVICE buffer of 4 + 4 * Mtot/128 int32,
+ * 16-byte aligned.  No counterpart in the reference, whose deep_gemm schedules inside the binary. */
+int pf8_grouped_items_build(const int32_t* m_indices, int64_t Mtot, int32_t* items,
+                            pf8_stream_t stream);
 
 /* fp32 scales that are powers of two -> UE8M0 exponent bytes, elementwise (any layout).  not_pow2,
  * when non-null, is a DEVICE int the kernel adds the number of scales to that are negative, zero,

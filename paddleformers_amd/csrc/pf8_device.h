@@ -243,4 +243,15 @@ __device__ __forceinline__ float expf_fixed(float x) {
 // silu(g) = g / (1 + exp(-g)), IEEE division
 __device__ __forceinline__ float silu_exact(float g) { return g / (1.0f + expf_fixed(-g)); }
 
+// Contiguous-grouped GEMM with UE8M0 scales: which of the two kernels takes an expert load, from the
+// work-item list's header {paired 256-row items, 128-row blocks}.  Rounds of tiles per compute unit,
+// a 256x256 block costing 1.6 times a 128x256 one (measured): few blocks per expert leave many
+// paired tiles half empty, and then the smaller tile wins.  Both kernels evaluate this on entry and
+// the one that loses returns (a host-side choice would need the row counts).
+__device__ __forceinline__ bool e8_paired_tiles_win(const int32_t* list_header, int64_t p_tiles, int64_t cus) {
+    const int64_t n = list_header[0], nb = list_header[1];
+    const int64_t rounds_pair = (n * p_tiles + cus - 1) / cus, rounds_128 = (nb * p_tiles + cus - 1) / cus;
+    return 16 * rounds_pair <= 10 * rounds_128;
+}
+
 }  // namespace pf8

@@ -17,6 +17,8 @@
 // 128(P) x 128(Q) x 128(K), each wavefront 64x64 = 4x4 MFMA tiles, operands staged through
 // registers into two 32 KB LDS stages).  LDS rows are 128 B with their 16-byte chunks XOR-swizzled
 // so that fragment reads (16 rows x 32 B per quarter-wave) are bank-conflict free.
+#include <type_traits>
+
 #include "pf8_device.h"
 #include "pf8_host.h"
 
@@ -41,6 +43,9 @@ struct GemmArgs {
     const int32_t* m_indices;   // GROUP_CONTIG: expert per row
     const int32_t* masked_m;    // GROUP_MASKED: valid rows per expert
     int32_t tile_start[257];    // GROUP_WGRAD: first 128-row block of each expert along the reduction axis
+    int64_t ldsq;               // UE8M0 forward: bytes between the K blocks of sq (0 = Qrows)
+    const int32_t* pair_list;   // UE8M0 forward: when set, the kernel runs only if the paired-tile kernel declines
+    int cus;                    //   (header of its work-item list, compute units both assume)
 };
 
 #ifndef PF8_SWZ
@@ -333,8 +338,16 @@ __device__ __forceinline__ void dma16_s(uint32_t voff, const uint8_t* sbase, uin
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase), "s"(lds_dst) : "memory");
 }
 
-template <int SQL>
+// SF = 1: the scales are UE8M0 exponent bytes (sq [KB, ldsq], sp [E][Prows/128, KB]) instead of floats;
+// the kernel is the same, a scale is decoded where the block's factors are formed.
+__device__ __forceinline__ float e8m0_to_f32(uint32_t b) { return u2f(b ? b << 23 : 0x00400000u); }
+
+template <int SQL, int SF = 0>
 __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
+    using ST = typename std::conditional<SF == 1, uint8_t, float>::type;
+    if (SF == 1 && a.pair_list && e8_paired_tiles_win(a.pair_list, a.Prows / 256, a.cus)) return;
+    const ST* const sp_base = reinterpret_cast<const ST*>(a.sp);
+    const ST* const sq_base = reinterpret_cast<const ST*>(a.sq);
     constexpr int BQ = 128, NPS = 8;
     constexpr int STAGE = 49152, Q_OFS = 32768;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -374,12 +387,12 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     if (ce < 0) ce = 0;
     const uint8_t* c_ptile = a.p + ((int64_t)ce * a.Prows + cp * 256) * a.red;
     const uint8_t* c_qtile = a.q + cq * BQ * a.red;
-    const float* c_spb = a.sp + ((int64_t)ce * PB + cp * 2 + wp) * KB;
-    const float* c_sq0 = SQL == 0 ? a.sq + (cq * BQ + wq * 64) * KB : a.sq + cq * BQ + wq * 64;
+    const ST* c_spb = sp_base + ((int64_t)ce * PB + cp * 2 + wp) * KB;
+    const ST* c_sq0 = SQL == 0 ? sq_base + (cq * BQ + wq * 64) * KB : sq_base + cq * BQ + wq * 64;
     const uint8_t* n_ptile = c_ptile;
     const uint8_t* n_qtile = c_qtile;
-    const float* n_spb = c_spb;
-    const float* n_sq0 = c_sq0;
+    const ST* n_spb = c_spb;
+    const ST* n_sq0 = c_sq0;
     int n_rows = 0;
 
     // copy i of a wavefront fills rows (4 i + wave) * 8 + (lane >> 3) of the tile; the 16-byte chunk a
@@ -388,7 +401,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     const uint32_t c_off = (uint32_t)((wave * 8 + crow) * a.red + ((cpos ^ swz_key(wave * 8 + crow)) << 4));
     const int64_t copy_step = 32 * a.red;                       // 32 rows between copy i and i+1
     const int64_t sq_t = SQL == 0 ? 16 * KB : 16;               // floats between the scale rows of t and t+1
-    const int64_t sq_k = SQL == 0 ? 1 : q_rows_total;           // floats between K blocks
+    const int64_t sq_k = SQL == 0 ? 1 : (SF == 1 && a.ldsq ? a.ldsq : q_rows_total);   // scales between K blocks
     const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
     int fp_ofs[2], fq_ofs[2];
 #pragma unroll
@@ -396,7 +409,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         fp_ofs[h] = swz(wp * 128 + li, 2 * kg + h);
         fq_ofs[h] = Q_OFS + swz(wq * 64 + li, 2 * kg + h);
     }
-    const uint32_t s_off = SQL == 0 ? (uint32_t)(li * KB * 4) : (uint32_t)(li * 4);
+    const uint32_t s_off = (SQL == 0 ? (uint32_t)(li * KB) : (uint32_t)li) * (uint32_t)sizeof(ST);
     uint32_t zero_off = 0;
     asm volatile("" : "+v"(zero_off));     // a VGPR holding 0 for the scalar-base address form
 
@@ -410,8 +423,10 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     } while (0)
 #define PF8_LOAD_S(sq_, sp_)                                                                           \
     _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                      \
-        asm volatile("global_load_dword %0, %1, %2" : "=v"(fq_nxt[t]) : "v"(s_off), "s"((sq_) + t * sq_t) : "memory"); \
-    asm volatile("global_load_dword %0, %1, %2" : "=v"(fpb_nxt) : "v"(zero_off), "s"(sp_) : "memory");
+        if (SF == 1) asm volatile("global_load_ubyte %0, %1, %2" : "=v"(fq_nxt[t]) : "v"(s_off), "s"((sq_) + t * sq_t) : "memory"); \
+        else asm volatile("global_load_dword %0, %1, %2" : "=v"(fq_nxt[t]) : "v"(s_off), "s"((sq_) + t * sq_t) : "memory"); \
+    if (SF == 1) asm volatile("global_load_ubyte %0, %1, %2" : "=v"(fpb_nxt) : "v"(zero_off), "s"(sp_) : "memory"); \
+    else asm volatile("global_load_dword %0, %1, %2" : "=v"(fpb_nxt) : "v"(zero_off), "s"(sp_) : "memory");
 #define PF8_PFRAG(ps_) ld_frag_lds(pbase + fp_ofs[0] + (ps_) * 2048, pbase + fp_ofs[1] + (ps_) * 2048)
 #define PF8_QFRAG(qs_) ld_frag_lds(pbase + fq_ofs[0] + (qs_) * 2048, pbase + fq_ofs[1] + (qs_) * 2048)
 
@@ -452,8 +467,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                     const int e = ne < 0 ? 0 : ne;
                     n_ptile = a.p + ((int64_t)e * a.Prows + np * 256) * a.red;
                     n_qtile = a.q + nq * BQ * a.red;
-                    n_spb = a.sp + ((int64_t)e * PB + np * 2 + wp) * KB;
-                    n_sq0 = SQL == 0 ? a.sq + (nq * BQ + wq * 64) * KB : a.sq + nq * BQ + wq * 64;
+                    n_spb = sp_base + ((int64_t)e * PB + np * 2 + wp) * KB;
+                    n_sq0 = SQL == 0 ? sq_base + (nq * BQ + wq * 64) * KB : sq_base + nq * BQ + wq * 64;
                 } else {
                     // past the last tile the copies and scale loads re-read this tile's first blocks:
                     // the same instruction count in every block keeps the vmcnt arithmetic fixed
@@ -462,13 +477,14 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
             }
             float fq_cur[4];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) fq_cur[t] = fq_nxt[t] * fpb_nxt;
+            for (int t = 0; t < 4; ++t)
+                fq_cur[t] = SF == 1 ? e8m0_to_f32(f2u(fq_nxt[t])) * e8m0_to_f32(f2u(fpb_nxt)) : fq_nxt[t] * fpb_nxt;
             const int nxt1 = cur == 2 ? 0 : cur + 1;         // stage of the next block
             const int nxt2 = cur >= 1 ? cur - 1 : cur + 2;   // stage the previous block used
             // scales of the next block, copies of the block after it: this tile's, or the next tile's
             const bool in1 = kb + 1 < KB, in2 = kb + 2 < KB;
-            const float* s_sq = in1 ? c_sq0 + (kb + 1) * sq_k : n_sq0;
-            const float* s_sp = in1 ? c_spb + (kb + 1) : n_spb;
+            const ST* s_sq = in1 ? c_sq0 + (kb + 1) * sq_k : n_sq0;
+            const ST* s_sp = in1 ? c_spb + (kb + 1) : n_spb;
             const uint8_t* cp_p = in2 ? c_ptile + (kb + 2) * 128 : n_ptile + (kb + 2 - KB) * 128;
             const uint8_t* cp_q = in2 ? c_qtile + (kb + 2) * 128 : n_qtile + (kb + 2 - KB) * 128;
             PF8_LOAD_S(s_sq, s_sp)
@@ -826,9 +842,28 @@ static int ensure_lds_attr() {
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
     done = 1;
     return PF8_OK;
+}
+
+int pf8_launch_deep_ue8m0(const uint8_t* p, const uint8_t* q, const uint8_t* sp8, const uint8_t* sq8, int64_t ldsq, void* out,
+                          int64_t Prows, int64_t Qrows, int64_t red, int E, const int32_t* m_indices, const int32_t* pair_list,
+                          hipStream_t stream, const char* where) {
+    if (Prows % 256 != 0 || Qrows % 128 != 0 || red % 128 != 0 || red < 384) return pf8_fail(PF8_EINVAL, where, "shape outside the persistent kernel's tiling");
+    int rc = ensure_lds_attr();
+    if (rc) return rc;
+    GemmArgs g = {};
+    g.p = p; g.q = q; g.sp = reinterpret_cast<const float*>(sp8); g.sq = reinterpret_cast<const float*>(sq8); g.out = out;
+    g.Prows = Prows; g.Qrows = Qrows; g.red = red; g.ldo = Prows; g.sq_layout = 1; g.group = GROUP_CONTIG; g.E = E;
+    g.m_indices = m_indices; g.ldsq = ldsq; g.pair_list = pair_list; g.cus = pf8_effective_cus();
+    const int64_t T128 = (Prows / 256) * (Qrows / 128), per_xcd = (T128 + 7) / 8;
+    int64_t w = pf8_effective_cus() / 8;
+    if (w < 1) w = 1;
+    if (w > per_xcd) w = per_xcd;
+    hipLaunchKernelGGL((k_gemm_fwd_deep<1, 1>), dim3((unsigned)(8 * w)), dim3(256), 147456, stream, g);
+    return pf8_check_launch(where);
 }
 
 extern "C" int pf8_gemm_nt(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b, const float* sb, int64_t M,

@@ -43,7 +43,8 @@ struct E8Args {
     int64_t Prows, Qrows, red, ldo, ldsq;
     int grouped;
     const int32_t* m_indices;
-    const int32_t* items;   // grouped: {n, -, -, -} then {block0, block1 or -1, expert, -} per item; may be null
+    const int32_t* items;   // grouped: {n, blocks, -, -} then {block0, block1 or -1, expert, -} per item; may be null
+    int cus;
 };
 
 __device__ __forceinline__ int e8_keyp(int row) { return (row & 7) ^ ((row >> 3) & 1); }
@@ -90,6 +91,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     constexpr int BAR = 44, CSTEP = 2;     // barrier position; MFMAs between two copies
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     asm volatile("" ::: "a255");
+    if (a.items && !e8_paired_tiles_win(a.items, a.Prows / 256, a.cus)) return;   // left to the 128-row-tile kernel
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wq = wave >> 1, wp = wave & 1;
@@ -366,13 +368,17 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
 // One workgroup of 1024 threads, each walking a contiguous run of blocks; two scans over the threads:
 // the parity of a block inside its expert's segment (a composition of {reset, flip} functions), then
 // the number of items opened before it (an item opens at every even block of a segment).
-// items = {n, 0, 0, 0} followed by {block0, block1 or -1, expert, 0} per item.
+// items = {n, number of 128-row blocks, 0, 0} followed by {block0, block1 or -1, expert, 0} per item.
 __global__ __launch_bounds__(1024) void k_e8_build_items(const int32_t* __restrict__ m_indices, int64_t NB, int32_t* __restrict__ items) {
+    constexpr int CACHE = 8192;                 // expert ids of the first blocks, read from memory once
     __shared__ int s_scan[2][1024];
+    __shared__ int s_e[CACHE];
     const int tid = threadIdx.x;
+    for (int64_t b = tid; b < NB && b < CACHE; b += 1024) s_e[b] = m_indices[b * 128];
+    __syncthreads();
     const int64_t chunk = (NB + 1023) / 1024;
     const int64_t lo = tid * chunk < NB ? tid * chunk : NB, hi = lo + chunk < NB ? lo + chunk : NB;
-    auto expert = [&](int64_t b) -> int { return (b < 0 || b >= NB) ? -2 : m_indices[b * 128]; };
+    auto expert = [&](int64_t b) -> int { return (b < 0 || b >= NB) ? -2 : (b < CACHE ? s_e[b] : m_indices[b * 128]); };
     // function codes: bit 1 = constant, bit 0 = its value (constant) or flip (otherwise); g after f:
     auto then = [](int f, int g) -> int { return (g & 2) ? g : (f ^ (g & 1)); };
     auto step_fn = [&](int prev_e, int e) -> int { return e < 0 ? 3 : (e != prev_e ? 2 : 1); };
@@ -389,7 +395,7 @@ __global__ __launch_bounds__(1024) void k_e8_build_items(const int32_t* __restri
         __syncthreads();
     }
     const int f_in = tid ? s_scan[cur][tid - 1] : 0;
-    int par = (f_in & 2) ? (f_in & 1) : (1 ^ (f_in & 1));     // parity of the block before `lo` (1 = none open)
+    const int par = (f_in & 2) ? (f_in & 1) : (1 ^ (f_in & 1));     // parity of the block before `lo` (1 = none open)
     __syncthreads();
     // items opened in this run of blocks
     int opened = 0, p = par;
@@ -410,7 +416,7 @@ __global__ __launch_bounds__(1024) void k_e8_build_items(const int32_t* __restri
         __syncthreads();
     }
     int t = (tid ? s_scan[cur][tid - 1] : 0) - 1;     // index of the item open before `lo`
-    if (tid == 1023) { items[0] = s_scan[cur][1023]; items[1] = 0; items[2] = 0; items[3] = 0; }
+    if (tid == 1023) { items[0] = s_scan[cur][1023]; items[1] = (int32_t)NB; items[2] = 0; items[3] = 0; }
     p = par;
     pe = expert(lo - 1);
     for (int64_t b = lo; b < hi; ++b) {
@@ -492,7 +498,7 @@ extern "C" int pf8_gemm_nt_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ld
 
 extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b,
                                                     const uint8_t* sb, int E, int64_t Mtot, int64_t N, int64_t K,
-                                                    const int32_t* m_indices, int32_t* items_ws, uint16_t* out,
+                                                    const int32_t* m_indices, const int32_t* items, uint16_t* out,
                                                     pf8_stream_t stream) {
     PF8_REQUIRE(E >= 0 && Mtot >= 0 && N >= 0 && K >= 0, "negative shape");
     int rc = check_e8_shapes(__func__, Mtot, N, K, ldsa);
@@ -505,15 +511,26 @@ extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint
     E8Args g = {};
     g.p = b; g.q = a; g.sp8 = sb; g.sq8 = sa; g.out = out;
     g.Prows = N; g.Qrows = Mtot; g.red = K; g.ldo = N; g.ldsq = ldsa; g.grouped = 1; g.m_indices = m_indices;
-    if (items_ws) {
-        PF8_REQUIRE((reinterpret_cast<uintptr_t>(items_ws) & 15u) == 0, "items_ws must be 16-byte aligned");
-        hipLaunchKernelGGL(k_e8_build_items, dim3(1), dim3(1024), 0, (hipStream_t)stream, m_indices, Mtot / 128, items_ws);
-        rc = pf8_check_launch(__func__);
+    if (items) {
+        // both kernels are launched; each decides on entry, from the list's header, whether this expert
+        // load is its own, and the other returns at once
+        PF8_REQUIRE((reinterpret_cast<uintptr_t>(items) & 15u) == 0, "items must be 16-byte aligned");
+        g.items = items;
+        g.cus = pf8_effective_cus();
+        rc = launch_e8(g, Mtot / 128, (hipStream_t)stream, __func__);
         if (rc) return rc;
-        g.items = items_ws;
-        return launch_e8(g, Mtot / 128, (hipStream_t)stream, __func__);
+        return pf8_launch_deep_ue8m0(b, a, sb, sa, ldsa, out, N, Mtot, K, E, m_indices, items, (hipStream_t)stream, __func__);
     }
     return launch_e8(g, (Mtot + 255) / 256, (hipStream_t)stream, __func__);
+}
+
+extern "C" int pf8_grouped_items_build(const int32_t* m_indices, int64_t Mtot, int32_t* items, pf8_stream_t stream) {
+    PF8_REQUIRE(Mtot >= 0 && Mtot % 128 == 0, "Mtot must be a non-negative multiple of 128");
+    PF8_REQUIRE(items && (reinterpret_cast<uintptr_t>(items) & 15u) == 0, "items must be a 16-byte aligned buffer");
+    PF8_REQUIRE(Mtot == 0 || m_indices, "null pointer");
+    PF8_REQUIRE(Mtot / 128 <= 0x3FFFFFFFll, "too many rows");
+    hipLaunchKernelGGL(k_e8_build_items, dim3(1), dim3(1024), 0, (hipStream_t)stream, m_indices, Mtot / 128, items);
+    return pf8_check_launch(__func__);
 }
 
 extern "C" int pf8_scales_to_ue8m0(const float* s, int64_t n, uint8_t* out, int* not_pow2, pf8_stream_t stream) {

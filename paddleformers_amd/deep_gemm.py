@@ -124,11 +124,25 @@ def fp8_gemm_nt(a, b, out: torch.Tensor, c: Optional[torch.Tensor] = None, recip
     return out
 
 
-def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.Tensor):
+def build_group_items(m_indices: torch.Tensor) -> torch.Tensor:
+    """Work-item list of the UE8M0 grouped GEMM for one m_indices (int32 [Mtot], Mtot a multiple of 128):
+    pass it as `items=` to every m_grouped_fp8_gemm_nt_contiguous call that shares the m_indices
+    (up+gate, down, dgrad).  No counterpart in the reference API; without it each call builds its own."""
+    _dev(m_indices, "m_indices")
+    if m_indices.dtype != torch.int32 or m_indices.numel() % 128 != 0:
+        raise ValueError("m_indices must be int32 with a multiple of 128 entries")
+    m_indices = m_indices if m_indices.is_contiguous() else m_indices.contiguous()
+    items = torch.empty(4 + 4 * (m_indices.numel() // 128), dtype=torch.int32, device=m_indices.device)
+    _lib.call("pf8_grouped_items_build", _p(m_indices), m_indices.numel(), _p(items), _stream())
+    return items
+
+
+def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.Tensor, items: Optional[torch.Tensor] = None):
     """Grouped GEMM over rows sorted by expert: row m uses b[m_indices[m]].
 
     transformers/fp8_utils.py:949-954: a [Mtot, K] + sa [Mtot, K/128] (any strides), b [E, N, K] +
     sb [E, N/128, K/128], m_indices int32 [Mtot]; every expert segment is a multiple of 128 rows.
+    `items` (optional, UE8M0 scales only): the list build_group_items made for this m_indices.
     """
     (ta, sa), (tb, sb) = _check_pair(a, "a"), _check_pair(b, "b")
     _dev(out, "out")
@@ -158,7 +172,10 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
         if _ue8m0_kernel_shape(Mtot, N, K):
             sa_k = _ue8m0_kmajor(sa, Mtot, K // 128, "a scale")
             sb_k = sb.view(torch.uint8).contiguous()
-            items = torch.empty(4 + 4 * (Mtot // 128), dtype=torch.int32, device=ta.device)
+            if items is None:
+                items = build_group_items(m_indices)
+            elif items.dtype != torch.int32 or items.numel() != 4 + 4 * (Mtot // 128) or not items.is_contiguous():
+                raise ValueError("items must come from build_group_items for this m_indices")
             _lib.call("pf8_grouped_gemm_nt_contiguous_ue8m0", _p(ta), _p(sa_k), sa_k.stride(0), _p(tb), _p(sb_k), E, Mtot, N, K,
                       _p(m_indices), _p(items), _p(out), _stream())
             return out

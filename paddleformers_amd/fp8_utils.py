@@ -87,9 +87,15 @@ def _get_fp8_weight_and_scale(weight, stacked=False, transpose=False):
     return weight.fp8_weight, weight.fp8_scale
 
 
-def fused_stack_quant(expert_weight_list, transpose=False):
-    """fp8_utils.py:91-102: use the per-step cache on expert 0's weight when present, else quantise."""
+def fused_stack_quant(expert_weight_list, transpose=False, using_pow2_scale=False):
+    """fp8_utils.py:91-102: use the per-step cache on expert 0's weight when present, else quantise.
+    using_pow2_scale asks for power-of-two scales (the `use_ue8m0` mode): a cache written without
+    them is refused rather than silently truncated."""
     w0 = expert_weight_list[0]
+    cached = hasattr(w0, "fp8_weight_stacked") or hasattr(w0, "fp8_weight_stacked_transpose")
+    if using_pow2_scale and cached and not getattr(w0, "fp8_scale_is_pow2", False):
+        raise RuntimeError("the cached FP8 expert weights do not carry power-of-two scales: "
+                           "call fp8_quant_weight(..., using_pow2_scale=True) for use_ue8m0")
     if transpose and hasattr(w0, "fp8_weight_stacked_transpose"):
         return _get_fp8_weight_and_scale(w0, stacked=True, transpose=True)
     if not transpose and hasattr(w0, "fp8_weight_stacked"):
@@ -99,7 +105,7 @@ def fused_stack_quant(expert_weight_list, transpose=False):
         return _get_fp8_weight_and_scale(w0, stacked=True, transpose=False)
     if hasattr(w0, "fp8_weight_stacked_transpose"):
         return _get_fp8_weight_and_scale(w0, stacked=True, transpose=True)
-    return F8.fused_stack_transpose_quant(expert_weight_list, transpose=transpose)
+    return F8.fused_stack_transpose_quant(expert_weight_list, transpose=transpose, using_pow2_scale=using_pow2_scale)
 
 
 def weight_quant(weight, transpose=False):
@@ -136,14 +142,15 @@ def cache_fp8_weight(weight, quant_transpose=None):
         raise ValueError("quant_transpose must be either True, False or None.")
 
 
-def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_transpose=None):
+def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_transpose=None, using_pow2_scale=False):
     """DeepseekV2MoE.fp8_quant_weight (cli/train/deepseek_v3_pretrain/modeling.py:506-567), the body
     FP8QuantWeightCallback.on_step_begin runs once per optimizer step: attach the stacked FP8 copies
     of the expert weights to the first weight of each list (batch mode) or to every weight.
 
     quant_transpose None caches both orientations; here they come from one read of the weights
     (`fused_stack_quant_both`) instead of two passes.  Weights that already carry a cache are left
-    alone, as in the reference."""
+    alone, as in the reference.  using_pow2_scale (for `use_ue8m0`, transformers/configuration_utils.py:454-459)
+    rounds every scale up to a power of two and marks the cache so."""
 
     def quantize_weights(weight_list, weight_obj=None):
         if weight_obj is None:
@@ -151,16 +158,18 @@ def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_tra
         if hasattr(weight_obj, "fp8_weight_stacked") or hasattr(weight_obj, "fp8_weight_stacked_transpose"):
             return
         if quant_transpose is None:
-            q, s, qt, st = F8.fused_stack_quant_both(weight_list)
+            q, s, qt, st = F8.fused_stack_quant_both(weight_list, using_pow2_scale=using_pow2_scale)
             weight_obj.fp8_weight_stacked, weight_obj.fp8_scale_stacked = q, s
             weight_obj.fp8_weight_stacked_transpose, weight_obj.fp8_scale_stacked_transpose = qt, st
         elif quant_transpose is False:
-            weight_obj.fp8_weight_stacked, weight_obj.fp8_scale_stacked = F8.fused_stack_transpose_quant(weight_list, transpose=False)
+            weight_obj.fp8_weight_stacked, weight_obj.fp8_scale_stacked = F8.fused_stack_transpose_quant(
+                weight_list, transpose=False, using_pow2_scale=using_pow2_scale)
         elif quant_transpose is True:
             weight_obj.fp8_weight_stacked_transpose, weight_obj.fp8_scale_stacked_transpose = F8.fused_stack_transpose_quant(
-                weight_list, transpose=True)
+                weight_list, transpose=True, using_pow2_scale=using_pow2_scale)
         else:
             raise ValueError("Invalid value for `quant_transpose`.")
+        weight_obj.fp8_scale_is_pow2 = bool(using_pow2_scale)
 
     w1s = [w for w in expert_w1_list if w is not None]
     w2s = [w for w in expert_w2_list if w is not None]
@@ -545,11 +554,17 @@ class FP8GroupGemmMlpFunctionNode:
     """
 
     def __init__(self, custom_map, recompute_fwd_gate_up=False, is_split_group_gemm=False,
-                 name="experts_group_gemm_contiguous_node"):
+                 name="experts_group_gemm_contiguous_node", use_ue8m0=False):
         self.experts = custom_map.experts
         self.recompute_fwd_gate_up = recompute_fwd_gate_up
         self.is_split_group_gemm = is_split_group_gemm
         self.name = name
+        # use_ue8m0 (transformers/configuration_utils.py:454-459): every operand of the four forward-type
+        # grouped GEMMs is quantized with power-of-two scales and the GEMMs take them as UE8M0 bytes
+        # (block-scaled MFMA kernel).  Pre-quantized inputs handed in as (fp8, scale) pairs must then
+        # carry power-of-two scales as well.
+        self.use_ue8m0 = use_ue8m0
+        self._group_items = None
         self.m_indices = None
         self.input = None
         self.input_fp8 = None
@@ -561,6 +576,7 @@ class FP8GroupGemmMlpFunctionNode:
 
     def reset_statue(self):
         self.m_indices = None
+        self._group_items = None
         self.fwd_subbatch = None
         self.bwd_subbatch = None
         self.clear_activation_tensors()
@@ -578,9 +594,22 @@ class FP8GroupGemmMlpFunctionNode:
         counts = torch.tensor([int(t) for t in tokens_per_expert], dtype=torch.int64)
         return torch.repeat_interleave(torch.arange(len(tokens_per_expert), dtype=torch.int32), counts).to(dev)
 
-    @staticmethod
-    def _stacked(expert_w, transpose, num_expert):
-        q, s = fused_stack_quant(expert_w, transpose=transpose)
+    def _grouped_gemm(self, a_fp8, a_scale, w_fp8, w_scale, out, m_indices):
+        """One forward-type grouped GEMM of the node; with use_ue8m0 the (power-of-two) scales go in as
+        exponent bytes and the work-item list of the node's own m_indices is built once and shared."""
+        if not self.use_ue8m0:
+            deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, a_scale), (w_fp8, w_scale), out, m_indices)
+            return
+        items = None
+        if m_indices is self.m_indices and a_fp8.shape[0] % 128 == 0:
+            if self._group_items is None:
+                self._group_items = deep_gemm.build_group_items(m_indices)
+            items = self._group_items
+        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, F8.scales_to_ue8m0(a_scale, check=False)),
+                                                   (w_fp8, F8.scales_to_ue8m0(w_scale, check=False)), out, m_indices, items=items)
+
+    def _stacked(self, expert_w, transpose, num_expert):
+        q, s = fused_stack_quant(expert_w, transpose=transpose, using_pow2_scale=self.use_ue8m0)
         q = q.reshape([num_expert, -1, q.shape[-1]])
         s = s.reshape([num_expert, -1, s.shape[-1]])
         w0 = expert_w[0]
@@ -602,15 +631,15 @@ class FP8GroupGemmMlpFunctionNode:
             x_fp8, x_scale = x
             x_scale = x_scale.t().contiguous().t()
         else:
-            x_fp8, x_scale = F8.fp8_quant_blockwise(x, output_scale_transpose=True, quant_method="1x128", input_transpose=False)
+            x_fp8, x_scale = F8.fp8_quant_blockwise(x, output_scale_transpose=True, quant_method="1x128", input_transpose=False,
+                                                    using_pow2_scale=self.use_ue8m0)
             x_scale = x_scale.T
         o1 = torch.empty([x_fp8.shape[0], w1_t_quant.shape[1]], dtype=expert_w1[0].dtype, device=x_fp8.device)
         if numpy.prod(x_fp8.shape) != 0:
             if self.is_split_group_gemm:
                 split_group_gemm(x_fp8, x_scale, w1_t_quant, w1_t_scale, tokens_per_expert, o1)
             else:
-                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((x_fp8, x_scale), (w1_t_quant, w1_t_scale), o1,
-                                                           self.m_indices if m_indices is None else m_indices)
+                self._grouped_gemm(x_fp8, x_scale, w1_t_quant, w1_t_scale, o1, self.m_indices if m_indices is None else m_indices)
         if m_indices is None:
             self.input_fp8 = x_fp8
             self.input_scale = x_scale
@@ -633,8 +662,7 @@ class FP8GroupGemmMlpFunctionNode:
             if self.is_split_group_gemm:
                 split_group_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, tokens_per_expert, o3)
             else:
-                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2_fp8, o2_scale), (w2_quant, w2_scale), o3,
-                                                           m_indices if self.fwd_subbatch else self.m_indices)
+                self._grouped_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, o3, m_indices if self.fwd_subbatch else self.m_indices)
         return o3
 
     def bwd_dowm_input(self, expert_w2, unzipped_grad, o1, tokens_per_expert, m_indices=None, unzipped_probs=None):
@@ -645,22 +673,24 @@ class FP8GroupGemmMlpFunctionNode:
             unzipped_grad_scale = unzipped_grad_scale.t().contiguous().t()
         else:
             unzipped_grad_fp8, unzipped_grad_scale = F8.fp8_quant_blockwise(unzipped_grad, output_scale_transpose=True,
-                                                                            quant_method="1x128", input_transpose=False)
+                                                                            quant_method="1x128", input_transpose=False,
+                                                                            using_pow2_scale=self.use_ue8m0)
             unzipped_grad_scale = unzipped_grad_scale.T
         do2_s = torch.empty([unzipped_grad_fp8.shape[0], bw_w2_quant.shape[1]], dtype=torch.bfloat16, device=o1.device)
         if numpy.prod(unzipped_grad_fp8.shape) != 0:
             if self.is_split_group_gemm:
                 split_group_gemm(unzipped_grad_fp8, unzipped_grad_scale, bw_w2_quant, bw_w2_scale, tokens_per_expert, do2_s)
             else:
-                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((unzipped_grad_fp8, unzipped_grad_scale), (bw_w2_quant, bw_w2_scale),
-                                                           do2_s, m_indices if self.bwd_subbatch else self.m_indices)
+                self._grouped_gemm(unzipped_grad_fp8, unzipped_grad_scale, bw_w2_quant, bw_w2_scale, do2_s,
+                                   m_indices if self.bwd_subbatch else self.m_indices)
         do1, probs_grad, o2_s = F8.fused_swiglu_weighted_bwd(o1, do2_s, unzipped_probs)
         return do1, o2_s, probs_grad
 
     def bwd_gate_up_input(self, do1, expert_w1, tokens_per_expert, m_indices=None, dx=None):
         """dx [m_sum, H] = do1 . w1^T (fp8_utils.py:1058-1094)."""
         bw_w1_quant, bw_w1_scale = self._stacked(expert_w1, False, len(expert_w1))
-        do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, output_scale_transpose=True, quant_method="1x128", input_transpose=False)
+        do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, output_scale_transpose=True, quant_method="1x128", input_transpose=False,
+                                                    using_pow2_scale=self.use_ue8m0)
         do1_scale = do1_scale.T
         dx_shape = [do1_fp8.shape[0], bw_w1_quant.shape[1]]
         if dx is None or dx.dtype != do1.dtype:
@@ -671,8 +701,7 @@ class FP8GroupGemmMlpFunctionNode:
             if self.is_split_group_gemm:
                 split_group_gemm(do1_fp8, do1_scale, bw_w1_quant, bw_w1_scale, tokens_per_expert, dx)
             else:
-                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((do1_fp8, do1_scale), (bw_w1_quant, bw_w1_scale), dx,
-                                                           m_indices if self.bwd_subbatch else self.m_indices)
+                self._grouped_gemm(do1_fp8, do1_scale, bw_w1_quant, bw_w1_scale, dx, m_indices if self.bwd_subbatch else self.m_indices)
         return dx
 
     def fused_transpose_split_quant(self, x, scale, tokens_per_expert, pow_2_scales):

@@ -303,7 +303,7 @@ def scales_to_ue8m0(scale: torch.Tensor, check: bool = True) -> torch.Tensor:
     _dev(scale, "scale")
     if scale.dtype != torch.float32:
         raise ValueError("scale must be float32")
-    dense = scale if scale.is_contiguous() or scale.t().is_contiguous() else scale.contiguous()
+    dense = scale if scale.is_contiguous() or (scale.dim() == 2 and scale.t().is_contiguous()) else scale.contiguous()
     out = torch.empty_like(dense, dtype=torch.uint8)      # preserves the strides of a dense tensor
     if out.stride() != dense.stride():
         dense = dense.contiguous()

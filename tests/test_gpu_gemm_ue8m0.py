@@ -159,10 +159,21 @@ def _grouped_pow2_case(E, N, K, rows, seed):
     return a, sa, np.stack(bs), np.stack(sbs), np.repeat(np.arange(E, dtype=np.int32), rows)
 
 
+@pytest.fixture
+def few_cus(dg):
+    """Eight compute units: every workgroup walks many work items, and the cost estimate that picks
+    between the two tilings (rounds of tiles per compute unit) can favour the paired 256-row tiles, which
+    on the whole device these small cases always leave to the 128-row kernel."""
+    dg.set_num_sms(8)
+    yield
+    dg.set_num_sms(0)
+
+
 def _grouped_call(dg, a, sa, b, sb, m_idx, out, paired):
-    """paired: through the mirror, which lets the library pair each expert's 128-row blocks into tiles;
-    otherwise the raw C ABI without a work-item list (aligned 256-row tiles, two passes over a tile
-    that holds two experts)."""
+    """paired: through the mirror, which lets the library pair each expert's 128-row blocks into 256-row
+    tiles or hand the call to the 128-row-tile kernel, whichever its cost estimate prefers; otherwise
+    the raw C ABI without a work-item list (aligned 256-row tiles, two passes over a tile that holds
+    two experts)."""
     ta, tb, tm = G.to_torch_fp8(a), G.to_torch_fp8(b), torch.from_numpy(m_idx).cuda()
     if paired:
         dg.m_grouped_fp8_gemm_nt_contiguous((ta, _e8(sa)), (tb, _e8(sb)), out, tm)
@@ -181,7 +192,10 @@ def _grouped_call(dg, a, sa, b, sb, m_idx, out, paired):
 # an odd number of blocks, empty experts, a half tile at the end
 @pytest.mark.parametrize("rows", [[128, 256, 0, 128], [0, 0, 384], [128] * 6, [256, 512], [384, 128, 640, 128]])
 @pytest.mark.parametrize("paired", [True, False])
-def test_grouped_contiguous_ue8m0_vs_oracle(dg, rows, paired):
+@pytest.mark.parametrize("cus", ["all", "few"])
+def test_grouped_contiguous_ue8m0_vs_oracle(dg, request, rows, paired, cus):
+    if cus == "few":
+        request.getfixturevalue("few_cus")
     E, N, K = len(rows), 512, 512
     a, sa, b, sb, m_idx = _grouped_pow2_case(E, N, K, rows, seed=sum(rows) + E)
     Mtot = a.shape[0]
@@ -197,9 +211,12 @@ def test_grouped_contiguous_ue8m0_vs_oracle(dg, rows, paired):
         start += r
 
 
-def test_grouped_contiguous_ue8m0_many_small_experts(dg):
+@pytest.mark.parametrize("cus", ["all", "few"])
+def test_grouped_contiguous_ue8m0_many_small_experts(dg, request, cus):
     """40 experts of 0..5 blocks in Zipf-like disorder, some followed by padding blocks (index -1): every
     routed row is computed with its own expert's weights and every padding row is left alone."""
+    if cus == "few":
+        request.getfixturevalue("few_cus")
     rng = np.random.default_rng(12)
     E, N, K = 40, 256, 384
     rows = [int(128 * rng.integers(0, 6)) for _ in range(E)]

@@ -215,3 +215,74 @@ def test_moe_backward_grouped_wgrad_when_main_grads_are_stacked():
     # not stacked: one expert's gradient lives elsewhere
     experts[2].w1.main_grad = torch.zeros((H, 2 * I), dtype=torch.float32, device="cuda")
     assert FP8GroupGemmMlpFunctionNode._stacked_main_grad([e.w1 for e in experts]) is None
+
+
+# ---------------------------------------------------------------------------------------------
+# use_ue8m0: power-of-two scales everywhere, forward-type GEMMs on the block-scaled MFMA kernel
+# ---------------------------------------------------------------------------------------------
+
+
+def test_moe_node_ue8m0_forward_against_oracle_chain():
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 4, 512, 384
+    rows = [128, 0, 384, 256]
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=21)
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    o3 = node.forward(G.to_torch_bf16(x), tp, rows)
+    m_idx = np.repeat(np.arange(E, dtype=np.int32), rows)
+    xq, xs = O.quant_1x128(x, 0, pow2=True)
+    w1q, w1s = O.stack_transpose_quant(w1, transpose=True, pow2=True)
+    w2q, w2s = O.stack_transpose_quant(w2, transpose=True, pow2=True)
+    eo1 = O.grouped_gemm_nt_contiguous(xq, xs, w1q.reshape(E, 2 * I, H), w1s.reshape(E, 2 * I // 128, H // 128), m_idx)
+    o1 = G.from_torch_bf16(node.o1)
+    assert G.rel_fro(O.bf16_bits_to_f32(o1), O.bf16_bits_to_f32(eo1)) <= 1e-3
+    q2, s2 = O.swiglu_weighted_quant(o1, probs, 0, True)
+    eo3 = O.grouped_gemm_nt_contiguous(q2, s2, w2q.reshape(E, H, I), w2s.reshape(E, H // 128, I // 128), m_idx)
+    assert G.rel_fro(O.bf16_bits_to_f32(G.from_torch_bf16(o3)), O.bf16_bits_to_f32(eo3)) <= 1e-3
+    assert node._group_items is not None      # one work-item list served both GEMMs
+
+
+def test_moe_node_ue8m0_forward_backward_against_fp32_moe():
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 3, 512, 384
+    rows = [256, 0, 384]
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=27)
+    dout = G.bf16_normal((sum(rows), H), seed=29, std=1e-3)
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    o3 = node.forward(G.to_torch_bf16(x), tp, rows)
+    dx, pg = node.backward(G.to_torch_bf16(dout), tp, rows)
+    ref_o3, ref_dx, ref_pg, ref_dw1, ref_dw2 = _fp32_moe(x, probs, w1, w2, rows, dout)
+    # power-of-two scales cost up to one bit of the FP8 mantissa: a little above the 0.08 of the exact scales
+    assert G.rel_fro(o3.float().cpu().numpy(), ref_o3) < 0.10
+    assert G.rel_fro(dx.float().cpu().numpy(), ref_dx) < 0.10
+    assert G.rel_fro(pg.cpu().numpy(), ref_pg) < 0.10
+    for e, r in enumerate(rows):
+        if r:
+            assert G.rel_fro(experts[e].w1.main_grad.cpu().numpy(), ref_dw1[e].numpy()) < 0.10
+            assert G.rel_fro(experts[e].w2.main_grad.cpu().numpy(), ref_dw2[e].numpy()) < 0.10
+
+
+def test_moe_node_ue8m0_needs_a_pow2_weight_cache():
+    from paddleformers_amd import fp8_utils as U
+
+    E, H, I = 2, 512, 384
+    rows = [256, 256]
+    _, _, experts, x, probs = _make(E, H, I, rows, seed=31)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    plain = U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True).forward(G.to_torch_bf16(x), tp, rows)
+    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True)
+    with pytest.raises(RuntimeError):
+        U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True).forward(G.to_torch_bf16(x), tp, rows)
+    for e in experts:
+        for w in (e.w1, e.w2):
+            for name in ("fp8_weight_stacked", "fp8_scale_stacked", "fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose",
+                         "fp8_scale_is_pow2"):
+                if hasattr(w, name):
+                    delattr(w, name)
+    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True, using_pow2_scale=True)
+    cached = U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True).forward(G.to_torch_bf16(x), tp, rows)
+    assert torch.equal(plain.view(torch.int16), cached.view(torch.int16))
