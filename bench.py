@@ -280,6 +280,17 @@ def bench_other_gemms(iters=10, warmup=3):
 
     ms = time_kernel(fwd_bwd, [()], 3, 2)
     out["moe_node_config5_fwd_bwd"] = {"flop": 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H), "ms": ms}
+    # the same step with power-of-two scales throughout (use_ue8m0): forward and dgrad GEMMs on the block-scaled MFMA kernel
+    for ex in exps:
+        for w in (ex.w1, ex.w2):
+            for name in ("fp8_weight_stacked", "fp8_scale_stacked", "fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose",
+                         "fp8_scale_is_pow2"):
+                if hasattr(w, name):
+                    delattr(w, name)
+    U8.fp8_quant_weight([ex.w1 for ex in exps], [ex.w2 for ex in exps], batch_mode=True, using_pow2_scale=True)
+    node = U8.FP8GroupGemmMlpFunctionNode(mp, use_ue8m0=True)
+    ms = time_kernel(fwd_bwd, [()], 3, 2)
+    out["moe_node_config5_fwd_bwd_ue8m0"] = {"flop": 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H), "ms": ms}
     del node, exps, g1, g2, xin, dout
     for v in out.values():
         if "flop" in v:

@@ -96,6 +96,7 @@ struct TileScale {
     float r_lo;   // reciprocal of s nudged down by 2^-20 (relative)
     float r_hi;   // reciprocal of s nudged up by 2^-20
     bool slow;    // tile must take the IEEE division path (scale too small for a finite reciprocal)
+    bool exact;   // s is a power of two: r_lo == r_hi == 1/s exactly, and v * r_lo IS the correctly rounded v / s
 };
 
 // s = amax/448 (IEEE divide), amax == 0 -> 1; pow2: decode scale rounded up to a power of two.
@@ -106,13 +107,27 @@ __device__ __forceinline__ TileScale make_scale_from(float s) {
     t.r_lo = r * 0.99999904632568359375f;   // 1 - 2^-20
     t.r_hi = r * 1.00000095367431640625f;   // 1 + 2^-20
     t.slow = !(s >= 1.0e-30f);
+    t.exact = false;
     return t;
 }
+// 1/s of a power of two s = 2^k, k in [-126, 126] (what the pow2 rule below yields), by exponent arithmetic
+__device__ __forceinline__ float pow2_recip(float s) { return u2f(0x7F000000u - f2u(s)); }
 __device__ __forceinline__ TileScale make_scale(uint32_t amax_bits, bool pow2) {
     float amax = u2f(amax_bits);
     float s = amax / 448.0f;
     if (pow2) s = u2f((f2u(s) + 0x007FFFFFu) & 0x7F800000u);
     if (amax_bits == 0u) s = 1.0f;
+    if (pow2) {
+        // dividing by a power of two is multiplying by its (exact) reciprocal: the product is the
+        // correctly rounded quotient, so one conversion per element and no bracket to check.  (With
+        // the bracket every exact e4m3 tie, one bf16 value in 32, would take the division path.)
+        TileScale t;
+        t.s = s;
+        t.r_lo = t.r_hi = pow2_recip(s);
+        t.slow = false;
+        t.exact = true;
+        return t;
+    }
     return make_scale_from(s);
 }
 
@@ -162,7 +177,14 @@ __device__ __forceinline__ void quant8_fix(const float (&v)[8], float s, uint2& 
         }
     }
 }
+__device__ __forceinline__ uint2 quant8_exact(const float (&v)[8], float r) {
+    uint2 o;
+    o.x = pack4_e4m3(v[0] * r, v[1] * r, v[2] * r, v[3] * r);
+    o.y = pack4_e4m3(v[4] * r, v[5] * r, v[6] * r, v[7] * r);
+    return o;
+}
 __device__ __forceinline__ uint2 quant8(const float (&v)[8], const TileScale& t) {
+    if (t.exact) return quant8_exact(v, t.r_lo);
     uint2 lo, hi;
     const float r_lo = t.slow ? 0.0f : t.r_lo, r_hi = t.slow ? __builtin_inff() : t.r_hi;   // slow: every element differs
     lo.x = pack4_e4m3(v[0] * r_lo, v[1] * r_lo, v[2] * r_lo, v[3] * r_lo);

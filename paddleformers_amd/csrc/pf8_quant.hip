@@ -51,6 +51,7 @@ __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict_
     const float sc = scale_of(am_sel, pow2 != 0);       // lane q of a quad: scale of tile q
     float r_lo, r_hi;
     scale_recips(sc, r_lo, r_hi);
+    if (pow2) r_lo = pow2_recip(sc);                    // exact: one conversion per element, nothing to check
     if (l < 4) {
         const int kb = kb0 + 4 * l + g;
         if (kb < KB) {
@@ -60,7 +61,13 @@ __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict_
     }
     // cross-lane reads see only active lanes: every broadcast happens while the wavefront is whole
     uint2 o[4];
-    {
+    if (pow2) {
+        float v[8];
+        unpack8(w[0], v); o[0] = quant8_exact(v, quad_bcast<0>(r_lo));
+        unpack8(w[1], v); o[1] = quant8_exact(v, quad_bcast<1>(r_lo));
+        unpack8(w[2], v); o[2] = quant8_exact(v, quad_bcast<2>(r_lo));
+        unpack8(w[3], v); o[3] = quant8_exact(v, quad_bcast<3>(r_lo));
+    } else {
         float v[8];
         unpack8(w[0], v); o[0] = quant8_r(v, quad_bcast<0>(r_lo), quad_bcast<0>(r_hi), quad_bcast<0>(sc));
         unpack8(w[1], v); o[1] = quant8_r(v, quad_bcast<1>(r_lo), quad_bcast<1>(r_hi), quad_bcast<1>(sc));
@@ -422,7 +429,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float4 f = lds_sc[8 * g + i];
-            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f;
+            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f; t.exact = pow2 != 0;
             const int64_t r = row0 + 8 * g + i;
             float v[8];
             unpack8(w[i], v);
@@ -447,7 +454,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
         for (int h = 0; h < 2; ++h) {
             const int j = 2 * k + h;
             const float4 f = lds_sc[128 + 8 * l + j];
-            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f;
+            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f; t.exact = pow2 != 0;
             cs[j] = t.s;
             lds_put_col(lds_t, l, g, j, h == 0 ? quant8(lo, t) : quant8(hi, t));
         }
