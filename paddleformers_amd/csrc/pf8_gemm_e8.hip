@@ -173,12 +173,12 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     bool n_valid = false;
 
     // copy c of a wavefront fills rows (4 c + wave) * 8 + (lane >> 3) of the stacked [P; Q] block.  P rows
-    // are swizzled by e8_keyp(row), Q rows by (row >> 3) & 7: a Q fragment's 16 lanes read rows 8 apart
+    // are swizzled by e8_keyp(row), Q rows by e8_keyp(row >> 3): a Q fragment's 16 lanes read rows 8 apart
     const int crow = lane >> 3, cpos = lane & 7;
     const uint32_t c_off_p = (uint32_t)((wave * 8 + crow) * a.red + ((cpos ^ e8_keyp(wave * 8 + crow)) << 4));
-    uint32_t c_off_q[2];
+    uint32_t c_off_q[4];
 #pragma unroll
-    for (int par = 0; par < 2; ++par) c_off_q[par] = (uint32_t)((wave * 8 + crow) * a.red + ((cpos ^ (4 * par + wave)) << 4));
+    for (int v = 0; v < 4; ++v) c_off_q[v] = (uint32_t)((wave * 8 + crow) * a.red + ((cpos ^ e8_keyp(4 * v + wave)) << 4));
     const int64_t copy_step = 32 * a.red;
     const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
     int fp_ofs[2], fq_ofs[2];
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     for (int h = 0; h < 2; ++h) {
         const int prow = wp * 128 + li;
         fp_ofs[h] = prow * 128 + (((2 * kg + h) ^ e8_keyp(prow)) << 4);
-        fq_ofs[h] = Q_OFS + (wq * 128 + li * 8) * 128 + (((2 * kg + h) ^ (li & 7)) << 4);
+        fq_ofs[h] = Q_OFS + (wq * 128 + li * 8) * 128 + (((2 * kg + h) ^ e8_keyp(li)) << 4);
     }
     const uint32_t s_off = (uint32_t)(li * 8);
     uint32_t zero_off = 0;
@@ -195,8 +195,8 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
 #define E8_COPY(c_, pt_, qt_, qt2_, slot_)                                                             \
     do {                                                                                               \
         if ((c_) < 8) e8_dma16(c_off_p, (pt_) + (c_) * copy_step, lds_base + (slot_) * SLOT + ((c_) * 4 + wave) * 1024); \
-        else if ((c_) < 12) e8_dma16(c_off_q[(c_) & 1], (qt_) + ((c_) - 8) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
-        else e8_dma16(c_off_q[(c_) & 1], (qt2_) + ((c_) - 12) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
+        else if ((c_) < 12) e8_dma16(c_off_q[(c_) & 3], (qt_) + ((c_) - 8) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
+        else e8_dma16(c_off_q[(c_) & 3], (qt2_) + ((c_) - 12) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
     } while (0)
     // the scale bytes of a block, straight into the VGPRs the MFMAs take them from: eight Q exponents per
     // lane and the P block's exponent (every lane the same byte).  Vector loads on purpose: the value of
