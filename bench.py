@@ -453,7 +453,7 @@ def main():
         "frac_fp8_peak": round(value / FP8_PEAK_TFLOPS, 4),
         "kernel_ms": {k: round(v, 4) for k, v in kms.items()},
         "roofline": {
-            "kernel": "pf8::k_gemm_fwd_deep<1> (up+gate grouped GEMM)",
+            "kernel": "pf8::k_gemm_fwd_deep<1, 0> (up+gate grouped GEMM)",
             "bound": "mfma",
             "achieved": round(ach, 2),
             "peak": FP8_PEAK_TFLOPS,
