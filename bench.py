@@ -109,6 +109,9 @@ def bench_quantizers(iters=20, warmup=5):
     ms = time_kernel(lambda o: _lib.call("pf8_swiglu_weighted_quant", vp(o.data_ptr()), None, M, I, vp(q.data_ptr()), vp(s.data_ptr()), None, 0, 0, st),
                      [(o,) for o in os_], iters, warmup)
     out["swiglu_quant_8192x4096"] = {"bytes": 84443136 - 32768, "ms": ms}
+    ms = time_kernel(lambda o: _lib.call("pf8_swiglu_weighted_quant", vp(o.data_ptr()), None, M, I, vp(q.data_ptr()), vp(s.data_ptr()), None, 0, 1, st),
+                     [(o,) for o in os_], iters, warmup)
+    out["swiglu_quant_8192x4096_pow2"] = {"bytes": 84443136 - 32768, "ms": ms}
     del os_, q, s
     # C4: fused quant + transpose on [16384, 7168]
     M, K = 16384, 7168
@@ -320,7 +323,7 @@ def cpu_baseline(H, I, rows=12288):
     t0 = time.perf_counter()
     xq, xs = O.quant_1x128(x, 0)
     o1 = O.gemm_nt(xq, xs, w1q, w1s)
-    o2q, o2s = O.swiglu_weighted_quant(o1, None, 0, False)
+    o2q, o2s = O.swiglu_weighted_quant(o1, None, 0, True)
     O.gemm_nt(o2q, o2s, w2q, w2s)
     dt = time.perf_counter() - t0
     flops = 2.0 * rows * H * 2 * I + 2.0 * rows * I * H
@@ -397,7 +400,8 @@ def main():
         if evs: evs[1].record()
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((xq, xs.T), (w1q, w1s), o1, m_idx)
         if evs: evs[2].record()
-        o2q, o2s = F8.fused_weighted_swiglu_act_quant(o1, None, using_pow2_scaling=False)
+        # power-of-two scales for the requantised activation, as the reference's fused node asks (transformers/fp8_utils.py:984-986)
+        o2q, o2s = F8.fused_weighted_swiglu_act_quant(o1, None, using_pow2_scaling=True)
         if evs: evs[3].record()
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2q, w2s), o3, m_idx)
         if evs: evs[4].record()
@@ -448,7 +452,7 @@ def main():
             "workload": "BASELINE config 3: DeepSeek-V3-shaped MoE FP8 forward, one GPU's local share",
             "experts": E, "hidden": H, "moe_intermediate": I, "routed_rows": ROUTED, "padded_rows": Mpad,
             "zipf_s": 1.1, "empty_experts": int((counts == 0).sum()),
-            "pipeline": "quant_1x128(X) -> grouped GEMM up+gate -> fused SwiGLU+requant -> grouped GEMM down",
+            "pipeline": "quant_1x128(X) -> grouped GEMM up+gate -> fused SwiGLU+requant (pow2 scales, fp8_utils.py:984-986) -> grouped GEMM down",
         },
         "frac_fp8_peak": round(value / FP8_PEAK_TFLOPS, 4),
         "kernel_ms": {k: round(v, 4) for k, v in kms.items()},

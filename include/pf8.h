@@ -189,8 +189,8 @@ int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_lay
  * the form `use_ue8m0` selects for deep_gemm (transformers/configuration_utils.py:454-459; byte
  * format quantization/checkpoint_dequant.py:121-131).  Both operands must have been quantized with
  * pow2 scales (using_pow2_scale=True).  sa u8 [K/128, ldsa] (1x128 scales, K-block major, ldsa >= M
- * and a multiple of 8); sb u8 [N/128, K/128] ([E, N/128, K/128] grouped), read as whole aligned
- * dwords.  M (Mtot) multiple of 128, N multiple of 256, K multiple of 128 and >= 384, ldo multiple
+ * and a multiple of 8, base 8-byte aligned); sb u8 [N/128, K/128] ([E, N/128, K/128] grouped).
+ * M (Mtot) multiple of 128, N multiple of 256, K multiple of 128 and >= 384, ldo multiple
  * of 8; other shapes return PF8_EINVAL (decode the scales and use the fp32-scale entry points).
  * items: the list pf8_grouped_items_build made for this m_indices (two 128-row blocks of one expert
  * per 256-row work item); with it the call also weighs the expert load and hands a GEMM whose
