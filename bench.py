@@ -214,6 +214,11 @@ def bench_other_gemms(iters=10, warmup=3):
     g = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
     ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True), [()], 5, 2)
     out["grouped_wgrad_config5_dw1"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms}
+    # the operands above carry power-of-two scales (pow_2_scales=True): scales applied inside the MFMA
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True, scales_pow2=True), [()], 5, 2)
+    out["grouped_wgrad_config5_dw1_pow2"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms}
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=False, scales_pow2=True), [()], 5, 2)
+    out["grouped_wgrad_config5_dw1_pow2_overwrite"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms}
     del a_t, sa_t, b_t, sb_t, g
     torch.cuda.empty_cache()
     # per-step weight requantization of config 3's up+gate experts: both orientations from one read

@@ -234,6 +234,19 @@ int pf8_grouped_wgrad(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t,
                       const int64_t* rows_per_expert, int E, int64_t Kin, int64_t N, float* out,
                       int accumulate, pf8_stream_t stream);
 
+/* pf8_gemm_nt_1d1d_f32 / pf8_grouped_wgrad for operands whose scales are ALL powers of two -- what
+ * fused_transpose_split_quant(..., pow_2_scales=True) emits, which is how the weight-gradient
+ * operands of the MoE node are quantized (transformers/fp8_utils.py:1096-1100, 1117-1129,
+ * 1170-1182): both scales go into the block-scaled MFMA (their exponent fields are its UE8M0
+ * bytes) and the matrix pipe accumulates the K blocks itself.  Same arguments and layouts; a
+ * scale that is not a power of two is NOT detected (its mantissa is dropped). */
+int pf8_gemm_nt_1d1d_f32_pow2(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t,
+                              const float* sb_t, int64_t Kin, int64_t N, int64_t M, float* out,
+                              int accumulate, pf8_stream_t stream);
+int pf8_grouped_wgrad_pow2(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t,
+                           const float* sb_t, const int64_t* rows_per_expert, int E, int64_t Kin,
+                           int64_t N, float* out, int accumulate, pf8_stream_t stream);
+
 /* Measurement hook: a plain device-to-device copy of nbytes (multiple of 16).  bench.py launches it
  * so that hardware traffic counters (FETCH_SIZE / WRITE_SIZE) can be scaled by a kernel whose
  * traffic is known. */

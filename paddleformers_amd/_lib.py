@@ -37,6 +37,7 @@ SIGNATURES = {
     "pf8_swiglu_weighted_bwd": [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp],
     "pf8_gemm_nt": [_vp, _vp, _i32, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
     "pf8_gemm_nt_1d1d_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp],
+    "pf8_gemm_nt_1d1d_f32_pow2": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp],
     "pf8_grouped_gemm_nt_contiguous": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp],
     "pf8_gemm_nt_ue8m0": [_vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
     "pf8_grouped_gemm_nt_contiguous_ue8m0": [_vp, _vp, _i64, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp],
@@ -44,6 +45,7 @@ SIGNATURES = {
     "pf8_grouped_items_build": [_vp, _i64, _vp, _vp],
     "pf8_grouped_gemm_nt_masked": [_vp, _vp, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _i32, _vp, _vp],
     "pf8_grouped_wgrad": [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _i32, _vp],
+    "pf8_grouped_wgrad_pow2": [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _i32, _vp],
     "pf8_debug_copy": [_vp, _vp, _i64, _vp],
     "pf8_debug_encode": [_vp, _i64, _vp, _vp],
     "pf8_debug_div_encode": [_vp, _vp, _i64, _vp, _vp],

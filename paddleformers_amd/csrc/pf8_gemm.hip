@@ -46,6 +46,7 @@ struct GemmArgs {
     int64_t ldsq;               // UE8M0 forward: bytes between the K blocks of sq (0 = Qrows)
     const int32_t* pair_list;   // UE8M0 forward: when set, the kernel runs only if the paired-tile kernel declines
     int cus;                    //   (header of its work-item list, compute units both assume)
+    int pow2_scales;            // wgrad: every scale is a power of two (applied inside the MFMA)
 };
 
 #ifndef PF8_SWZ
@@ -600,6 +601,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
 // memory operations complete in order, so a scale load issued after the copies would make every
 // later wait on it wait for the copies as well.
 // ---------------------------------------------------------------------------------------------
+template <bool POW2>
 __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
     constexpr int NPS = 4, STAGE = 32768, Q_OFS = 16384;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -669,12 +671,22 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
         sp_ptr[t] = spb + c;
     }
 
+    // POW2: the block-scaled MFMA wants, from lane l, the scale of A row l % 16 (a P row) and of B
+    // column l % 16 (a Q row): one scalar per fragment and lane on both sides
+    const float* sp1_ptr[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        int64_t c = p0 + wp * 64 + t * 16 + li;
+        if (c > a.Prows - 1) c = a.Prows - 1;
+        sp1_ptr[t] = spb + c;
+    }
+
     f32x4 acc[NPS][4];
 #pragma unroll
     for (int i = 0; i < NPS; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float fq_nxt[4];
+    float fq_nxt[4], fp1_nxt[4];
     f32x4 fp_nxt[4];
 
 #define PF8_DMA(kb_, stage_)                                                                           \
@@ -685,7 +697,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
 #define PF8_LOAD_S(kb_)                                                                                \
     _Pragma("unroll") for (int t = 0; t < 4; ++t) {                                                    \
         fq_nxt[t] = sq_ptr[t][(kb_) * a.Qrows];                                                        \
-        fp_nxt[t] = *reinterpret_cast<const f32x4*>(sp_ptr[t] + (kb_) * a.Prows);                      \
+        if (POW2) fp1_nxt[t] = sp1_ptr[t][(kb_) * a.Prows];                                            \
+        else fp_nxt[t] = *reinterpret_cast<const f32x4*>(sp_ptr[t] + (kb_) * a.Prows);                 \
     }
 #define PF8_PFRAG(ps_) ld_frag_lds(base + fp_ofs[0] + (ps_) * 2048, base + fp_ofs[1] + (ps_) * 2048)
 #define PF8_QFRAG(qs_) ld_frag_lds(base + fq_ofs[0] + (qs_) * 2048, base + fq_ofs[1] + (qs_) * 2048)
@@ -701,8 +714,13 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
         __syncthreads();                 // everyone's copies landed; everyone is done with stage cur^1
         float fq_cur[4];
         f32x4 fp_cur[4];
+        int eq_cur[4], ep_cur[4];      // POW2: the scales' exponent fields = UE8M0 bytes
 #pragma unroll
-        for (int t = 0; t < 4; ++t) { fq_cur[t] = fq_nxt[t]; fp_cur[t] = fp_nxt[t]; }
+        for (int t = 0; t < 4; ++t) {
+            fq_cur[t] = fq_nxt[t];
+            if (POW2) { eq_cur[t] = (int)(f2u(fq_nxt[t]) >> 23); ep_cur[t] = (int)(f2u(fp1_nxt[t]) >> 23); }
+            else fp_cur[t] = fp_nxt[t];
+        }
         const int64_t kbn = kb + 1 < KB ? kb + 1 : kb;
         PF8_LOAD_S(kbn)
         __builtin_amdgcn_sched_barrier(0);
@@ -726,6 +744,16 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         pf[3] = PF8_PFRAG(3);
         __builtin_amdgcn_sched_barrier(0);
+        if (POW2) {
+            // both operands' power-of-two scales go into the MFMA, which accumulates the block itself
+#pragma unroll
+            for (int j = 0; j < NPS * 4; ++j) {
+                const int ps = j >> 2, qs = j & 3;
+                acc[ps][qs] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(pf[ps], qf[qs], acc[ps][qs], 0, 0, 0, ep_cur[ps], 0, eq_cur[qs]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < NPS * 4; ++j) {
             const int ps = j >> 2, qs = j & 3;
@@ -820,7 +848,8 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
     } else {
         const int64_t Tw = ((a.Prows + 127) / 128) * ((a.Qrows + 127) / 128);
         dim3 gw((unsigned)(((Tw + 7) / 8) * 8), grid.y);
-        hipLaunchKernelGGL(k_gemm_wgrad, gw, dim3(256), lds_bytes, st, a);
+        if (a.pow2_scales) hipLaunchKernelGGL(k_gemm_wgrad<true>, gw, dim3(256), lds_bytes, st, a);
+        else hipLaunchKernelGGL(k_gemm_wgrad<false>, gw, dim3(256), lds_bytes, st, a);
     }
     return pf8_check_launch(where);
 }
@@ -837,7 +866,8 @@ static int ensure_lds_attr() {
     static int done = 0;
     if (done) return PF8_OK;
     hipError_t e = hipSuccess;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_wgrad), hipFuncAttributeMaxDynamicSharedMemorySize, 69632);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_wgrad<false>), hipFuncAttributeMaxDynamicSharedMemorySize, 69632);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_wgrad<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 69632);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
@@ -930,50 +960,74 @@ extern "C" int pf8_grouped_gemm_nt_masked(const uint8_t* a, const float* sa, con
     return launch_gemm(g, MODE_FWD, dim3((unsigned)tiles, (unsigned)E), (hipStream_t)stream, __func__);
 }
 
-extern "C" int pf8_gemm_nt_1d1d_f32(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t, int64_t Kin,
-                                    int64_t N, int64_t M, float* out, int accumulate, pf8_stream_t stream) {
-    PF8_REQUIRE(Kin >= 0 && N >= 0 && M >= 0, "negative shape");
-    PF8_REQUIRE(M % 128 == 0, "M (the reduction axis) must be a multiple of 128");
-    PF8_REQUIRE(N % 4 == 0, "N must be a multiple of 4");
+#define PF8_REQUIRE_AT(where, cond, msg) do { if (!(cond)) return pf8_fail(PF8_EINVAL, where, msg); } while (0)
+
+static int gemm_nt_1d1d_f32(const char* where, const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t,
+                            int64_t Kin, int64_t N, int64_t M, float* out, int accumulate, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE_AT(where, Kin >= 0 && N >= 0 && M >= 0, "negative shape");
+    PF8_REQUIRE_AT(where, M % 128 == 0, "M (the reduction axis) must be a multiple of 128");
+    PF8_REQUIRE_AT(where, N % 4 == 0, "N must be a multiple of 4");
     if (Kin == 0 || N == 0) return PF8_OK;
-    PF8_REQUIRE(out, "null pointer");
-    PF8_REQUIRE(M == 0 || (a_t && sa_t && b_t && sb_t), "null pointer");
-    PF8_REQUIRE(PF8_ALIGNED16(a_t) && PF8_ALIGNED16(b_t) && PF8_ALIGNED16(out) && PF8_ALIGNED16(sb_t), "pointers must be 16-byte aligned");
+    PF8_REQUIRE_AT(where, out, "null pointer");
+    PF8_REQUIRE_AT(where, M == 0 || (a_t && sa_t && b_t && sb_t), "null pointer");
+    PF8_REQUIRE_AT(where, PF8_ALIGNED16(a_t) && PF8_ALIGNED16(b_t) && PF8_ALIGNED16(out) && PF8_ALIGNED16(sb_t), "pointers must be 16-byte aligned");
     if (M == 0 && accumulate) return PF8_OK;
     int rc = ensure_lds_attr();
     if (rc) return rc;
     GemmArgs g = {};
     g.p = b_t; g.q = a_t; g.sp = sb_t; g.sq = sa_t; g.out = out;
-    g.Prows = N; g.Qrows = Kin; g.red = M; g.ldo = N; g.accumulate = accumulate; g.group = GROUP_NONE;
+    g.Prows = N; g.Qrows = Kin; g.red = M; g.ldo = N; g.accumulate = accumulate; g.group = GROUP_NONE; g.pow2_scales = pow2;
     const int64_t tiles = ((N + 127) / 128) * ((Kin + 127) / 128);
-    PF8_REQUIRE(tiles <= 0x7FFFFFFF, "too many tiles");
-    return launch_gemm(g, MODE_WGRAD, dim3((unsigned)tiles), (hipStream_t)stream, __func__);
+    PF8_REQUIRE_AT(where, tiles <= 0x7FFFFFFF, "too many tiles");
+    return launch_gemm(g, MODE_WGRAD, dim3((unsigned)tiles), (hipStream_t)stream, where);
+}
+
+extern "C" int pf8_gemm_nt_1d1d_f32(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t, int64_t Kin,
+                                    int64_t N, int64_t M, float* out, int accumulate, pf8_stream_t stream) {
+    return gemm_nt_1d1d_f32(__func__, a_t, sa_t, b_t, sb_t, Kin, N, M, out, accumulate, 0, stream);
+}
+
+extern "C" int pf8_gemm_nt_1d1d_f32_pow2(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t, int64_t Kin,
+                                         int64_t N, int64_t M, float* out, int accumulate, pf8_stream_t stream) {
+    return gemm_nt_1d1d_f32(__func__, a_t, sa_t, b_t, sb_t, Kin, N, M, out, accumulate, 1, stream);
+}
+
+static int grouped_wgrad(const char* where, const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t,
+                         const int64_t* rows_per_expert, int E, int64_t Kin, int64_t N, float* out, int accumulate, int pow2,
+                         pf8_stream_t stream) {
+    PF8_REQUIRE_AT(where, E >= 0 && Kin >= 0 && N >= 0, "negative shape");
+    PF8_REQUIRE_AT(where, E <= 256, "at most 256 experts per call");
+    PF8_REQUIRE_AT(where, N % 4 == 0, "N must be a multiple of 4");
+    if (E == 0 || Kin == 0 || N == 0) return PF8_OK;
+    PF8_REQUIRE_AT(where, rows_per_expert && out, "null pointer");
+    GemmArgs g = {};
+    int64_t total = 0;
+    for (int e = 0; e < E; ++e) {
+        PF8_REQUIRE_AT(where, rows_per_expert[e] >= 0 && rows_per_expert[e] % 128 == 0, "rows_per_expert entries must be non-negative multiples of 128");
+        g.tile_start[e] = (int32_t)(total / 128);
+        total += rows_per_expert[e];
+    }
+    g.tile_start[E] = (int32_t)(total / 128);
+    PF8_REQUIRE_AT(where, total == 0 || (a_t && sa_t && b_t && sb_t), "null pointer");
+    PF8_REQUIRE_AT(where, PF8_ALIGNED16(a_t) && PF8_ALIGNED16(b_t) && PF8_ALIGNED16(out) && PF8_ALIGNED16(sb_t), "pointers must be 16-byte aligned");
+    if (total == 0 && accumulate) return PF8_OK;
+    int rc = ensure_lds_attr();
+    if (rc) return rc;
+    g.p = b_t; g.q = a_t; g.sp = sb_t; g.sq = sa_t; g.out = out;
+    g.Prows = N; g.Qrows = Kin; g.red = 0; g.ldo = N; g.accumulate = accumulate; g.group = GROUP_WGRAD; g.E = E; g.pow2_scales = pow2;
+    const int64_t tiles = ((N + 127) / 128) * ((Kin + 127) / 128);
+    PF8_REQUIRE_AT(where, tiles <= 0x7FFFFFFF, "too many tiles");
+    return launch_gemm(g, MODE_WGRAD, dim3((unsigned)tiles, (unsigned)E), (hipStream_t)stream, where);
 }
 
 extern "C" int pf8_grouped_wgrad(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t,
                                  const int64_t* rows_per_expert, int E, int64_t Kin, int64_t N, float* out, int accumulate,
                                  pf8_stream_t stream) {
-    PF8_REQUIRE(E >= 0 && Kin >= 0 && N >= 0, "negative shape");
-    PF8_REQUIRE(E <= 256, "at most 256 experts per call");
-    PF8_REQUIRE(N % 4 == 0, "N must be a multiple of 4");
-    if (E == 0 || Kin == 0 || N == 0) return PF8_OK;
-    PF8_REQUIRE(rows_per_expert && out, "null pointer");
-    GemmArgs g = {};
-    int64_t total = 0;
-    for (int e = 0; e < E; ++e) {
-        PF8_REQUIRE(rows_per_expert[e] >= 0 && rows_per_expert[e] % 128 == 0, "rows_per_expert entries must be non-negative multiples of 128");
-        g.tile_start[e] = (int32_t)(total / 128);
-        total += rows_per_expert[e];
-    }
-    g.tile_start[E] = (int32_t)(total / 128);
-    PF8_REQUIRE(total == 0 || (a_t && sa_t && b_t && sb_t), "null pointer");
-    PF8_REQUIRE(PF8_ALIGNED16(a_t) && PF8_ALIGNED16(b_t) && PF8_ALIGNED16(out) && PF8_ALIGNED16(sb_t), "pointers must be 16-byte aligned");
-    if (total == 0 && accumulate) return PF8_OK;
-    int rc = ensure_lds_attr();
-    if (rc) return rc;
-    g.p = b_t; g.q = a_t; g.sp = sb_t; g.sq = sa_t; g.out = out;
-    g.Prows = N; g.Qrows = Kin; g.red = 0; g.ldo = N; g.accumulate = accumulate; g.group = GROUP_WGRAD; g.E = E;
-    const int64_t tiles = ((N + 127) / 128) * ((Kin + 127) / 128);
-    PF8_REQUIRE(tiles <= 0x7FFFFFFF, "too many tiles");
-    return launch_gemm(g, MODE_WGRAD, dim3((unsigned)tiles, (unsigned)E), (hipStream_t)stream, __func__);
+    return grouped_wgrad(__func__, a_t, sa_t, b_t, sb_t, rows_per_expert, E, Kin, N, out, accumulate, 0, stream);
+}
+
+extern "C" int pf8_grouped_wgrad_pow2(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t, const float* sb_t,
+                                      const int64_t* rows_per_expert, int E, int64_t Kin, int64_t N, float* out, int accumulate,
+                                      pf8_stream_t stream) {
+    return grouped_wgrad(__func__, a_t, sa_t, b_t, sb_t, rows_per_expert, E, Kin, N, out, accumulate, 1, stream);
 }

@@ -236,9 +236,10 @@ class FP8LinearFunctionBase:
         return F8.fp8_quant_blockwise(tensor, output_scale_transpose=True, quant_method="1x128", input_transpose=True)
 
     @staticmethod
-    def kitchen_gemm(x_fp8, x_scale, w_fp8, w_scale, is_a_1d_scaled, is_b_1d_scaled, out=None, rtn_dtype=torch.bfloat16):
+    def kitchen_gemm(x_fp8, x_scale, w_fp8, w_scale, is_a_1d_scaled, is_b_1d_scaled, out=None, rtn_dtype=torch.bfloat16,
+                     scales_pow2=False):
         """fp8_utils.py:176-221: weight-gradient GEMM, accumulate when `out` is given; zero-sized
-        operands give zeros."""
+        operands give zeros.  scales_pow2: see functional.fp8_gemm_blockwise."""
         if out is not None:
             accumulate, out_dtype = True, out.dtype
         else:
@@ -247,11 +248,11 @@ class FP8LinearFunctionBase:
             if out is None and out_dtype != torch.float32:
                 y = F8.fp8_gemm_blockwise(a=x_fp8, a_decode_scale=x_scale, b=w_fp8, b_decode_scale=w_scale, out_dtype=torch.float32,
                                           out=None, accumulate=False, use_split_accumulator=True,
-                                          is_a_1d_scaled=is_a_1d_scaled, is_b_1d_scaled=is_b_1d_scaled)
+                                          is_a_1d_scaled=is_a_1d_scaled, is_b_1d_scaled=is_b_1d_scaled, scales_pow2=scales_pow2)
                 return y.to(out_dtype)
             return F8.fp8_gemm_blockwise(a=x_fp8, a_decode_scale=x_scale, b=w_fp8, b_decode_scale=w_scale, out_dtype=out_dtype,
                                          out=out, accumulate=accumulate, use_split_accumulator=True,
-                                         is_a_1d_scaled=is_a_1d_scaled, is_b_1d_scaled=is_b_1d_scaled)
+                                         is_a_1d_scaled=is_a_1d_scaled, is_b_1d_scaled=is_b_1d_scaled, scales_pow2=scales_pow2)
         y = torch.zeros([x_fp8.shape[0], w_fp8.shape[0]], dtype=out_dtype, device=x_fp8.device)
         if out is not None:
             return out + y
@@ -291,7 +292,7 @@ class FP8LinearFunctionBase:
 
     @staticmethod
     def compute_expert_w_grad(input_t, input_t_scale, dout_t, dout_t_scale, is_a_1d_scaled=True, is_b_1d_scaled=True, weight=None,
-                              rtn_dtype=torch.bfloat16):
+                              rtn_dtype=torch.bfloat16, scales_pow2=False):
         """fp8_utils.py:293-350: accumulate one expert's weight gradient into weight.main_grad
         (or weight.grad), optionally deferred through WeightGradStore."""
         if input_t is None or numpy.prod(input_t.shape) == 0:
@@ -301,16 +302,16 @@ class FP8LinearFunctionBase:
                 weight.main_grad = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device)
             if WeightGradStore.enabled:
                 WeightGradStore.put(partial(FP8LinearFunctionBase.kitchen_gemm, input_t, input_t_scale, dout_t, dout_t_scale,
-                                            is_a_1d_scaled, is_b_1d_scaled, weight.main_grad, rtn_dtype))
+                                            is_a_1d_scaled, is_b_1d_scaled, weight.main_grad, rtn_dtype, scales_pow2))
                 result = None
             else:
                 result = FP8LinearFunctionBase.kitchen_gemm(input_t, input_t_scale, dout_t, dout_t_scale, is_a_1d_scaled,
-                                                            is_b_1d_scaled, weight.main_grad, rtn_dtype)
+                                                            is_b_1d_scaled, weight.main_grad, rtn_dtype, scales_pow2)
         else:
             if getattr(weight, "grad", None) is None:
                 weight.grad = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device)
             result = FP8LinearFunctionBase.kitchen_gemm(input_t, input_t_scale, dout_t, dout_t_scale, is_a_1d_scaled, is_b_1d_scaled,
-                                                        weight.grad, rtn_dtype)
+                                                        weight.grad, rtn_dtype, scales_pow2)
         if hasattr(weight, "_apply_backward_hook"):
             weight._apply_backward_hook()
         return result
@@ -726,22 +727,27 @@ class FP8GroupGemmMlpFunctionNode:
         return torch.as_strided(g0, (len(grads), K, N), (K * N, N, 1))
 
     @staticmethod
-    def _expert_wgrads(a_t, sa_t, b_t, sb_t, expert_w):
+    def _expert_wgrads(a_t, sa_t, b_t, sb_t, expert_w, scales_pow2=False):
         """The per-expert loop of fp8_utils.py:1117-1129 / :1170-1182.  When the experts' main_grad
-        tensors are slices of one [E, K, N] buffer, all experts run in one grouped launch."""
+        tensors are slices of one [E, K, N] buffer, all experts run in one grouped launch.
+        scales_pow2: both operands were quantized by this node (pow_2_scales=True)."""
         with torch.no_grad():
             stacked = FP8GroupGemmMlpFunctionNode._stacked_main_grad(expert_w) if len(expert_w) > 1 else None
             if stacked is not None:
-                F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, stacked, accumulate=True)
+                F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, stacked, accumulate=True, scales_pow2=scales_pow2)
                 for w in expert_w:
                     if hasattr(w, "_apply_backward_hook"):
                         w._apply_backward_hook()
                 return
             for i in range(len(expert_w)):
-                FP8LinearFunctionBase.compute_expert_w_grad(a_t[i], sa_t[i], b_t[i], sb_t[i], True, True, expert_w[i], torch.float32)
+                FP8LinearFunctionBase.compute_expert_w_grad(a_t[i], sa_t[i], b_t[i], sb_t[i], True, True, expert_w[i], torch.float32,
+                                                            scales_pow2=scales_pow2)
 
-    def bwd_down_weight(self, do3, o2, expert_w2, tokens_per_expert):
-        """dw2[e] [I, H] += o2_e^T . do3_e (fp8_utils.py:1102-1134)."""
+    def bwd_down_weight(self, do3, o2, expert_w2, tokens_per_expert, scales_pow2=None):
+        """dw2[e] [I, H] += o2_e^T . do3_e (fp8_utils.py:1102-1134).  Operands handed in as
+        (fp8_t, scale_t) pairs are taken to carry arbitrary scales unless scales_pow2 says otherwise."""
+        if scales_pow2 is None:
+            scales_pow2 = not isinstance(o2, tuple) and not isinstance(do3, tuple)
         if isinstance(o2, tuple):
             o2_t_fp8, o2_t_scale = o2
         else:
@@ -750,7 +756,7 @@ class FP8GroupGemmMlpFunctionNode:
             do3_t_fp8, do3_t_scale = do3
         else:
             do3_t_fp8, do3_t_scale = self.fused_transpose_split_quant(do3, None, tokens_per_expert, True)
-        fn = partial(self._expert_wgrads, o2_t_fp8, o2_t_scale, do3_t_fp8, do3_t_scale, expert_w2)
+        fn = partial(self._expert_wgrads, o2_t_fp8, o2_t_scale, do3_t_fp8, do3_t_scale, expert_w2, scales_pow2)
         if WeightGradStore.enabled:
             WeightGradStore.put(fn)
         else:
@@ -769,7 +775,7 @@ class FP8GroupGemmMlpFunctionNode:
             self.input_scale = None
             self.input = None
         do1_t_fp8, do1_t_scale = self.fused_transpose_split_quant(do1, None, tokens_per_expert, True)
-        fn = partial(self._expert_wgrads, input_x_t_fp8, input_x_t_scale, do1_t_fp8, do1_t_scale, expert_w1)
+        fn = partial(self._expert_wgrads, input_x_t_fp8, input_x_t_scale, do1_t_fp8, do1_t_scale, expert_w1, True)
         if WeightGradStore.enabled:
             WeightGradStore.put(fn)
         else:
@@ -835,7 +841,7 @@ class FP8GroupGemmMlpFunctionNode:
         del do1
         if isinstance(out_grad, tuple):
             do3_fp8, do3_scale = self.fused_transpose_split_quant(out_grad[0], out_grad[1], tokens_per_expert, True)
-            self.bwd_down_weight((do3_fp8, do3_scale), o2_s, expert_w2, tokens_per_expert)
+            self.bwd_down_weight((do3_fp8, do3_scale), o2_s, expert_w2, tokens_per_expert, scales_pow2=True)
         else:
             self.bwd_down_weight(out_grad, o2_s, expert_w2, tokens_per_expert)
         if reset_status:

@@ -388,11 +388,14 @@ def fused_swiglu_weighted_bwd(o1: torch.Tensor, do2_s: torch.Tensor, probs: torc
 
 
 def fp8_gemm_blockwise(a, a_decode_scale, b, b_decode_scale, out_dtype=torch.float32, out=None, accumulate=False,
-                       use_split_accumulator=True, is_a_1d_scaled=True, is_b_1d_scaled=True):
+                       use_split_accumulator=True, is_a_1d_scaled=True, is_b_1d_scaled=True, scales_pow2=False):
     """y[Ka, Nb] (+)= a[Ka, M] . b[Nb, M]^T with both operands 1x128-scaled along M.
 
     transformers/fp8_utils.py:203-214 (kitchen_gemm): a_decode_scale [M/128, Ka], b_decode_scale
-    [M/128, Nb]; fp32 output; accumulate adds into `out`.
+    [M/128, Nb]; fp32 output; accumulate adds into `out`.  scales_pow2 (not in the reference's
+    signature): the caller vouches that every scale is a power of two, as
+    fused_transpose_split_quant(..., pow_2_scales=True) makes them; the scales then go into the
+    block-scaled MFMA.  Other scales would lose their mantissa unnoticed.
     """
     if not (is_a_1d_scaled and is_b_1d_scaled):
         raise ValueError("only the 1x128-by-1x128 scaled form is implemented (is_a_1d_scaled = is_b_1d_scaled = True)")
@@ -418,15 +421,17 @@ def fp8_gemm_blockwise(a, a_decode_scale, b, b_decode_scale, out_dtype=torch.flo
     else:
         if out.dtype != torch.float32 or tuple(out.shape) != (Ka, Nb) or not out.is_contiguous():
             raise ValueError("out must be a contiguous float32 [Ka, Nb] tensor")
-    _lib.call("pf8_gemm_nt_1d1d_f32", _p(a), _p(sa), _p(b), _p(sb), Ka, Nb, M, _p(out), int(bool(accumulate)), _stream())
+    _lib.call("pf8_gemm_nt_1d1d_f32_pow2" if scales_pow2 else "pf8_gemm_nt_1d1d_f32", _p(a), _p(sa), _p(b), _p(sb), Ka, Nb, M, _p(out),
+              int(bool(accumulate)), _stream())
     return out
 
 
-def grouped_wgrad(a_t_list, sa_t_list, b_t_list, sb_t_list, out: torch.Tensor, accumulate: bool = True):
+def grouped_wgrad(a_t_list, sa_t_list, b_t_list, sb_t_list, out: torch.Tensor, accumulate: bool = True, scales_pow2: bool = False):
     """All experts' weight gradients in one launch: out[e] (+)= a_t[e] . b_t[e]^T.
 
     Replaces the per-expert Python loops of transformers/fp8_utils.py:1117-1129 and :1170-1182.
-    The lists must be the outputs of fused_transpose_split_quant (views of one packed buffer).
+    The lists must be the outputs of fused_transpose_split_quant (views of one packed buffer);
+    scales_pow2 says they were made with pow_2_scales=True (see fp8_gemm_blockwise).
     """
     E = len(a_t_list)
     rows = [int(t.shape[1]) for t in a_t_list]
@@ -448,8 +453,8 @@ def grouped_wgrad(a_t_list, sa_t_list, b_t_list, sb_t_list, out: torch.Tensor, a
         return C.c_void_p(p)
 
     arr = (C.c_int64 * E)(*rows)
-    _lib.call("pf8_grouped_wgrad", base(a_t_list), base(sa_t_list), base(b_t_list), base(sb_t_list), arr, E, Kin, N, _p(out),
-              int(bool(accumulate)), _stream())
+    _lib.call("pf8_grouped_wgrad_pow2" if scales_pow2 else "pf8_grouped_wgrad", base(a_t_list), base(sa_t_list), base(b_t_list),
+              base(sb_t_list), arr, E, Kin, N, _p(out), int(bool(accumulate)), _stream())
     return out
 
 

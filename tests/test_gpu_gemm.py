@@ -44,6 +44,8 @@ def _bf(bits):
 
 BLOCK_FRO = 6e-4      # bf16 outputs vs the block-accumulating oracle (bf16 rounding flips included)
 F32_FRO = 5e-5        # fp32 outputs vs the oracle
+F32_FRO_MFMA_ACC = 1e-4   # the same when the running sum stays inside the matrix pipe (scales applied by the MFMA):
+                          # its adder keeps fewer bits than an fp32 FMA chain; measured up to 5.04e-5
 ELEM_ABS = 4e-5       # per-element slack as a fraction of sum|a||b|
 
 
@@ -271,6 +273,46 @@ def test_wgrad_1d1d(dg, Kin, N, M):
     assert torch.equal(buf, buf2)
 
 
+@pytest.mark.parametrize("Kin,N,M", [(128, 128, 128), (256, 384, 512), (200, 132, 256)])
+def test_wgrad_1d1d_pow2_scales_inside_the_mfma(dg, Kin, N, M):
+    """Operands quantized with power-of-two scales through the entry point that hands the scales to the
+    block-scaled MFMA: same oracle and bound as the fp32-scale form, and the two forms agree."""
+    from paddleformers_amd import functional as F8
+
+    x = G.bf16_normal((M, Kin), seed=Kin + N + M, outlier_frac=1e-3, outlier_scale=40.0)
+    d = G.bf16_normal((M, N), seed=Kin + N + M + 1, std=1e-3)
+    a_t, sa_t = O.quant_1x128(np.ascontiguousarray(x.T), 1, pow2=True)
+    b_t, sb_t = O.quant_1x128(np.ascontiguousarray(d.T), 1, pow2=True)
+    ta, tb = G.to_torch_fp8(a_t), G.to_torch_fp8(b_t)
+    tsa, tsb = torch.from_numpy(sa_t).cuda(), torch.from_numpy(sb_t).cuda()
+    y = F8.fp8_gemm_blockwise(a=ta, a_decode_scale=tsa, b=tb, b_decode_scale=tsb, scales_pow2=True)
+    exp = O.gemm_nt_1d1d_f32(a_t, sa_t, b_t, sb_t)
+    err = G.rel_fro(y.cpu().numpy(), exp)
+    assert err <= F32_FRO_MFMA_ACC, err
+    y0 = F8.fp8_gemm_blockwise(a=ta, a_decode_scale=tsa, b=tb, b_decode_scale=tsb)
+    assert G.rel_fro(y.cpu().numpy(), y0.cpu().numpy()) <= F32_FRO_MFMA_ACC
+    base = np.random.default_rng(1).standard_normal((Kin, N)).astype(np.float32)
+    buf = torch.from_numpy(base.copy()).cuda()
+    F8.fp8_gemm_blockwise(a=ta, a_decode_scale=tsa, b=tb, b_decode_scale=tsb, out=buf, accumulate=True, scales_pow2=True)
+    assert G.rel_fro(buf.cpu().numpy(), O.gemm_nt_1d1d_f32(a_t, sa_t, b_t, sb_t, out=base)) <= F32_FRO_MFMA_ACC
+
+
+def test_wgrad_pow2_scales_are_applied_per_row_and_block(dg):
+    """Ones times ones with a different power of two for every (row, K block) on both sides:
+    out[i, j] = sum_kb 128 * sa[kb, i] * sb[kb, j] exactly -- catches swapped or mis-indexed scale lanes."""
+    from paddleformers_amd import functional as F8
+
+    Kin, N, M = 256, 128, 384
+    rng = np.random.default_rng(8)
+    one = O.e4m3_encode_array(np.ones(1, np.float32))[0]
+    a_t, b_t = np.full((Kin, M), one, np.uint8), np.full((N, M), one, np.uint8)
+    sa_t = np.exp2(rng.integers(-4, 4, (M // 128, Kin))).astype(np.float32)
+    sb_t = np.exp2(rng.integers(-3, 3, (M // 128, N))).astype(np.float32)
+    y = F8.fp8_gemm_blockwise(a=G.to_torch_fp8(a_t), a_decode_scale=torch.from_numpy(sa_t).cuda(), b=G.to_torch_fp8(b_t),
+                              b_decode_scale=torch.from_numpy(sb_t).cuda(), scales_pow2=True)
+    assert np.array_equal(y.cpu().numpy(), (128.0 * (sa_t.T.astype(np.float64) @ sb_t.astype(np.float64))).astype(np.float32))
+
+
 def test_grouped_wgrad_equals_per_expert_loop(dg):
     from paddleformers_amd import functional as F8
 
@@ -295,3 +337,15 @@ def test_grouped_wgrad_equals_per_expert_loop(dg):
     F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, out0, accumulate=False)
     assert torch.equal(out0[1], torch.zeros_like(out0[1]))
     assert torch.allclose(out0[0], out[0] - base[0], rtol=1e-4, atol=1e-6)
+    # the operands carry power-of-two scales (pow_2_scales=True above): scales inside the MFMA give the
+    # same gradients, grouped launch and per-expert launches bit for bit
+    outp = base.clone()
+    F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, outp, accumulate=True, scales_pow2=True)
+    for e, r in enumerate(rows):
+        if r == 0:
+            assert torch.equal(outp[e], base[e])
+            continue
+        ref = base[e].clone()
+        F8.fp8_gemm_blockwise(a=a_t[e], a_decode_scale=sa_t[e], b=b_t[e], b_decode_scale=sb_t[e], out=ref, accumulate=True, scales_pow2=True)
+        assert torch.equal(outp[e], ref), f"expert {e}"
+        assert G.rel_fro((outp[e] - base[e]).cpu().numpy(), (out[e] - base[e]).cpu().numpy()) <= 1e-4
