@@ -211,6 +211,44 @@ def test_grouped_contiguous_ue8m0_vs_oracle(dg, request, rows, paired, cus):
         start += r
 
 
+def _pair_blocks(block_experts):
+    """Serial statement of the pairing: consecutive 128-row blocks of one expert two by two, an odd one
+    out alone, padding blocks (expert < 0) skipped."""
+    items, prev, par = [], -2, 1
+    for b, e in enumerate(block_experts):
+        if e < 0:
+            par, prev = 1, e
+            continue
+        par = 0 if e != prev else par ^ 1
+        if par == 0:
+            items.append([b, -1, int(e)])
+        else:
+            items[-1][1] = b
+        prev = e
+    return items
+
+
+# 40 blocks: one block per thread of the list builder; 3000: several blocks per thread; 9000: more blocks
+# than the builder keeps in LDS
+@pytest.mark.parametrize("nb", [40, 3000, 9000])
+def test_build_group_items_pairs_each_experts_blocks(dg, nb):
+    rng = np.random.default_rng(nb)
+    blocks = []
+    e = 0
+    while len(blocks) < nb:
+        blocks += [e] * int(rng.integers(0, 7))
+        if rng.random() < 0.25:
+            blocks += [-1] * int(rng.integers(1, 3))
+        e += 1
+    blocks = np.array(blocks[:nb], np.int32)
+    m_idx = torch.from_numpy(np.repeat(blocks, 128)).cuda()
+    items = dg.build_group_items(m_idx).cpu().numpy()
+    exp = _pair_blocks(blocks)
+    assert items[0] == len(exp) and items[1] == nb
+    got = items[4:4 + 4 * len(exp)].reshape(-1, 4)[:, :3]
+    assert np.array_equal(got, np.array(exp, np.int32).reshape(-1, 3))
+
+
 @pytest.mark.parametrize("cus", ["all", "few"])
 def test_grouped_contiguous_ue8m0_many_small_experts(dg, request, cus):
     """40 experts of 0..5 blocks in Zipf-like disorder, some followed by padding blocks (index -1): every
