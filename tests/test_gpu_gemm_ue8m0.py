@@ -323,3 +323,40 @@ def test_ue8m0_gemms_at_config3_size_agree_with_the_fp32_scale_kernels(dg):
     sl = slice(3 * rows, 4 * rows)
     dg.fp8_gemm_nt((xq[sl], F.scales_to_ue8m0(xs_l[sl].contiguous())), (wq[3], F.scales_to_ue8m0(ws[3])), one)
     assert torch.equal(one.view(torch.int16), out[sl].view(torch.int16))
+
+
+def test_ue8m0_grouped_gemm_at_config5_size_agrees_with_the_fp32_scale_kernel(dg):
+    """128 experts with a Zipf(1.0) load over 131072 routed rows (segments of 2..190 blocks, 1083 blocks in
+    all): here the cost estimate picks the paired 256-row tiles on the whole device, and the list builder
+    walks two blocks per thread."""
+    from bench import zipf_counts
+    from paddleformers_amd import functional as F
+
+    E, H, N = 128, 4096, 2816
+    _, padded = zipf_counts(131072, E, 1.0, seed=5, n_empty=0)
+    rows = [int(r) for r in padded]
+    Mtot = sum(rows)
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn((Mtot, H), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    xq, xs = F.fp8_quant_blockwise(x, output_scale_transpose=True, quant_method="1x128", input_transpose=False, using_pow2_scale=True)
+    del x
+    wq = torch.empty((E, N, H), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, N // 128, H // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        w = (torch.randn((N, H), generator=gen, device="cuda", dtype=torch.float32) * 0.02).to(torch.bfloat16)
+        q, s_ = F.fused_stack_transpose_quant([w], transpose=False, using_pow2_scale=True)
+        wq[e], ws[e] = q.view(N, H), s_.view(N // 128, H // 128)
+    m_idx = torch.repeat_interleave(torch.arange(E, dtype=torch.int32), torch.tensor(rows)).cuda()
+    xs_l = xs.t() if tuple(xs.shape) == (H // 128, Mtot) else xs
+    ref = torch.empty((Mtot, N), dtype=torch.bfloat16, device="cuda")
+    dg.m_grouped_fp8_gemm_nt_contiguous((xq, xs_l), (wq, ws), ref, m_idx)
+    out = torch.full_like(ref, float("nan"))
+    dg.m_grouped_fp8_gemm_nt_contiguous((xq, F.scales_to_ue8m0(xs_l)), (wq, F.scales_to_ue8m0(ws)), out, m_idx)
+    items = dg.build_group_items(m_idx).cpu().numpy()
+    assert items[1] == Mtot // 128 and items[0] == sum((r // 128 + 1) // 2 for r in rows)
+    num = den = 0.0
+    for lo in range(0, Mtot, 16384):      # in slices: the fp32 copies of two 780 MB outputs are not needed at once
+        a, b = out[lo:lo + 16384].float(), ref[lo:lo + 16384].float()
+        num += float((a - b).pow(2).sum())
+        den += float(b.pow(2).sum())
+    assert (num / den) ** 0.5 <= 3e-4
