@@ -255,6 +255,18 @@ def bench_other_gemms(iters=10, warmup=3):
     out["moe_unpermute_config5"] = {"bytes": Tt * tk * Ht * 2 + Tt * Ht * 2, "ms": ms}
     del xt, ux, rowmap, up
     torch.cuda.empty_cache()
+    # the RMSNorm the dense FP8 MLP recomputes: forward and backward on [16384, 7168] bf16
+    Mn, Hn = 16384, 7168
+    xn = torch.randn((Mn, Hn), device="cuda").to(torch.bfloat16)
+    wn = torch.randn((Hn,), device="cuda").to(torch.bfloat16)
+    dn = torch.randn((Mn, Hn), device="cuda").to(torch.bfloat16)
+    ms = time_kernel(lambda: F8.fused_rms_norm_ext(xn, wn, 1e-6), [()], 5, 2)
+    out["rms_norm_fwd_16384x7168"] = {"bytes": Mn * Hn * 4 + Mn * 4, "ms": ms}
+    _, ivn = F8.fused_rms_norm_ext(xn, wn, 1e-6)
+    ms = time_kernel(lambda: F8.fused_rms_norm_ext_grad(xn, wn, ivn, dn, 1e-6), [()], 5, 2)
+    out["rms_norm_bwd_16384x7168"] = {"bytes": Mn * Hn * 6 + Mn * 4 + Hn * 4, "ms": ms}
+    del xn, dn, ivn
+    torch.cuda.empty_cache()
     # the fused FP8 MoE node end to end at config 5: forward + backward (dgrad and wgrad, both GEMMs),
     # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers
     from paddleformers_amd import fp8_utils as U8

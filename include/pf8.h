@@ -149,11 +149,15 @@ int pf8_moe_unpermute(const uint16_t* unzipped, const int32_t* rowmap, const int
  * paddle._C_ops.fused_rms_norm_ext_grad(x, norm_w, invvar, dy, eps) -> (dx, dw), the norm that
  * FusedNormFP8MLPFunction recomputes (transformers/fp8_utils.py:470-475, 520-541, 687-741).
  * x, dy, y, dx bf16 [M,H], w bf16 [H], invar fp32 [M] = 1/sqrt(mean(x^2)+eps); y = bf16(x*invar*w).
- * dw fp32 [H] is ADDED to (the caller zeroes it), with atomics: its rounding depends on the order. */
+ * dw fp32 [H] is ADDED to (the caller zeroes it).  ws: DEVICE scratch of ws_rows x H floats, 16-byte
+ * aligned (1024 rows use the whole device); each workgroup leaves its share of dw in a row of it
+ * and a second kernel adds the rows up in order.  ws == NULL: the shares go to dw by atomics
+ * (several times slower at training sizes, and the rounding then depends on the order). */
 int pf8_rms_norm_fwd(const uint16_t* x, const uint16_t* w, float eps, int64_t M, int64_t H,
                      uint16_t* y, float* invar, pf8_stream_t stream);
 int pf8_rms_norm_bwd(const uint16_t* x, const uint16_t* w, const float* invar, const uint16_t* dy,
-                     int64_t M, int64_t H, uint16_t* dx, float* dw, pf8_stream_t stream);
+                     int64_t M, int64_t H, uint16_t* dx, float* dw, float* ws, int64_t ws_rows,
+                     pf8_stream_t stream);
 
 /* fused_swiglu_weighted_bwd(o1, do2_s, probs) -- transformers/fp8_utils.py:1049-1052; un-fused
  * definition ernie token_dispatcher/fp8_utils.py:1088-1092.  -> do1 bf16 [M,2I], probs_grad fp32 [M],

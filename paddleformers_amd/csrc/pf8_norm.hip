@@ -1,7 +1,10 @@
 // pf8_norm.hip -- RMSNorm forward and backward for the FP8 MLP with norm recompute
 // (FusedNormFP8MLPFunction): y = bf16(x * invar * w), invar = 1/sqrt(mean(x^2) + eps) per row.
-// HBM-bound row kernels: one workgroup per row forward, one per block of rows backward (the weight
-// gradient is accumulated per workgroup in registers and added to the fp32 output once).
+// HBM-bound row kernels: one workgroup per row forward; backward, a fixed number of workgroups walk the
+// rows with a stride, each keeps its share of the weight gradient in registers and writes it to a
+// row of a caller-provided workspace, which a second kernel sums into dw (without a workspace the
+// partial sums go to dw by atomics: every workgroup then adds to the same H addresses, and on
+// [16384, 7168] that alone takes four times as long as moving the data).
 #include "pf8_device.h"
 #include "pf8_host.h"
 #include "../../include/pf8.h"
@@ -54,7 +57,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_fwd(const uint16_t* __restrict
 template <int MAXC>   // column chunks (of 8) per thread whose weight gradient lives in registers
 __global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                       const float* __restrict__ invar, const uint16_t* __restrict__ dy, int64_t M, int64_t H,
-                                                      int rows_per_wg, uint16_t* __restrict__ dx, float* __restrict__ dw) {
+                                                      uint16_t* __restrict__ dx, float* __restrict__ dw, float* __restrict__ ws) {
     __shared__ float lds4[4];
     const int tid = threadIdx.x;
     const int64_t chunks = H / 8;
@@ -64,8 +67,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict
     for (int j = 0; j < MAXC; ++j)
 #pragma unroll
         for (int i = 0; i < 8; ++i) dwa[j][i] = 0.0f;
-    const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
-    for (int64_t r = r0; r < r0 + rows_per_wg && r < M; ++r) {
+    for (int64_t r = blockIdx.x; r < M; r += gridDim.x) {
         const uint4* xr = reinterpret_cast<const uint4*>(x + r * H);
         const uint4* dr = reinterpret_cast<const uint4*>(dy + r * H);
         const float iv = invar[r];
@@ -105,10 +107,33 @@ __global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict
 #pragma unroll
     for (int j = 0; j < MAXC; ++j) {
         const int64_t c = tid + 256 * j;
-        if (c < chunks)
+        if (c < chunks) {
+            if (ws) {
+                float* o = ws + (int64_t)blockIdx.x * H + c * 8;
+                *reinterpret_cast<f32x4*>(o) = (f32x4){dwa[j][0], dwa[j][1], dwa[j][2], dwa[j][3]};
+                *reinterpret_cast<f32x4*>(o + 4) = (f32x4){dwa[j][4], dwa[j][5], dwa[j][6], dwa[j][7]};
+            } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) atomicAdd(dw + c * 8 + i, dwa[j][i]);
+                for (int i = 0; i < 8; ++i) atomicAdd(dw + c * 8 + i, dwa[j][i]);
+            }
+        }
     }
+}
+
+// dw[c] += sum over the workspace rows, in row order (the result does not depend on scheduling)
+__global__ __launch_bounds__(256) void k_rms_norm_dw_reduce(const float* __restrict__ ws, int rows, int64_t H, float* __restrict__ dw) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= H) return;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    int r = 0;
+    for (; r + 4 <= rows; r += 4) {
+        s0 += ws[(int64_t)r * H + c];
+        s1 += ws[(int64_t)(r + 1) * H + c];
+        s2 += ws[(int64_t)(r + 2) * H + c];
+        s3 += ws[(int64_t)(r + 3) * H + c];
+    }
+    for (; r < rows; ++r) s0 += ws[(int64_t)r * H + c];
+    dw[c] += (s0 + s1) + (s2 + s3);
 }
 
 }  // namespace pf8
@@ -130,20 +155,24 @@ extern "C" int pf8_rms_norm_fwd(const uint16_t* x, const uint16_t* w, float eps,
 }
 
 extern "C" int pf8_rms_norm_bwd(const uint16_t* x, const uint16_t* w, const float* invar, const uint16_t* dy, int64_t M, int64_t H,
-                                uint16_t* dx, float* dw, pf8_stream_t stream) {
+                                uint16_t* dx, float* dw, float* ws, int64_t ws_rows, pf8_stream_t stream) {
     PF8_REQUIRE(M >= 0 && H > 0 && H % 8 == 0, "H must be a positive multiple of 8");
     PF8_REQUIRE(H <= 8 * 256 * 8, "H larger than 16384 is not supported");
     if (M == 0) return PF8_OK;
     PF8_REQUIRE(x && w && invar && dy && dx && dw, "null pointer");
     PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(w) && PF8_ALIGNED16(dy) && PF8_ALIGNED16(dx), "pointers must be 16-byte aligned");
-    // enough workgroups to fill the device, few enough that the atomics on dw stay a small share
-    int rows = (int)((M + 2047) / 2048);
-    if (rows < 1) rows = 1;
-    const int64_t wgs = (M + rows - 1) / rows;
+    PF8_REQUIRE(!ws || (ws_rows >= 1 && PF8_ALIGNED16(ws)), "the workspace must be 16-byte aligned and hold at least one row");
+    // with a workspace: as many workgroups as it has rows (1024 fill the device four deep); without: one per
+    // compute unit, to keep the atomics on dw few
+    int64_t wgs = ws ? (ws_rows < 1024 ? ws_rows : 1024) : 256;
+    if (wgs > M) wgs = M;
     const int64_t chunks = H / 8;
     hipStream_t st = (hipStream_t)stream;
-    if (chunks <= 256 * 2) hipLaunchKernelGGL(k_rms_norm_bwd<2>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, rows, dx, dw);
-    else if (chunks <= 256 * 4) hipLaunchKernelGGL(k_rms_norm_bwd<4>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, rows, dx, dw);
-    else hipLaunchKernelGGL(k_rms_norm_bwd<8>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, rows, dx, dw);
+    if (chunks <= 256 * 2) hipLaunchKernelGGL(k_rms_norm_bwd<2>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, dx, dw, ws);
+    else if (chunks <= 256 * 4) hipLaunchKernelGGL(k_rms_norm_bwd<4>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, dx, dw, ws);
+    else hipLaunchKernelGGL(k_rms_norm_bwd<8>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, dx, dw, ws);
+    int rc = pf8_check_launch(__func__);
+    if (rc || !ws) return rc;
+    hipLaunchKernelGGL(k_rms_norm_dw_reduce, dim3((unsigned)((H + 255) / 256)), dim3(256), 0, st, ws, (int)wgs, H, dw);
     return pf8_check_launch(__func__);
 }

@@ -528,7 +528,9 @@ def fused_rms_norm_ext_grad(x: torch.Tensor, norm_weight: torch.Tensor, invvar: 
         raise ValueError("invvar must have one entry per row")
     dx = torch.empty_like(x2)
     dw = torch.zeros((H,), dtype=torch.float32, device=x.device)
-    _lib.call("pf8_rms_norm_bwd", _p(x2), _p(norm_weight.contiguous()), _p(iv), _p(d2), M, H, _p(dx), _p(dw), _stream())
+    ws_rows = min(1024, max(int(M), 1))
+    ws = torch.empty((ws_rows, H), dtype=torch.float32, device=x.device)      # per-workgroup shares of dw
+    _lib.call("pf8_rms_norm_bwd", _p(x2), _p(norm_weight.contiguous()), _p(iv), _p(d2), M, H, _p(dx), _p(dw), _p(ws), ws_rows, _stream())
     return dx.reshape(x.shape), dw
 
 
