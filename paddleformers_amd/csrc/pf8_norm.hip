@@ -72,13 +72,24 @@ __global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict
         const uint4* dr = reinterpret_cast<const uint4*>(dy + r * H);
         const float iv = invar[r];
         float s1 = 0.0f;
+        uint4 xp[MAXC], dp[MAXC];          // the row stays in registers (packed) between the two passes
+#pragma unroll
+        for (int j = 0; j < MAXC; ++j) {
+            const int64_t c = tid + 256 * j;
+            xp[j] = make_uint4(0, 0, 0, 0);
+            dp[j] = make_uint4(0, 0, 0, 0);
+            if (c < chunks) {
+                xp[j] = xr[c];
+                dp[j] = dr[c];
+            }
+        }
 #pragma unroll
         for (int j = 0; j < MAXC; ++j) {
             const int64_t c = tid + 256 * j;
             if (c < chunks) {
                 float xv[8], dv[8], gv[8];
-                unpack8(xr[c], xv);
-                unpack8(dr[c], dv);
+                unpack8(xp[j], xv);
+                unpack8(dp[j], dv);
                 unpack8(wr[c], gv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
@@ -95,8 +106,8 @@ __global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict
             const int64_t c = tid + 256 * j;
             if (c < chunks) {
                 float xv[8], dv[8], gv[8], o[8];
-                unpack8(xr[c], xv);
-                unpack8(dr[c], dv);
+                unpack8(xp[j], xv);
+                unpack8(dp[j], dv);
                 unpack8(wr[c], gv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) o[i] = dv[i] * gv[i] * iv - xv[i] * k;
