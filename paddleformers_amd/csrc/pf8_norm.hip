@@ -21,6 +21,7 @@ __device__ __forceinline__ float block_sum(float v, float* lds4) {
     return (lds4[0] + lds4[1]) + (lds4[2] + lds4[3]);
 }
 
+template <int MAXC>   // column chunks (of 8) per thread, kept packed in registers between the two passes (0: re-read)
 __global__ __launch_bounds__(256) void k_rms_norm_fwd(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float eps, int64_t M,
                                                       int64_t H, uint16_t* __restrict__ y, float* __restrict__ invar) {
     __shared__ float lds4[4];
@@ -28,21 +29,37 @@ __global__ __launch_bounds__(256) void k_rms_norm_fwd(const uint16_t* __restrict
     const int tid = threadIdx.x;
     const int64_t chunks = H / 8;
     const uint4* xr = reinterpret_cast<const uint4*>(x + r * H);
+    uint4 xp[MAXC > 0 ? MAXC : 1];
     float ss = 0.0f;
-    for (int64_t c = tid; c < chunks; c += 256) {
-        float v[8];
-        unpack8(xr[c], v);
+    if (MAXC > 0) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ss = __builtin_fmaf(v[i], v[i], ss);
+        for (int j = 0; j < MAXC; ++j) {
+            const int64_t c = tid + 256 * j;
+            xp[j] = c < chunks ? xr[c] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < MAXC; ++j) {
+            float v[8];
+            unpack8(xp[j], v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = __builtin_fmaf(v[i], v[i], ss);
+        }
+    } else {
+        for (int64_t c = tid; c < chunks; c += 256) {
+            float v[8];
+            unpack8(xr[c], v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = __builtin_fmaf(v[i], v[i], ss);
+        }
     }
     ss = block_sum(ss, lds4);
     const float iv = 1.0f / __builtin_sqrtf(ss / (float)H + eps);
     if (tid == 0) invar[r] = iv;
     uint4* yr = reinterpret_cast<uint4*>(y + r * H);
     const uint4* wr = reinterpret_cast<const uint4*>(w);
-    for (int64_t c = tid; c < chunks; c += 256) {
+    auto emit = [&](int64_t c, uint4 xw) {
         float v[8], g[8];
-        unpack8(xr[c], v);
+        unpack8(xw, v);
         unpack8(wr[c], g);
         uint4 o;
         o.x = pack_bf16(v[0] * iv * g[0], v[1] * iv * g[1]);
@@ -50,6 +67,15 @@ __global__ __launch_bounds__(256) void k_rms_norm_fwd(const uint16_t* __restrict
         o.z = pack_bf16(v[4] * iv * g[4], v[5] * iv * g[5]);
         o.w = pack_bf16(v[6] * iv * g[6], v[7] * iv * g[7]);
         yr[c] = o;
+    };
+    if (MAXC > 0) {
+#pragma unroll
+        for (int j = 0; j < MAXC; ++j) {
+            const int64_t c = tid + 256 * j;
+            if (c < chunks) emit(c, xp[j]);
+        }
+    } else {
+        for (int64_t c = tid; c < chunks; c += 256) emit(c, xr[c]);
     }
 }
 
@@ -161,7 +187,12 @@ extern "C" int pf8_rms_norm_fwd(const uint16_t* x, const uint16_t* w, float eps,
     PF8_REQUIRE(M <= 0x7FFFFFFF, "too many rows");
     PF8_REQUIRE(x && w && y && invar, "null pointer");
     PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(w) && PF8_ALIGNED16(y), "pointers must be 16-byte aligned");
-    hipLaunchKernelGGL(k_rms_norm_fwd, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, x, w, eps, M, H, y, invar);
+    const int64_t chunks = H / 8;
+    hipStream_t st = (hipStream_t)stream;
+    if (chunks <= 256 * 2) hipLaunchKernelGGL(k_rms_norm_fwd<2>, dim3((unsigned)M), dim3(256), 0, st, x, w, eps, M, H, y, invar);
+    else if (chunks <= 256 * 4) hipLaunchKernelGGL(k_rms_norm_fwd<4>, dim3((unsigned)M), dim3(256), 0, st, x, w, eps, M, H, y, invar);
+    else if (chunks <= 256 * 8) hipLaunchKernelGGL(k_rms_norm_fwd<8>, dim3((unsigned)M), dim3(256), 0, st, x, w, eps, M, H, y, invar);
+    else hipLaunchKernelGGL(k_rms_norm_fwd<0>, dim3((unsigned)M), dim3(256), 0, st, x, w, eps, M, H, y, invar);
     return pf8_check_launch(__func__);
 }
 
