@@ -16,6 +16,7 @@ struct PermuteArgs {
 
 // One workgroup per expert: rank the tokens routed to it (stable in token order) with wave ballots
 // and a running offset, fill its column of the row map, clear its padding rows' probabilities.
+template <int TOPK>   // compile-time top-k (a multiple of 4: the routing row is read as 16-byte words), 0 = generic
 __global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restrict__ routemap, int64_t T, int topk, PermuteArgs pa,
                                                         int32_t* __restrict__ rowmap, float* __restrict__ out_probs,
                                                         int32_t* __restrict__ overflow) {
@@ -35,8 +36,17 @@ __global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restri
         for (int j = 0; j < J; ++j) {
             const int64_t t = t0 + j * 1024 + tid;
             hit[j] = false;
-            if (t < T)
-                for (int k = 0; k < topk; ++k) hit[j] |= routemap[t * topk + k] == e;
+            if (t < T) {
+                if (TOPK > 0) {
+#pragma unroll
+                    for (int k = 0; k < TOPK; k += 4) {
+                        const int4 v = *reinterpret_cast<const int4*>(routemap + t * TOPK + k);
+                        hit[j] |= v.x == e || v.y == e || v.z == e || v.w == e;
+                    }
+                } else {
+                    for (int k = 0; k < topk; ++k) hit[j] |= routemap[t * topk + k] == e;
+                }
+            }
         }
 #pragma unroll
         for (int j = 0; j < J; ++j) {
@@ -184,7 +194,10 @@ extern "C" int pf8_moe_permute(const void* x, int x_is_fp8, const float* xs, con
     PF8_REQUIRE(T == 0 || (x && routemap && PF8_ALIGNED16(x)), "null or misaligned input");
     hipStream_t st = (hipStream_t)stream;
     const int64_t scale_cols = xs ? H / 128 : 0;
-    hipLaunchKernelGGL(k_permute_rowmap, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
+    const bool rm16 = (reinterpret_cast<uintptr_t>(routemap) & 15u) == 0;
+    if (topk == 8 && rm16) hipLaunchKernelGGL(k_permute_rowmap<8>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
+    else if (topk == 4 && rm16) hipLaunchKernelGGL(k_permute_rowmap<4>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
+    else hipLaunchKernelGGL(k_permute_rowmap<0>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
     int rc = pf8_check_launch(__func__);
     if (rc) return rc;
     if (max_pad > 0 && row_bytes > 0) {
