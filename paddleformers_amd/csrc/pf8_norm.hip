@@ -157,20 +157,44 @@ __global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict
     }
 }
 
-// dw[c] += sum over the workspace rows, in row order (the result does not depend on scheduling)
-__global__ __launch_bounds__(256) void k_rms_norm_dw_reduce(const float* __restrict__ ws, int rows, int64_t H, float* __restrict__ dw) {
-    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (c >= H) return;
-    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
-    int r = 0;
-    for (; r + 4 <= rows; r += 4) {
-        s0 += ws[(int64_t)r * H + c];
-        s1 += ws[(int64_t)(r + 1) * H + c];
-        s2 += ws[(int64_t)(r + 2) * H + c];
-        s3 += ws[(int64_t)(r + 3) * H + c];
+// dw[c] += sum over the workspace rows, in a fixed order (the result does not depend on scheduling). A workgroup
+// owns 64 columns: 16 lanes of four floats across, 64 row slots down; a slot sums the rows r = slot, slot + 64, ...
+// and the slots are folded through LDS in slot order.
+__global__ __launch_bounds__(1024) void k_rms_norm_dw_reduce(const float* __restrict__ ws, int rows, int64_t H, float* __restrict__ dw) {
+    __shared__ f32x4 part[64][16];
+    const int lane = threadIdx.x & 15, slot = threadIdx.x >> 4;
+    const int64_t c4 = (int64_t)blockIdx.x * 16 + lane;
+    const bool live = c4 * 4 < H;
+    f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0, s2 = s0, s3 = s0;
+    if (live) {
+        const float* col = ws + c4 * 4;
+        int r = slot;
+        for (; r + 192 < rows; r += 256) {
+            const f32x4 v0 = *reinterpret_cast<const f32x4*>(col + (int64_t)r * H);
+            const f32x4 v1 = *reinterpret_cast<const f32x4*>(col + (int64_t)(r + 64) * H);
+            const f32x4 v2 = *reinterpret_cast<const f32x4*>(col + (int64_t)(r + 128) * H);
+            const f32x4 v3 = *reinterpret_cast<const f32x4*>(col + (int64_t)(r + 192) * H);
+            s0 += v0; s1 += v1; s2 += v2; s3 += v3;
+        }
+        for (; r < rows; r += 64) s0 += *reinterpret_cast<const f32x4*>(col + (int64_t)r * H);
     }
-    for (; r < rows; ++r) s0 += ws[(int64_t)r * H + c];
-    dw[c] += (s0 + s1) + (s2 + s3);
+    part[slot][lane] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const int64_t c = (int64_t)blockIdx.x * 64 + threadIdx.x;
+        if (c < H) {
+            const float* pl = reinterpret_cast<const float*>(&part[0][0]) + threadIdx.x;
+            float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 64; k += 4) {
+                t0 += pl[k * 64];
+                t1 += pl[(k + 1) * 64];
+                t2 += pl[(k + 2) * 64];
+                t3 += pl[(k + 3) * 64];
+            }
+            dw[c] += (t0 + t1) + (t2 + t3);
+        }
+    }
 }
 
 }  // namespace pf8
@@ -215,6 +239,6 @@ extern "C" int pf8_rms_norm_bwd(const uint16_t* x, const uint16_t* w, const floa
     else hipLaunchKernelGGL(k_rms_norm_bwd<8>, dim3((unsigned)wgs), dim3(256), 0, st, x, w, invar, dy, M, H, dx, dw, ws);
     int rc = pf8_check_launch(__func__);
     if (rc || !ws) return rc;
-    hipLaunchKernelGGL(k_rms_norm_dw_reduce, dim3((unsigned)((H + 255) / 256)), dim3(256), 0, st, ws, (int)wgs, H, dw);
+    hipLaunchKernelGGL(k_rms_norm_dw_reduce, dim3((unsigned)((H + 63) / 64)), dim3(1024), 0, st, ws, (int)wgs, H, dw);
     return pf8_check_launch(__func__);
 }
