@@ -614,7 +614,11 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
     const int64_t per_xcd = (T + 7) / 8;
     const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (logical >= T) return;
-    const int64_t p_tile = logical % p_tiles, q_tile = logical / p_tiles;
+    // tiles are walked in strips eight P tiles wide, P fastest inside a strip: the 64 workgroups an XCD
+    // runs at a time then cover about 8 x 8 tiles and share 16 operand panels in its L2 instead of 34
+    const int64_t strip_w = 8 * q_tiles, strip = logical / strip_w, in_strip = logical - strip * strip_w;
+    const int64_t strip_p = p_tiles - strip * 8 < 8 ? p_tiles - strip * 8 : 8;
+    const int64_t p_tile = strip * 8 + in_strip % strip_p, q_tile = in_strip / strip_p;
     const int64_t p0 = p_tile * 128, q0 = q_tile * 128;
 
     const uint8_t* pbase = a.p;
