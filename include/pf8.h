@@ -100,6 +100,15 @@ int pf8_transpose_split_quant(const void* x, const float* xs, int x_is_fp8, int 
                               const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q_t, float* s_t,
                               int pow2, pf8_stream_t stream);
 
+/* The two quantizations the MoE node's backward applies to the SAME bf16 gradient, from one read:
+ * fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True, using_pow2_scale=pow2_rows)
+ * for the dgrad GEMM and fused_transpose_split_quant(x, None, tokens_per_expert, pow2_t) for the wgrad
+ * GEMM -- out_grad at transformers/fp8_utils.py:1030-1036 and :1115, do1 at :1073-1079 and :1168.  q e4m3 [Mtot,K], s fp32 [K/128,Mtot]; q_t / s_t packed as pf8_transpose_split_quant
+ * writes them.  Every output is bit-identical to the separate calls'. */
+int pf8_quant_and_transpose_split(const uint16_t* x, const int64_t* rows_per_expert, int E, int64_t K,
+                                  uint8_t* q, float* s, int pow2_rows, uint8_t* q_t, float* s_t,
+                                  int pow2_t, pf8_stream_t stream);
+
 /* fused_act_dequant(q, s) -- transformers/fp8_utils.py:136-138, 779.  1x128 dequant to bf16. */
 int pf8_act_dequant(const uint8_t* q, const float* s, int scale_layout, int64_t M, int64_t K,
                     uint16_t* out, pf8_stream_t stream);

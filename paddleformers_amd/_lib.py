@@ -27,6 +27,7 @@ SIGNATURES = {
     "pf8_stack_quant_both": [_vp, _i32, _i64, _i64, _vp, _vp, _vp, _vp, _i32, _vp],
     "pf8_swiglu_weighted_quant": [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i32, _i32, _vp],
     "pf8_transpose_split_quant": [_vp, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp, _i32, _vp],
+    "pf8_quant_and_transpose_split": [_vp, _vp, _i32, _i64, _vp, _vp, _i32, _vp, _vp, _i32, _vp],
     "pf8_act_dequant": [_vp, _vp, _i32, _i64, _i64, _vp, _vp],
     "pf8_weight_dequant": [_vp, _vp, _i64, _i64, _vp, _vp],
     "pf8_block_dequant": [_vp, _vp, _i32, _i64, _i64, _i64, _i64, _i64, _vp, _i32, _vp],

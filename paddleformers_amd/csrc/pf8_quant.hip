@@ -362,6 +362,7 @@ __device__ __forceinline__ void load_patch_packed(const TileSrc& src, int64_t ro
 // Row-scaled copy (optional) + column-scaled transposed copy of one 128x128 tile.
 //   SPLIT=false: q[M,K] + s, qt[K,M] + st                (fused quant+transpose)
 //   SPLIT=true : qt / st packed per expert               (transpose-split-quant), source bf16 or e4m3
+// pow2: bit 0 = power-of-two scales for the transposed copy, bit 1 = for the row-scaled copy.
 // Per element the kernel spends one masked copy, two packed-u16 max (row and column amax), one
 // unpack and two bracketing conversions; the 128 row scales and 128 column scales are each computed
 // once (threads 0..127 / 128..255) and handed round through LDS instead of sixteen times over.
@@ -416,7 +417,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
             am = (c & 1) ? (pk & 0xFFFF0000u) : (pk << 16);
         }
         if (tid >= 128 || want_rows) {
-            const TileScale t = make_scale(am, pow2 != 0);
+            const TileScale t = make_scale(am, (pow2 & (tid < 128 ? 2 : 1)) != 0);
             lds_sc[tid] = make_float4(t.s, t.r_lo, t.r_hi, t.slow ? 1.0f : 0.0f);
         }
     }
@@ -429,7 +430,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float4 f = lds_sc[8 * g + i];
-            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f; t.exact = pow2 != 0;
+            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f; t.exact = (pow2 & 2) != 0;
             const int64_t r = row0 + 8 * g + i;
             float v[8];
             unpack8(w[i], v);
@@ -454,7 +455,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
         for (int h = 0; h < 2; ++h) {
             const int j = 2 * k + h;
             const float4 f = lds_sc[128 + 8 * l + j];
-            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f; t.exact = pow2 != 0;
+            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f; t.exact = (pow2 & 1) != 0;
             cs[j] = t.s;
             lds_put_col(lds_t, l, g, j, h == 0 ? quant8(lo, t) : quant8(hi, t));
         }
@@ -745,34 +746,38 @@ extern "C" int pf8_quant_transpose(const uint16_t* x, int64_t M, int64_t K, uint
     SplitArgs sp = {};
     dim3 grid((unsigned)(K / 128), (unsigned)(M / 128)), block(256);
     if (scale_layout == 0)
-        hipLaunchKernelGGL((k_quant_rowcol<false, 0>), grid, block, 0, (hipStream_t)stream, src, M, K, q, s, q_t, s_t, sp, pow2);
+        hipLaunchKernelGGL((k_quant_rowcol<false, 0>), grid, block, 0, (hipStream_t)stream, src, M, K, q, s, q_t, s_t, sp, pow2 ? 3 : 0);
     else
-        hipLaunchKernelGGL((k_quant_rowcol<false, 1>), grid, block, 0, (hipStream_t)stream, src, M, K, q, s, q_t, s_t, sp, pow2);
+        hipLaunchKernelGGL((k_quant_rowcol<false, 1>), grid, block, 0, (hipStream_t)stream, src, M, K, q, s, q_t, s_t, sp, pow2 ? 3 : 0);
     return pf8_check_launch(__func__);
 }
 
-extern "C" int pf8_transpose_split_quant(const void* x, const float* xs, int x_is_fp8, int xs_layout, const int64_t* rows_per_expert,
-                                         int E, int64_t K, uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream) {
-    PF8_REQUIRE(xs_layout == 0 || xs_layout == 1, "xs_layout must be 0 or 1");
-    PF8_REQUIRE(E >= 0 && K >= 0, "negative shape");
-    PF8_REQUIRE(K % 128 == 0, "K must be a multiple of 128");
-    PF8_REQUIRE(E <= 256, "at most 256 experts per call");
+// shared by pf8_transpose_split_quant and pf8_quant_and_transpose_split: q/s null = no row-scaled copy
+static int transpose_split_quant(const char* where, const void* x, const float* xs, int x_is_fp8, int xs_layout,
+                                 const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
+                                 int pow2_bits, pf8_stream_t stream) {
+#define PF8_REQUIRE_AT(cond, msg) do { if (!(cond)) return pf8_fail(PF8_EINVAL, where, msg); } while (0)
+    PF8_REQUIRE_AT(xs_layout == 0 || xs_layout == 1, "xs_layout must be 0 or 1");
+    PF8_REQUIRE_AT(E >= 0 && K >= 0, "negative shape");
+    PF8_REQUIRE_AT(K % 128 == 0, "K must be a multiple of 128");
+    PF8_REQUIRE_AT(E <= 256, "at most 256 experts per call");
     if (E == 0 || K == 0) return PF8_OK;
-    PF8_REQUIRE(rows_per_expert, "null pointer");
+    PF8_REQUIRE_AT(rows_per_expert, "null pointer");
     SplitArgs sp = {};
     int64_t total = 0;
     for (int e = 0; e < E; ++e) {
-        PF8_REQUIRE(rows_per_expert[e] >= 0 && rows_per_expert[e] % 128 == 0, "rows_per_expert entries must be non-negative multiples of 128");
+        PF8_REQUIRE_AT(rows_per_expert[e] >= 0 && rows_per_expert[e] % 128 == 0, "rows_per_expert entries must be non-negative multiples of 128");
         sp.tile_start[e] = (int32_t)(total / 128);
         total += rows_per_expert[e];
     }
-    PF8_REQUIRE(total / 128 <= 65535, "too many rows");
+    PF8_REQUIRE_AT(total / 128 <= 65535, "too many rows");
     sp.tile_start[E] = (int32_t)(total / 128);
     sp.E = E;
     if (total == 0) return PF8_OK;
-    PF8_REQUIRE(x && q_t && s_t, "null pointer");
-    PF8_REQUIRE(!x_is_fp8 || xs, "fp8 input needs its scales");
-    PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q_t) && PF8_ALIGNED16(s_t), "pointers must be 16-byte aligned");
+    PF8_REQUIRE_AT(x && q_t && s_t, "null pointer");
+    PF8_REQUIRE_AT(!x_is_fp8 || xs, "fp8 input needs its scales");
+    PF8_REQUIRE_AT(PF8_ALIGNED16(x) && PF8_ALIGNED16(q_t) && PF8_ALIGNED16(s_t) && PF8_ALIGNED16(q), "pointers must be 16-byte aligned");
+#undef PF8_REQUIRE_AT
     TileSrc src;
     src.x = x_is_fp8 ? nullptr : (const uint16_t*)x;
     src.xq = x_is_fp8 ? (const uint8_t*)x : nullptr;
@@ -781,9 +786,19 @@ extern "C" int pf8_transpose_split_quant(const void* x, const float* xs, int x_i
     src.rows = total;
     src.xs_layout = xs_layout;
     dim3 grid((unsigned)(K / 128), (unsigned)(total / 128)), block(256);
-    hipLaunchKernelGGL((k_quant_rowcol<true, 1>), grid, block, 0, (hipStream_t)stream, src, total, K, (uint8_t*)nullptr,
-                       (float*)nullptr, q_t, s_t, sp, pow2);
-    return pf8_check_launch(__func__);
+    hipLaunchKernelGGL((k_quant_rowcol<true, 1>), grid, block, 0, (hipStream_t)stream, src, total, K, q, s, q_t, s_t, sp, pow2_bits);
+    return pf8_check_launch(where);
+}
+
+extern "C" int pf8_transpose_split_quant(const void* x, const float* xs, int x_is_fp8, int xs_layout, const int64_t* rows_per_expert,
+                                         int E, int64_t K, uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream) {
+    return transpose_split_quant(__func__, x, xs, x_is_fp8, xs_layout, rows_per_expert, E, K, nullptr, nullptr, q_t, s_t, pow2 ? 1 : 0, stream);
+}
+
+extern "C" int pf8_quant_and_transpose_split(const uint16_t* x, const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q, float* s,
+                                             int pow2_rows, uint8_t* q_t, float* s_t, int pow2_t, pf8_stream_t stream) {
+    PF8_REQUIRE(q && s, "null pointer");
+    return transpose_split_quant(__func__, x, nullptr, 0, 0, rows_per_expert, E, K, q, s, q_t, s_t, (pow2_t ? 1 : 0) | (pow2_rows ? 2 : 0), stream);
 }
 
 extern "C" int pf8_swiglu_weighted_quant(const uint16_t* o1, const float* probs, int64_t M, int64_t I, uint8_t* q, float* s,

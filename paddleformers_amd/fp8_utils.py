@@ -565,6 +565,9 @@ class FP8GroupGemmMlpFunctionNode:
         # (block-scaled MFMA kernel).  Pre-quantized inputs handed in as (fp8, scale) pairs must then
         # carry power-of-two scales as well.
         self.use_ue8m0 = use_ue8m0
+        # backward quantizes out_grad and do1 twice each (row-wise for the dgrad GEMM, transposed per expert
+        # for the wgrad GEMM); with this set both come from one read of the gradient, bit-identical
+        self.fuse_bwd_quant = True
         self._group_items = None
         self.m_indices = None
         self.input = None
@@ -688,14 +691,19 @@ class FP8GroupGemmMlpFunctionNode:
         return do1, o2_s, probs_grad
 
     def bwd_gate_up_input(self, do1, expert_w1, tokens_per_expert, m_indices=None, dx=None):
-        """dx [m_sum, H] = do1 . w1^T (fp8_utils.py:1058-1094)."""
+        """dx [m_sum, H] = do1 . w1^T (fp8_utils.py:1058-1094).  do1: bf16, or the (fp8, scale) pair of
+        its row-wise quantization (scale [m_sum, 2I/128] as a view of [2I/128, m_sum] memory)."""
         bw_w1_quant, bw_w1_scale = self._stacked(expert_w1, False, len(expert_w1))
-        do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, output_scale_transpose=True, quant_method="1x128", input_transpose=False,
-                                                    using_pow2_scale=self.use_ue8m0)
-        do1_scale = do1_scale.T
+        if isinstance(do1, tuple):
+            do1_fp8, do1_scale = do1
+        else:
+            do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, output_scale_transpose=True, quant_method="1x128", input_transpose=False,
+                                                        using_pow2_scale=self.use_ue8m0)
+            do1_scale = do1_scale.T
+        do1 = do1_fp8
         dx_shape = [do1_fp8.shape[0], bw_w1_quant.shape[1]]
-        if dx is None or dx.dtype != do1.dtype:
-            dx = torch.empty(dx_shape, dtype=do1.dtype, device=do1.device)
+        if dx is None or dx.dtype != torch.bfloat16:
+            dx = torch.empty(dx_shape, dtype=torch.bfloat16, device=do1.device)
         else:
             assert list(dx.shape) == dx_shape, f"{list(dx.shape)} vs {dx_shape}"
         if numpy.prod(do1_fp8.shape) != 0:
@@ -764,7 +772,8 @@ class FP8GroupGemmMlpFunctionNode:
 
     def bwd_gate_up_weight(self, do1, input_x, expert_w1, tokens_per_expert, input_fp8_slice=None, input_scale_slice=None,
                            clear_input=False):
-        """dw1[e] [H, 2I] += x_e^T . do1_e (fp8_utils.py:1136-1189)."""
+        """dw1[e] [H, 2I] += x_e^T . do1_e (fp8_utils.py:1136-1189).  do1: bf16, or the (fp8_t, scale_t)
+        lists fused_transpose_split_quant(do1, None, tokens_per_expert, True) returns."""
         if input_x is None:
             inp = (input_fp8_slice, input_scale_slice) if self.bwd_subbatch else (self.input_fp8, self.input_scale)
             input_x_t_fp8, input_x_t_scale = self.fused_transpose_split_quant(inp[0], inp[1], tokens_per_expert, True)
@@ -774,7 +783,10 @@ class FP8GroupGemmMlpFunctionNode:
             self.input_fp8 = None
             self.input_scale = None
             self.input = None
-        do1_t_fp8, do1_t_scale = self.fused_transpose_split_quant(do1, None, tokens_per_expert, True)
+        if isinstance(do1, tuple):
+            do1_t_fp8, do1_t_scale = do1
+        else:
+            do1_t_fp8, do1_t_scale = self.fused_transpose_split_quant(do1, None, tokens_per_expert, True)
         fn = partial(self._expert_wgrads, input_x_t_fp8, input_x_t_scale, do1_t_fp8, do1_t_scale, expert_w1, True)
         if WeightGradStore.enabled:
             WeightGradStore.put(fn)
@@ -827,19 +839,33 @@ class FP8GroupGemmMlpFunctionNode:
             o1 = self.fwd_gate_up(inp, expert_w1, len(expert_w1), tokens_per_expert, m_indices=m_indices)
         else:
             o1 = self.o1
+        # one read per gradient for its two quantizations (not for the split-GEMM loop, which wants plain
+        # per-expert tensors, nor beyond the 256 experts one launch of the quantizer takes)
+        fuse = self.fuse_bwd_quant and not self.is_split_group_gemm and len(tokens_per_expert) <= 256
+        do3_t = None
+        if fuse and not isinstance(out_grad, tuple) and out_grad.dtype == torch.bfloat16:
+            g_fp8, g_scale, g_t_fp8, g_t_scale = F8.quant_and_transpose_split(out_grad, tokens_per_expert, self.use_ue8m0, True)
+            out_grad, do3_t = (g_fp8, g_scale.T), (g_t_fp8, g_t_scale)
         do1, o2_s, probs_grad = self.bwd_dowm_input(expert_w2, out_grad, o1, tokens_per_expert, unzipped_probs=unzipped_probs,
                                                     m_indices=m_indices)
         del o1
         self.o1 = None
-        self.bwd_gate_up_weight(do1, None, expert_w1, tokens_per_expert, input_fp8_slice=input_fp8_slice,
+        do1_rows = do1_t = do1
+        if fuse:
+            d_fp8, d_scale, d_t_fp8, d_t_scale = F8.quant_and_transpose_split(do1, tokens_per_expert, self.use_ue8m0, True)
+            do1_rows, do1_t = (d_fp8, d_scale.T), (d_t_fp8, d_t_scale)
+        del do1
+        self.bwd_gate_up_weight(do1_t, None, expert_w1, tokens_per_expert, input_fp8_slice=input_fp8_slice,
                                 input_scale_slice=input_scale_slice, clear_input=reset_status)
         if reset_status:
             self.input_fp8 = None
             self.input_scale = None
             self.input = None
-        dx = self.bwd_gate_up_input(do1, expert_w1, tokens_per_expert, dx=None, m_indices=m_indices)
-        del do1
-        if isinstance(out_grad, tuple):
+        dx = self.bwd_gate_up_input(do1_rows, expert_w1, tokens_per_expert, dx=None, m_indices=m_indices)
+        del do1_rows, do1_t
+        if do3_t is not None:
+            self.bwd_down_weight(do3_t, o2_s, expert_w2, tokens_per_expert, scales_pow2=True)
+        elif isinstance(out_grad, tuple):
             do3_fp8, do3_scale = self.fused_transpose_split_quant(out_grad[0], out_grad[1], tokens_per_expert, True)
             self.bwd_down_weight((do3_fp8, do3_scale), o2_s, expert_w2, tokens_per_expert, scales_pow2=True)
         else:

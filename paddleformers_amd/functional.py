@@ -290,6 +290,44 @@ def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], 
     return qs, ss
 
 
+def quant_and_transpose_split(x: torch.Tensor, tokens_per_expert: Sequence[int], using_pow2_scale: bool = False,
+                              pow_2_scales: bool = True):
+    """fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True, using_pow2_scale=...) and
+    fused_transpose_split_quant(x, None, tokens_per_expert, pow_2_scales) from ONE read of x: the two
+    quantizations the MoE node's backward applies to the same gradient (transformers/fp8_utils.py:1030-1036
+    with :1115, :1073-1079 with :1168).  Returns (q [M,K], s [K/128,M], q_t list, s_t list), each
+    bit-identical to the separate calls' outputs.  At most 256 experts."""
+    _dev(x, "x")
+    if x.dim() != 2 or x.dtype != torch.bfloat16:
+        raise ValueError("x must be a 2-D bfloat16 tensor")
+    if not x.is_contiguous():
+        x = x.contiguous()
+    Mtot, K = x.shape
+    rows = [int(t) for t in tokens_per_expert]
+    if sum(rows) != Mtot:
+        raise ValueError(f"tokens_per_expert sums to {sum(rows)} but x has {Mtot} rows")
+    if any(r % 128 != 0 or r < 0 for r in rows):
+        raise ValueError("every tokens_per_expert entry must be a non-negative multiple of 128")
+    if K % 128 != 0:
+        raise ValueError(f"last dimension must be divisible by 128, got {K}")
+    if len(rows) > 256:
+        raise ValueError("at most 256 experts")
+    q = torch.empty((Mtot, K), dtype=FP8, device=x.device)
+    s = torch.empty((K // 128, Mtot), dtype=torch.float32, device=x.device)
+    q_t = torch.empty((K * Mtot,), dtype=FP8, device=x.device)
+    s_t = torch.empty(((Mtot // 128) * K,), dtype=torch.float32, device=x.device)
+    if Mtot and K:
+        arr = (C.c_int64 * len(rows))(*rows)
+        _lib.call("pf8_quant_and_transpose_split", _p(x), arr, len(rows), K, _p(q), _p(s), int(bool(using_pow2_scale)),
+                  _p(q_t), _p(s_t), int(bool(pow_2_scales)), _stream())
+    qs, ss, off = [], [], 0
+    for r in rows:
+        qs.append(q_t[off * K:(off + r) * K].view(K, r))
+        ss.append(s_t[(off // 128) * K:((off + r) // 128) * K].view(r // 128, K))
+        off += r
+    return q, s, qs, ss
+
+
 # ---------------------------------------------------------------------------------------------
 # dequantizers
 # ---------------------------------------------------------------------------------------------

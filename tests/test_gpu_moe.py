@@ -286,3 +286,30 @@ def test_moe_node_ue8m0_needs_a_pow2_weight_cache():
     U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True, using_pow2_scale=True)
     cached = U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True).forward(G.to_torch_bf16(x), tp, rows)
     assert torch.equal(plain.view(torch.int16), cached.view(torch.int16))
+
+
+@pytest.mark.parametrize("ue8m0", [False, True])
+def test_moe_node_backward_fused_gradient_quantization_is_bit_identical(ue8m0):
+    # backward quantizes out_grad and do1 once (row-wise + transposed from one read) or twice (the
+    # reference's call sequence): same dx, probs_grad and weight gradients to the bit
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 3, 512, 384
+    rows = [256, 0, 384]
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=31)
+    dout = G.to_torch_bf16(G.bf16_normal((sum(rows), H), seed=33, std=1e-3))
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    res = []
+    for fuse in (True, False):
+        for ex in experts:
+            ex.w1.main_grad = torch.zeros_like(ex.w1, dtype=torch.float32)
+            ex.w2.main_grad = torch.zeros_like(ex.w2, dtype=torch.float32)
+        node = FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=ue8m0)
+        node.fuse_bwd_quant = fuse
+        node.forward(G.to_torch_bf16(x), tp, rows)
+        dx, pg = node.backward(dout, tp, rows)
+        res.append((dx, pg, [ex.w1.main_grad for ex in experts], [ex.w2.main_grad for ex in experts]))
+    a, b = res
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    for ga, gb in zip(a[2] + a[3], b[2] + b[3]):
+        assert torch.equal(ga, gb)

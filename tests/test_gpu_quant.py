@@ -398,6 +398,42 @@ def test_fused_transpose_split_quant_fp8_input(F, scale_transposed):
             _scales_same(ss[e].cpu().numpy(), ess[e], f"expert {e} scales")
 
 
+@pytest.mark.parametrize("rows", [[128], [256, 0, 128], [0, 0, 384, 128, 0]])
+@pytest.mark.parametrize("pow2_rows", [False, True])
+def test_quant_and_transpose_split_equals_the_two_separate_quantizers(F, rows, pow2_rows):
+    # one read, both quantizations of the MoE backward: row-wise 1x128 (scales [K/128, M]) and the
+    # per-expert transposed copy with power-of-two scales
+    K = 384
+    M = sum(rows)
+    bits = G.bf16_normal((M, K), seed=3 * M + len(rows), outlier_frac=1e-3, outlier_scale=100.0)
+    q, s, qs, ss = F.quant_and_transpose_split(G.to_torch_bf16(bits), rows, pow2_rows, True)
+    eq, es = O.quant_1x128(bits, 1, pow2=pow2_rows)
+    _same(G.from_torch_fp8(q), eq, "row-wise bytes")
+    _scales_same(s.cpu().numpy(), es, "row-wise scales")
+    eqs, ess = O.transpose_split_quant(bits, None, rows, True)
+    for e, r in enumerate(rows):
+        assert tuple(qs[e].shape) == (K, r) and tuple(ss[e].shape) == (r // 128, K)
+        if r:
+            _same(G.from_torch_fp8(qs[e]), eqs[e], f"expert {e} bytes")
+            _scales_same(ss[e].cpu().numpy(), ess[e], f"expert {e} scales")
+    # and against the library's own separate entry points
+    q1, s1 = F.fp8_quant_blockwise(G.to_torch_bf16(bits), output_scale_transpose=True, quant_method="1x128", input_transpose=False,
+                                   using_pow2_scale=pow2_rows)
+    assert torch.equal(q1.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s1, s)
+
+
+def test_quant_and_transpose_split_rejects_bad_input(F):
+    x = torch.zeros((256, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        F.quant_and_transpose_split(x, [128, 64, 64])
+    with pytest.raises(ValueError):
+        F.quant_and_transpose_split(x, [128])
+    with pytest.raises(ValueError):
+        F.quant_and_transpose_split(x.float(), [256])
+    q, s, qs, ss = F.quant_and_transpose_split(torch.zeros((0, 256), dtype=torch.bfloat16, device="cuda"), [0, 0])
+    assert tuple(q.shape) == (0, 256) and len(qs) == 2
+
+
 # ---------------------------------------------------------------------------------------------
 # dequantizers and SwiGLU backward
 # ---------------------------------------------------------------------------------------------
