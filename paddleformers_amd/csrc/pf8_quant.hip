@@ -348,12 +348,11 @@ __device__ __forceinline__ void load_patch_packed(const TileSrc& src, int64_t ro
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float f[8];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                f[j] = e4m3_to_f32((q[i].x >> (8 * j)) & 0xFFu) * sc[i];
-                f[4 + j] = e4m3_to_f32((q[i].y >> (8 * j)) & 0xFFu) * sc[i];
-            }
+            // hardware e4m3 -> fp32 (exact), two bytes per instruction
+            const f32x2 a0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[i].x, false), a1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[i].x, true);
+            const f32x2 b0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[i].y, false), b1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[i].y, true);
+            const float f[8] = {a0[0] * sc[i], a0[1] * sc[i], a1[0] * sc[i], a1[1] * sc[i],
+                                b0[0] * sc[i], b0[1] * sc[i], b1[0] * sc[i], b1[1] * sc[i]};
             w[i] = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
         }
     }
