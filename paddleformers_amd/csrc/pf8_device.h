@@ -243,6 +243,12 @@ __device__ __forceinline__ float e4m3_to_f32(uint32_t c) {
     return u2f(f2u(v) | sign);
 }
 
+// four e4m3 codes of one word -> fp32 with the hardware convert (exact, two bytes per instruction)
+__device__ __forceinline__ void e4m3x4_to_f32(uint32_t w, float* f) {
+    const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    f[0] = lo[0]; f[1] = lo[1]; f[2] = hi[0]; f[3] = hi[1];
+}
+
 // expf restated operation for operation from the CPU checker: clamp, Cody-Waite reduction with two
 // fused steps, degree-5 Horner polynomial with fused multiply-adds, exact power-of-two scaling.
 __device__ __forceinline__ float expf_fixed(float x) {

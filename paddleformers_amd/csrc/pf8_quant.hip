@@ -249,11 +249,11 @@ __device__ __forceinline__ void load_patch(const TileSrc& src, int64_t row0, int
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
+            float f[8];
+            e4m3x4_to_f32(w[i].x, f);
+            e4m3x4_to_f32(w[i].y, f + 4);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v[i][j] = round_bf16(e4m3_to_f32((w[i].x >> (8 * j)) & 0xFFu) * sc[i]);
-                v[i][4 + j] = round_bf16(e4m3_to_f32((w[i].y >> (8 * j)) & 0xFFu) * sc[i]);
-            }
+            for (int j = 0; j < 8; ++j) v[i][j] = round_bf16(f[j] * sc[i]);
         }
     }
 }
@@ -510,11 +510,10 @@ __global__ __launch_bounds__(256) void k_act_dequant(const uint8_t* __restrict__
     const float sc = LAYOUT == 0 ? s[r * KB + kb] : s[kb * M + r];
     uint2 w = *reinterpret_cast<const uint2*>(q + idx * 8);
     float f[8];
+    e4m3x4_to_f32(w.x, f);
+    e4m3x4_to_f32(w.y, f + 4);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        f[j] = e4m3_to_f32((w.x >> (8 * j)) & 0xFFu) * sc;
-        f[4 + j] = e4m3_to_f32((w.y >> (8 * j)) & 0xFFu) * sc;
-    }
+    for (int j = 0; j < 8; ++j) f[j] *= sc;
     uint4 o;
     o.x = pack_bf16(f[0], f[1]); o.y = pack_bf16(f[2], f[3]); o.z = pack_bf16(f[4], f[5]); o.w = pack_bf16(f[6], f[7]);
     *reinterpret_cast<uint4*>(out + idx * 8) = o;
@@ -576,10 +575,12 @@ __global__ __launch_bounds__(256) void k_block_dequant(const uint8_t* __restrict
     const bool one_scale = cb0 == cb1;
     const float s0 = load_block_scale(s, fmt, srow + cb0);
 #pragma unroll
+    for (int i = 0; i < 4; ++i) e4m3x4_to_f32(w[i], f + 4 * i);
+#pragma unroll
     for (int i = 0; i < 16; ++i) {
         float sc = s0;
         if (!one_scale && i < n) sc = load_block_scale(s, fmt, srow + (c0 + i) / (IDX)bc);
-        f[i] = e4m3_to_f32((w[i >> 2] >> (8 * (i & 3))) & 0xFFu) * sc;
+        f[i] *= sc;
     }
     if (OUT_F32) {
         float* op = reinterpret_cast<float*>(out) + (int64_t)row * C + c0;
