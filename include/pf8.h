@@ -203,12 +203,13 @@ int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_lay
  * format quantization/checkpoint_dequant.py:121-131).  Both operands must have been quantized with
  * pow2 scales (using_pow2_scale=True).  sa u8 [K/128, ldsa] (1x128 scales, K-block major, ldsa >= M
  * and a multiple of 8, base 8-byte aligned); sb u8 [N/128, K/128] ([E, N/128, K/128] grouped).
- * M (Mtot) multiple of 128, N multiple of 256, K multiple of 128 and >= 384, ldo multiple
+ * M (Mtot) multiple of 128, N multiple of 128 and >= 256, K multiple of 128 and >= 384, ldo multiple
  * of 8; other shapes return PF8_EINVAL (decode the scales and use the fp32-scale entry points).
  * items: the list pf8_grouped_items_build made for this m_indices (two 128-row blocks of one expert
- * per 256-row work item); with it the call also weighs the expert load and hands a GEMM whose
- * experts are too small for 256-row tiles to the 128-row-tile kernel.  NULL makes the call walk
- * aligned 256-row tiles and visit those that hold two experts twice. */
+ * per 256-row work item); with it the call also weighs the expert load and, when N is a multiple of
+ * 256, hands a GEMM whose experts are too small for 256-row tiles to the 128-row-tile kernel (with
+ * N = 256 t + 128 the paired tiles always run; the last column tile is then half empty).  NULL makes
+ * the call walk aligned 256-row tiles and visit those that hold two experts twice. */
 int pf8_gemm_nt_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b,
                       const uint8_t* sb, int64_t M, int64_t N, int64_t K, uint16_t* out, int64_t ldo,
                       pf8_stream_t stream);

@@ -45,6 +45,7 @@ struct E8Args {
     const int32_t* m_indices;
     const int32_t* items;   // grouped: {n, blocks, -, -} then {block0, block1 or -1, expert, -} per item; may be null
     int cus;
+    int force;              // with items: run them here whatever the list's header says
 };
 
 __device__ __forceinline__ int e8_keyp(int row) { return (row & 7) ^ ((row >> 3) & 1); }
@@ -91,13 +92,15 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     constexpr int BAR = 44, CSTEP = 2;     // barrier position; MFMAs between two copies
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     asm volatile("" ::: "a255");
-    if (a.items && !e8_paired_tiles_win(a.items, a.Prows / 256, a.cus)) return;   // left to the 128-row-tile kernel
+    if (a.items && !a.force && !e8_paired_tiles_win(a.items, a.Prows / 256, a.cus)) return;   // left to the 128-row-tile kernel
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wq = wave >> 1, wp = wave & 1;
     const int li = lane & 15, kg = lane >> 4;
 
-    const int64_t p_tiles = a.Prows / 256, q_tiles = a.items ? (int64_t)__builtin_amdgcn_readfirstlane(a.items[0]) : (a.Qrows + 255) / 256;
+    // Prows = 256 t + 128: the last column tile has one 128-row half; its second half re-reads the first
+    // (as a missing Q half does) and the wavefronts that own it store nothing
+    const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = a.items ? (int64_t)__builtin_amdgcn_readfirstlane(a.items[0]) : (a.Qrows + 255) / 256;
     const int64_t T = p_tiles * q_tiles;
     // consecutive workgroups go round-robin to the 8 XCDs: every XCD owns a contiguous run of
     // logical tiles (groups of 8 q-tiles x all p-tiles), walked W tiles at a time by its W workgroups
@@ -125,39 +128,42 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
         else { e = e0; mask = 1; second_e = e1; }
     };
     auto has_tail = [&](int64_t qt) -> bool { return qt * 256 + 128 >= a.Qrows; };
+    auto p_tail = [&](int64_t pt) -> bool { return pt * 256 + 128 >= a.Prows; };
 
     // work item = (tile, expert, halves to store); c_* current, n_* next; all wave-uniform
     int64_t cq = 0, cp = 0, nq = 0, np = 0, tn = 0;
     if (!tile_coords(0, cq, cp)) return;
     int c_mask, c_second = -1, n_mask = 0, n_second = -1;
     int64_t c_orow, n_orow = 0;                 // first output row of this wavefront's half
-    const uint8_t *c_ptile, *c_qtile, *c_qtile2, *c_sq, *c_sp;
+    const uint8_t *c_ptile, *c_ptile2, *c_qtile, *c_qtile2, *c_sq, *c_sp;
     // aligned tile qt of expert e
-    auto setup = [&](int64_t qt, int64_t pt, int e, const uint8_t*& ptile, const uint8_t*& qtile, const uint8_t*& qtile2,
+    auto setup = [&](int64_t qt, int64_t pt, int e, const uint8_t*& ptile, const uint8_t*& ptile2, const uint8_t*& qtile, const uint8_t*& qtile2,
                      const uint8_t*& sq, const uint8_t*& sp, int64_t& orow) {
         const bool tail = has_tail(qt);
         ptile = a.p + ((int64_t)e * a.Prows + pt * 256) * a.red;
+        ptile2 = p_tail(pt) ? ptile : ptile + 128 * a.red;
         qtile = a.q + qt * 256 * a.red;
         qtile2 = tail ? qtile : qtile + 128 * a.red;     // a missing second half re-reads the first
         sq = a.sq8 + qt * 256 + ((wq && !tail) ? 128 : 0);
-        sp = a.sp8 + ((int64_t)e * PB + pt * 2 + wp) * KB;
+        sp = a.sp8 + ((int64_t)e * PB + pt * 2 + (p_tail(pt) ? 0 : wp)) * KB;
         orow = qt * 256 + wq * 128;
     };
     // listed item {block0, block1 or -1, expert}
-    auto setup_item = [&](i32x4 it, int64_t pt, int& mask, const uint8_t*& ptile, const uint8_t*& qtile, const uint8_t*& qtile2,
+    auto setup_item = [&](i32x4 it, int64_t pt, int& mask, const uint8_t*& ptile, const uint8_t*& ptile2, const uint8_t*& qtile, const uint8_t*& qtile2,
                           const uint8_t*& sq, const uint8_t*& sp, int64_t& orow) {
         const int64_t b0 = it.x, b1 = it.y < 0 ? it.x : it.y;
         mask = it.y < 0 ? 1 : 3;
         ptile = a.p + ((int64_t)it.z * a.Prows + pt * 256) * a.red;
+        ptile2 = p_tail(pt) ? ptile : ptile + 128 * a.red;
         qtile = a.q + b0 * 128 * a.red;
         qtile2 = a.q + b1 * 128 * a.red;
         sq = a.sq8 + (wq ? b1 : b0) * 128;
-        sp = a.sp8 + ((int64_t)it.z * PB + pt * 2 + wp) * KB;
+        sp = a.sp8 + ((int64_t)it.z * PB + pt * 2 + (p_tail(pt) ? 0 : wp)) * KB;
         orow = (wq ? b1 : b0) * 128;
     };
     if (a.items) {
         const int32_t* ip = a.items + 4 + 4 * cq;
-        setup_item((i32x4){__builtin_amdgcn_readfirstlane(ip[0]), __builtin_amdgcn_readfirstlane(ip[1]), __builtin_amdgcn_readfirstlane(ip[2]), 0}, cp, c_mask, c_ptile, c_qtile, c_qtile2, c_sq, c_sp, c_orow);
+        setup_item((i32x4){__builtin_amdgcn_readfirstlane(ip[0]), __builtin_amdgcn_readfirstlane(ip[1]), __builtin_amdgcn_readfirstlane(ip[2]), 0}, cp, c_mask, c_ptile, c_ptile2, c_qtile, c_qtile2, c_sq, c_sp, c_orow);
     } else {
         int e0 = 0, e1 = has_tail(cq) ? -1 : 0, c_e;
         if (a.grouped) {
@@ -165,11 +171,11 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
             if (!has_tail(cq)) e1 = __builtin_amdgcn_readfirstlane(a.m_indices[cq * 256 + 128]);
         }
         classify(e0, e1, c_e, c_mask, c_second);
-        setup(cq, cp, c_e, c_ptile, c_qtile, c_qtile2, c_sq, c_sp, c_orow);
+        setup(cq, cp, c_e, c_ptile, c_ptile2, c_qtile, c_qtile2, c_sq, c_sp, c_orow);
     }
     int ld_e0 = 0, ld_e1 = 0;      // expert ids of the next tile's halves
     i32x4 ld_item = {0, 0, 0, 0};  // or its list entry
-    const uint8_t *n_ptile = c_ptile, *n_qtile = c_qtile, *n_qtile2 = c_qtile2, *n_sq = c_sq, *n_sp = c_sp;
+    const uint8_t *n_ptile = c_ptile, *n_ptile2 = c_ptile2, *n_qtile = c_qtile, *n_qtile2 = c_qtile2, *n_sq = c_sq, *n_sp = c_sp;
     bool n_valid = false;
 
     // copy c of a wavefront fills rows (4 c + wave) * 8 + (lane >> 3) of the stacked [P; Q] block.  P rows
@@ -192,9 +198,10 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     uint32_t zero_off = 0;
     asm volatile("" : "+v"(zero_off));     // a VGPR holding 0 (the address form needs one)
 
-#define E8_COPY(c_, pt_, qt_, qt2_, slot_)                                                             \
+#define E8_COPY(c_, pt_, pt2_, qt_, qt2_, slot_)                                                       \
     do {                                                                                               \
-        if ((c_) < 8) e8_dma16(c_off_p, (pt_) + (c_) * copy_step, lds_base + (slot_) * SLOT + ((c_) * 4 + wave) * 1024); \
+        if ((c_) < 4) e8_dma16(c_off_p, (pt_) + (c_) * copy_step, lds_base + (slot_) * SLOT + ((c_) * 4 + wave) * 1024); \
+        else if ((c_) < 8) e8_dma16(c_off_p, (pt2_) + ((c_) - 4) * copy_step, lds_base + (slot_) * SLOT + ((c_) * 4 + wave) * 1024); \
         else if ((c_) < 12) e8_dma16(c_off_q[(c_) & 3], (qt_) + ((c_) - 8) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
         else e8_dma16(c_off_q[(c_) & 3], (qt2_) + ((c_) - 12) * copy_step, lds_base + (slot_) * SLOT + Q_OFS + (((c_) - 8) * 4 + wave) * 1024); \
     } while (0)
@@ -216,10 +223,10 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
     {
         E8_LOAD_S(c_sq, c_sp);
 #pragma unroll
-        for (int c = 0; c < 16; ++c) E8_COPY(c, c_ptile, c_qtile, c_qtile2, 0);
+        for (int c = 0; c < 16; ++c) E8_COPY(c, c_ptile, c_ptile2, c_qtile, c_qtile2, 0);
 #pragma unroll
         for (int c = 0; c < 16; ++c)
-            if (c * CSTEP < 64 - BAR) E8_COPY(c, c_ptile + 128, c_qtile + 128, c_qtile2 + 128, 1);
+            if (c * CSTEP < 64 - BAR) E8_COPY(c, c_ptile + 128, c_ptile2 + 128, c_qtile + 128, c_qtile2 + 128, 1);
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(sq_nxt), "+v"(sp_nxt) : : "memory");
         __syncthreads();
 #pragma unroll
@@ -250,17 +257,17 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
         if (kb == 1) {
             if (c_second >= 0) {
                 nq = cq; np = cp; n_mask = 2; n_second = -1;
-                setup(nq, np, c_second, n_ptile, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
+                setup(nq, np, c_second, n_ptile, n_ptile2, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
             } else if (n_valid && a.items) {
-                setup_item(ld_item, np, n_mask, n_ptile, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
+                setup_item(ld_item, np, n_mask, n_ptile, n_ptile2, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
             } else if (n_valid) {
                 const int e0 = a.grouped ? ld_e0 : 0, e1 = has_tail(nq) ? -1 : (a.grouped ? ld_e1 : 0);
                 int ne;
                 classify(e0, e1, ne, n_mask, n_second);
-                setup(nq, np, ne, n_ptile, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
+                setup(nq, np, ne, n_ptile, n_ptile2, n_qtile, n_qtile2, n_sq, n_sp, n_orow);
             } else {
                 // past the last item the copies and scale loads re-read this item's first blocks
-                n_ptile = c_ptile; n_qtile = c_qtile; n_qtile2 = c_qtile2; n_sq = c_sq; n_sp = c_sp;
+                n_ptile = c_ptile; n_ptile2 = c_ptile2; n_qtile = c_qtile; n_qtile2 = c_qtile2; n_sq = c_sq; n_sp = c_sp;
             }
         }
         const u32x2 sq_cur = sq_nxt;
@@ -270,9 +277,11 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
         const uint8_t* s_sq = in1 ? c_sq + (kb + 1) * a.ldsq : n_sq;
         const uint8_t* s_sp = in1 ? c_sp + (kb + 1) : n_sp;
         const uint8_t* cp1_p = (in1 ? c_ptile : n_ptile) + o1;
+        const uint8_t* cp1_p2 = (in1 ? c_ptile2 : n_ptile2) + o1;
         const uint8_t* cp1_q = (in1 ? c_qtile : n_qtile) + o1;
         const uint8_t* cp1_q2 = (in1 ? c_qtile2 : n_qtile2) + o1;
         const uint8_t* cp2_p = (in2 ? c_ptile : n_ptile) + o2;
+        const uint8_t* cp2_p2 = (in2 ? c_ptile2 : n_ptile2) + o2;
         const uint8_t* cp2_q = (in2 ? c_qtile : n_qtile) + o2;
         const uint8_t* cp2_q2 = (in2 ? c_qtile2 : n_qtile2) + o2;
         E8_LOAD_S(s_sq, s_sp);
@@ -298,11 +307,11 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
             // copies: the block after next into the slot this block has just left, continued in the
             // next block before its barrier
             if constexpr (m >= BAR && (m - BAR) % CSTEP == 0 && (m - BAR) / CSTEP < 16) {
-                E8_COPY((m - BAR) / CSTEP, cp2_p, cp2_q, cp2_q2, PAR);
+                E8_COPY((m - BAR) / CSTEP, cp2_p, cp2_p2, cp2_q, cp2_q2, PAR);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (m < BAR && (m + 64 - BAR) % CSTEP == 0 && (m + 64 - BAR) / CSTEP < 16) {
-                E8_COPY((m + 64 - BAR) / CSTEP, cp1_p, cp1_q, cp1_q2, PAR ^ 1);
+                E8_COPY((m + 64 - BAR) / CSTEP, cp1_p, cp1_p2, cp1_q, cp1_q2, PAR ^ 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // the next block's P fragments and first Q fragments, from the slot just declared landed
@@ -321,7 +330,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
 
         // ---- item finished: the wavefronts whose half is stored write it out through a private LDS
         // slice, one Q fragment (16 rows x 128 columns) at a time, as whole 256-byte rows
-        if ((c_mask >> wq) & 1) {
+        if (((c_mask >> wq) & 1) && !(wp && p_tail(cp))) {
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written back before they are read
             uint8_t* ep = lds + EP_OFS + wave * (16 * EP_LD);
             const int er = lane >> 4, ec = lane & 15;
@@ -351,7 +360,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
         e8_static_for<64>([&](auto ix) { e8_acc_zero4<decltype(ix)::value>(); });
         if (c_second < 0) ++tn;
         cq = nq; cp = np; c_mask = n_mask; c_second = n_second; c_orow = n_orow;
-        c_ptile = n_ptile; c_qtile = n_qtile; c_qtile2 = n_qtile2; c_sq = n_sq; c_sp = n_sp;
+        c_ptile = n_ptile; c_ptile2 = n_ptile2; c_qtile = n_qtile; c_qtile2 = n_qtile2; c_sq = n_sq; c_sp = n_sp;
         kb = 0;
         return false;
     };
@@ -462,7 +471,7 @@ static int launch_e8(const E8Args& a, int64_t max_q_tiles, hipStream_t st, const
         if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, where, hipGetErrorString(e));
         attr_done = 1;
     }
-    const int64_t T = (a.Prows / 256) * max_q_tiles, per_xcd = (T + 7) / 8;
+    const int64_t T = ((a.Prows + 255) / 256) * max_q_tiles, per_xcd = (T + 7) / 8;
     int64_t w = pf8_effective_cus() / 8;
     if (w < 1) w = 1;
     if (w > per_xcd) w = per_xcd;
@@ -472,7 +481,7 @@ static int launch_e8(const E8Args& a, int64_t max_q_tiles, hipStream_t st, const
 
 static int check_e8_shapes(const char* where, int64_t M, int64_t N, int64_t K, int64_t ldsa) {
     if (M % 128 != 0) return pf8_fail(PF8_EINVAL, where, "M must be a multiple of 128");
-    if (N % 256 != 0) return pf8_fail(PF8_EINVAL, where, "N must be a multiple of 256");
+    if (N % 128 != 0 || (N != 0 && N < 256)) return pf8_fail(PF8_EINVAL, where, "N must be a multiple of 128 and at least 256");
     if (K % 128 != 0 || K < 384) return pf8_fail(PF8_EINVAL, where, "K must be a multiple of 128 and at least 384");
     if (ldsa < M || ldsa % 8 != 0) return pf8_fail(PF8_EINVAL, where, "ldsa must be >= M and a multiple of 8");
     if (K > (1ll << 24)) return pf8_fail(PF8_EINVAL, where, "K too large");
@@ -517,8 +526,9 @@ extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint
         PF8_REQUIRE((reinterpret_cast<uintptr_t>(items) & 15u) == 0, "items must be 16-byte aligned");
         g.items = items;
         g.cus = pf8_effective_cus();
+        g.force = N % 256 != 0;      // the 128x256-tile kernel takes whole 256-column tiles only
         rc = launch_e8(g, Mtot / 128, (hipStream_t)stream, __func__);
-        if (rc) return rc;
+        if (rc || g.force) return rc;
         return pf8_launch_deep_ue8m0(b, a, sb, sa, ldsa, out, N, Mtot, K, E, m_indices, items, (hipStream_t)stream, __func__);
     }
     return launch_e8(g, (Mtot + 255) / 256, (hipStream_t)stream, __func__);

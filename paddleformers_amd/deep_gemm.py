@@ -59,8 +59,20 @@ def _decode_ue8m0(s: torch.Tensor) -> torch.Tensor:
     return torch.exp2(s.view(torch.uint8).to(torch.float32) - 127.0)
 
 
-def _ue8m0_kernel_shape(M: int, N: int, K: int) -> bool:
-    return M % 128 == 0 and N % 256 == 0 and K % 128 == 0 and K >= 384
+def _ue8m0_kernel_shape(M: int, N: int, K: int, experts: int = 0) -> bool:
+    """Shapes the block-scaled MFMA kernel takes: 256-column tiles, the last one may be a 128-column half.
+    A grouped launch with such a half tile cannot fall back to the 128-row-tile kernel on the device
+    (that kernel wants whole 256-column tiles), so the choice the list header would make there is made
+    here from an upper bound of the number of paired tiles (every expert with an odd block)."""
+    if not (M % 128 == 0 and N % 128 == 0 and N >= 256 and K % 128 == 0 and K >= 384):
+        return False
+    if experts and N % 256 != 0:
+        cus = get_num_sms() or 256
+        p_tiles = (N + 255) // 256
+        rounds_pair = -(-(M // 256 + experts) * p_tiles // cus)
+        rounds_128 = -(-(M // 128) * p_tiles // cus)
+        return 16 * rounds_pair <= 10 * rounds_128
+    return True
 
 
 def fp8_gemm_nt(a, b, out: torch.Tensor, c: Optional[torch.Tensor] = None, recipe=None, compiled_dims: str = "nk"):
@@ -169,7 +181,7 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
     if _is_ue8m0(sa):
         if tuple(sb.shape) != (E, (N + 127) // 128, K // 128):
             raise ValueError(f"b scale must be [{E}, {(N + 127) // 128}, {K // 128}]")
-        if _ue8m0_kernel_shape(Mtot, N, K):
+        if _ue8m0_kernel_shape(Mtot, N, K, E):
             sa_k = _ue8m0_kmajor(sa, Mtot, K // 128, "a scale")
             sb_k = sb.view(torch.uint8).contiguous()
             if items is None:

@@ -86,8 +86,9 @@ def test_scales_to_ue8m0_matches_oracle_and_rejects_other_scales():
         F.scales_to_ue8m0(torch.tensor([1.0, 0.0, -2.0], device="cuda"))
 
 
-# 384 and 640 rows end in a half tile; 128 is a lone half tile
-@pytest.mark.parametrize("M,N,K", [(256, 256, 384), (512, 768, 1024), (384, 512, 512), (128, 256, 640), (640, 1024, 896)])
+# 384 and 640 rows end in a half tile; 128 is a lone half tile; 384, 640 and 1408 columns end in a half tile
+@pytest.mark.parametrize("M,N,K", [(256, 256, 384), (512, 768, 1024), (384, 512, 512), (128, 256, 640), (640, 1024, 896),
+                                   (256, 384, 512), (384, 640, 640), (512, 1408, 384)])
 @pytest.mark.parametrize("kmajor", [False, True])
 def test_gemm_nt_ue8m0_vs_oracle(dg, M, N, K, kmajor):
     a, sa, b, sb = _pow2_case(M, N, K, seed=M + N + K)
@@ -97,11 +98,12 @@ def test_gemm_nt_ue8m0_vs_oracle(dg, M, N, K, kmajor):
     _check(G.from_torch_bf16(out), a, sa, b, sb, f"ue8m0 gemm {M}x{N}x{K}")
 
 
-def test_gemm_nt_ue8m0_scales_are_applied_per_row_and_block(dg):
+@pytest.mark.parametrize("N", [512, 640])
+def test_gemm_nt_ue8m0_scales_are_applied_per_row_and_block(dg, N):
     """Ones times ones with a distinct exponent for every (row, K block) and (column block, K block):
     the result is sum_kb 128 * 2^(ea[m,kb] + eb[n/128,kb]) exactly -- catches a transposed, mis-selected
     (op_sel) or mis-indexed scale byte and a wrong row permutation inside a fragment."""
-    M, N, K = 512, 512, 512
+    M, K = 512, 512
     rng = np.random.default_rng(5)
     one = O.e4m3_encode_array(np.ones(1, np.float32))[0]
     a = np.full((M, K), one, np.uint8)
@@ -130,7 +132,7 @@ def test_gemm_nt_ue8m0_exact_integer_case_with_row_stride(dg):
     assert (wide[:, N:] == 5.0).all()
 
 
-@pytest.mark.parametrize("M,N,K", [(200, 384, 256), (256, 384, 512), (256, 256, 256)])
+@pytest.mark.parametrize("M,N,K", [(200, 384, 256), (256, 128, 512), (256, 256, 256)])
 def test_gemm_nt_ue8m0_other_shapes_take_the_decoded_scale_kernel(dg, M, N, K):
     """Shapes outside the block-scaled kernel's tiling give the same result through the fp32-scale kernel."""
     a, sa, b, sb = _pow2_case(M, N, K, seed=7)
@@ -201,6 +203,38 @@ def test_grouped_contiguous_ue8m0_vs_oracle(dg, request, rows, paired, cus):
     Mtot = a.shape[0]
     out = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     _grouped_call(dg, a, sa, b, sb, m_idx, out, paired)
+    exp = O.grouped_gemm_nt_contiguous(a, sa, b, sb, m_idx)
+    got = G.from_torch_bf16(out)
+    assert G.rel_fro(_bf(got), _bf(exp)) <= BLOCK_FRO
+    start = 0
+    for e, r in enumerate(rows):
+        if r:
+            _elementwise_ok(_bf(got[start:start + r]), a[start:start + r], sa[start:start + r], b[e], sb[e], f"expert {e}")
+        start += r
+
+
+# 640 = two column tiles and a half: the wavefronts of the missing half compute on a copy of the first and
+# store nothing.  Through the raw C ABI, so that the block-scaled kernel runs whatever the load: with a
+# work-item list (paired 256-row tiles) and without (aligned tiles, two passes where experts meet).
+@pytest.mark.parametrize("rows", [[128, 256, 0, 128], [384, 128, 640, 128], [256, 512]])
+@pytest.mark.parametrize("with_items", [True, False])
+@pytest.mark.parametrize("cus", ["all", "few"])
+def test_grouped_contiguous_ue8m0_half_column_tile(dg, request, rows, with_items, cus):
+    from paddleformers_amd import _lib
+
+    if cus == "few":
+        request.getfixturevalue("few_cus")
+    E, N, K = len(rows), 640, 512
+    a, sa, b, sb, m_idx = _grouped_pow2_case(E, N, K, rows, seed=sum(rows) + 3 * E)
+    Mtot = a.shape[0]
+    out = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ta, tb, tm = G.to_torch_fp8(a), G.to_torch_fp8(b), torch.from_numpy(m_idx).cuda()
+    tsa, tsb = _e8(np.ascontiguousarray(sa.T)), _e8(sb)
+    items = dg.build_group_items(tm) if with_items else None
+    _lib.call("pf8_grouped_gemm_nt_contiguous_ue8m0", ta.data_ptr(), tsa.data_ptr(), tsa.stride(0), tb.data_ptr(), tsb.data_ptr(),
+              E, Mtot, N, K, tm.data_ptr(), items.data_ptr() if with_items else None, out.data_ptr(),
+              torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
     exp = O.grouped_gemm_nt_contiguous(a, sa, b, sb, m_idx)
     got = G.from_torch_bf16(out)
     assert G.rel_fro(_bf(got), _bf(exp)) <= BLOCK_FRO
@@ -325,14 +359,18 @@ def test_ue8m0_gemms_at_config3_size_agree_with_the_fp32_scale_kernels(dg):
     assert torch.equal(one.view(torch.int16), out[sl].view(torch.int16))
 
 
-def test_ue8m0_grouped_gemm_at_config5_size_agrees_with_the_fp32_scale_kernel(dg):
+# N = 2816: the up+gate GEMM; N = 1408 (five column tiles and a half): the dgrad GEMM of the down projection
+@pytest.mark.parametrize("N", [2816, 1408])
+def test_ue8m0_grouped_gemm_at_config5_size_agrees_with_the_fp32_scale_kernel(dg, N):
     """128 experts with a Zipf(1.0) load over 131072 routed rows (segments of 2..190 blocks, 1083 blocks in
     all): here the cost estimate picks the paired 256-row tiles on the whole device, and the list builder
     walks two blocks per thread."""
     from bench import zipf_counts
+    from paddleformers_amd import deep_gemm as DG
     from paddleformers_amd import functional as F
 
-    E, H, N = 128, 4096, 2816
+    E, H = 128, 4096
+    assert DG._ue8m0_kernel_shape(138624, N, H, E)
     _, padded = zipf_counts(131072, E, 1.0, seed=5, n_empty=0)
     rows = [int(r) for r in padded]
     Mtot = sum(rows)
