@@ -267,6 +267,43 @@ def bench_other_gemms(iters=10, warmup=3):
     out["rms_norm_bwd_16384x7168"] = {"bytes": Mn * Hn * 6 + Mn * 4 + Hn * 4, "ms": ms}
     del xn, dn, ivn
     torch.cuda.empty_cache()
+    # dequantizers on a [16384, 7168] activation / a [7168, 4096] weight
+    qa = rnd8(Mn, Hn)
+    sa_d = torch.rand((Hn // 128, Mn), device="cuda")
+    ms = time_kernel(lambda: F8.fused_act_dequant(qa, sa_d.T), [()], 5, 2)
+    out["act_dequant_16384x7168"] = {"bytes": Mn * Hn * 3 + Mn * (Hn // 128) * 4, "ms": ms}
+    qw2, sw2 = rnd8(Hn, 4096), torch.rand((Hn // 128, 4096 // 128), device="cuda")
+    ms = time_kernel(lambda: F8.weight_dequant(qw2, sw2), [()], 5, 2)
+    out["weight_dequant_7168x4096"] = {"bytes": Hn * 4096 * 3 + sw2.numel() * 4, "ms": ms}
+    del qa, sa_d, qw2, sw2
+    # SwiGLU backward of the MoE node at config 5: o1 [Mp, 2I], do2_s [Mp, I] -> do1, o2_s, probs_grad
+    o1b = torch.randn((Mp, 2 * I), device="cuda").to(torch.bfloat16)
+    d2b = (torch.randn((Mp, I), device="cuda") * 1e-3).to(torch.bfloat16)
+    prb = torch.rand((Mp, 1), device="cuda")
+    ms = time_kernel(lambda: F8.fused_swiglu_weighted_bwd(o1b, d2b, prb), [()], 5, 2)
+    out["swiglu_bwd_config5"] = {"bytes": Mp * I * 12 + Mp * 8, "ms": ms}
+    del o1b, d2b, prb
+    # dense weight gradient of config 2: dW [7168, 4096] = x^T [7168, 8192] . dy^T [4096, 8192]^T, fp32 out
+    Mw, Kw, Nw = 8192, 7168, 4096
+    xt_q, dyt_q = rnd8(Kw, Mw), rnd8(Nw, Mw)
+    sxt = torch.exp2(torch.randint(-3, 3, (Mw // 128, Kw), device="cuda").float())
+    sdy = torch.exp2(torch.randint(-3, 3, (Mw // 128, Nw), device="cuda").float())
+    dwd = torch.zeros((Kw, Nw), dtype=torch.float32, device="cuda")
+    ms = time_kernel(lambda: F8.fp8_gemm_blockwise(xt_q, sxt, dyt_q, sdy, out=dwd, accumulate=True), [()], iters, warmup)
+    out["wgrad_dense_config2"] = {"flop": 2.0 * Mw * Kw * Nw, "ms": ms}
+    ms = time_kernel(lambda: F8.fp8_gemm_blockwise(xt_q, sxt, dyt_q, sdy, out=dwd, accumulate=True, scales_pow2=True), [()], iters, warmup)
+    out["wgrad_dense_config2_pow2"] = {"flop": 2.0 * Mw * Kw * Nw, "ms": ms}
+    del xt_q, dyt_q, sxt, sdy, dwd
+    # masked grouped GEMM (fixed capacity per expert): 32 experts x 512 rows, 256..512 of them valid
+    Em, Cm, Km, Nm = 32, 512, 7168, 4096
+    am, bm = rnd8(Em, Cm, Km), rnd8(Em, Nm, Km)
+    sam, sbm = torch.rand((Em, Cm, Km // 128), device="cuda"), torch.rand((Em, Nm // 128, Km // 128), device="cuda")
+    mm = torch.from_numpy(np.random.default_rng(7).integers(256, Cm + 1, Em).astype(np.int32)).cuda()
+    om = torch.empty((Em, Cm, Nm), dtype=torch.bfloat16, device="cuda")
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_masked((am, sam), (bm, sbm), om, mm, Cm), [()], iters, warmup)
+    out["grouped_masked_32x512"] = {"flop": 2.0 * float(mm.sum().item()) * Km * Nm, "ms": ms}
+    del am, bm, sam, sbm, om
+    torch.cuda.empty_cache()
     # the fused FP8 MoE node end to end at config 5: forward + backward (dgrad and wgrad, both GEMMs),
     # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers
     from paddleformers_amd import fp8_utils as U8

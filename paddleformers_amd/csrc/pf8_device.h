@@ -232,17 +232,6 @@ __device__ __forceinline__ void unpack8(uint4 w, float (&v)[8]) {
     v[6] = bf16_lo(w.w); v[7] = bf16_hi(w.w);
 }
 
-// e4m3 code -> fp32 (exact).  Subnormals and the NaN code handled explicitly.
-__device__ __forceinline__ float e4m3_to_f32(uint32_t c) {
-    uint32_t mag = c & 0x7Fu;
-    uint32_t sign = (c & 0x80u) << 24;
-    float v;
-    if (mag >= 8u) v = u2f((mag << 20) + 0x3C000000u);          // (e - 7 + 127) << 23 | m << 20
-    else v = (float)mag * 0.001953125f;                        // m * 2^-9
-    if (mag == 0x7Fu) v = u2f(0x7FC00000u);
-    return u2f(f2u(v) | sign);
-}
-
 // four e4m3 codes of one word -> fp32 with the hardware convert (exact, two bytes per instruction)
 __device__ __forceinline__ void e4m3x4_to_f32(uint32_t w, float* f) {
     const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);

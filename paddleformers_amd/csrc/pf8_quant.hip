@@ -519,16 +519,6 @@ __global__ __launch_bounds__(256) void k_act_dequant(const uint8_t* __restrict__
     *reinterpret_cast<uint4*>(out + idx * 8) = o;
 }
 
-// 128x128 dequant, arbitrary R and C: one thread per element (checkpoint-load path, not hot)
-__global__ __launch_bounds__(256) void k_weight_dequant(const uint8_t* __restrict__ q, const float* __restrict__ s, int64_t R,
-                                                        int64_t C, uint16_t* __restrict__ out) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= R * C) return;
-    const int64_t r = idx / C, c = idx % C, CB = (C + 127) / 128;
-    float f = e4m3_to_f32(q[idx]) * s[(r / 128) * CB + c / 128];
-    out[idx] = (uint16_t)(pack_bf16(f, 0.0f) & 0xFFFFu);
-}
-
 // ---------------------------------------------------------------------------------------------
 // Block-FP8 checkpoint dequantization: out = cast(e4m3(q) * scale(block)), any block geometry on the
 // last two axes, partial trailing blocks cropped, scales as UE8M0 exponent bytes or fp32/bf16/fp16.
@@ -853,16 +843,6 @@ extern "C" int pf8_act_dequant(const uint8_t* q, const float* s, int scale_layou
     return pf8_check_launch(__func__);
 }
 
-extern "C" int pf8_weight_dequant(const uint8_t* q, const float* s, int64_t R, int64_t C, uint16_t* out, pf8_stream_t stream) {
-    PF8_REQUIRE(R >= 0 && C >= 0, "negative shape");
-    if (R == 0 || C == 0) return PF8_OK;
-    PF8_REQUIRE(q && s && out, "null pointer");
-    const int64_t n = R * C;
-    dim3 grid((unsigned)((n + 255) / 256)), block(256);
-    hipLaunchKernelGGL(k_weight_dequant, grid, block, 0, (hipStream_t)stream, q, s, R, C, out);
-    return pf8_check_launch(__func__);
-}
-
 extern "C" int pf8_block_dequant(const uint8_t* q, const void* scale, int scale_format, int64_t B, int64_t R, int64_t C,
                                  int64_t block_r, int64_t block_c, void* out, int out_f32, pf8_stream_t stream) {
     PF8_REQUIRE(B >= 0 && R >= 0 && C >= 0, "negative shape");
@@ -881,6 +861,14 @@ extern "C" int pf8_block_dequant(const uint8_t* q, const void* scale, int scale_
     else if (small) hipLaunchKernelGGL((k_block_dequant<0, uint32_t>), grid, block, 0, st, q, scale, scale_format, B, R, C, block_r, block_c, out);
     else hipLaunchKernelGGL((k_block_dequant<0, int64_t>), grid, block, 0, st, q, scale, scale_format, B, R, C, block_r, block_c, out);
     return pf8_check_launch(__func__);
+}
+
+// 128x128-block dequant to bf16: the block dequantizer with fp32 scales and one 128x128 geometry
+extern "C" int pf8_weight_dequant(const uint8_t* q, const float* s, int64_t R, int64_t C, uint16_t* out, pf8_stream_t stream) {
+    PF8_REQUIRE(R >= 0 && C >= 0, "negative shape");
+    if (R == 0 || C == 0) return PF8_OK;
+    PF8_REQUIRE(q && s && out, "null pointer");
+    return pf8_block_dequant(q, s, SCALE_F32, 1, R, C, 128, 128, out, 0, stream);
 }
 
 extern "C" int pf8_debug_copy(const void* src, void* dst, int64_t nbytes, pf8_stream_t stream) {
