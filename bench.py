@@ -304,6 +304,55 @@ def bench_other_gemms(iters=10, warmup=3):
     out["grouped_masked_32x512"] = {"flop": 2.0 * float(mm.sum().item()) * Km * Nm, "ms": ms}
     del am, bm, sam, sbm, om
     torch.cuda.empty_cache()
+    # the masked-layout expert node (fixed capacity per expert) end to end: 32 experts x 512 rows, 256..512 valid
+    from paddleformers_amd import ernie_fp8_utils as EU
+
+    class _Lin:
+        def __init__(self, w):
+            self.weight = w
+
+    class _ExM:
+        pass
+
+    class _CfgM:
+        fp8_fused_ops_configs = {"stack_quant": True, "swiglu_probs_bwd": True}
+
+    class _MpM:
+        pass
+
+    Hm, Im = 4096, 1408
+    gm1 = torch.zeros((Em, Hm, 2 * Im), dtype=torch.float32, device="cuda")
+    gm2 = torch.zeros((Em, Im, Hm), dtype=torch.float32, device="cuda")
+    exm = []
+    for e in range(Em):
+        ex = _ExM()
+        ex.up_gate_proj = _Lin((torch.randn((Hm, 2 * Im), device="cuda") * 0.02).to(torch.bfloat16))
+        ex.down_proj = _Lin((torch.randn((Im, Hm), device="cuda") * 0.02).to(torch.bfloat16))
+        ex.up_gate_proj.weight.main_grad, ex.down_proj.weight.main_grad = gm1[e], gm2[e]
+        exm.append(ex)
+    # the per-step weight quantization is cached on the first weight of each list, as the node expects it
+    for ws_m in ([ex.up_gate_proj.weight for ex in exm], [ex.down_proj.weight for ex in exm]):
+        qn, sn = F8.fused_stack_transpose_quant(ws_m, False)
+        qt, st_ = F8.fused_stack_transpose_quant(ws_m, True)
+        ws_m[0].fp8_weight_stacked, ws_m[0].fp8_scale_stacked = qn, sn
+        ws_m[0].fp8_weight_stacked_transpose, ws_m[0].fp8_scale_stacked_transpose = qt, st_
+    mpm = _MpM()
+    mpm.experts, mpm.config = exm, _CfgM()
+    nodem = EU.ExpertsGroupGemmNode(exm, mpm)
+    xm = torch.randn((Em * Cm, Hm), device="cuda").to(torch.bfloat16)
+    dm = (torch.randn((Em, Cm, Hm), device="cuda") * 1e-3).to(torch.bfloat16)
+    prm = torch.rand((Em * Cm,), device="cuda")
+
+    def fwd_bwd_masked():
+        nodem.forward(xm, prm, mm)
+        nodem.backward(dm, mm, None, Cm)
+
+    ms = time_kernel(fwd_bwd_masked, [()], 3, 2)
+    valid_rows = float(mm.sum().item())
+    out["ernie_masked_node_32x512_fwd_bwd"] = {"flop": 2 * (2.0 * valid_rows * Hm * 2 * Im + 2.0 * valid_rows * Im * Hm)
+                                               + (2.0 * Em * Cm * Hm * 2 * Im + 2.0 * Em * Cm * Im * Hm), "ms": ms}
+    del exm, gm1, gm2, xm, dm, nodem
+    torch.cuda.empty_cache()
     # the fused FP8 MoE node end to end at config 5: forward + backward (dgrad and wgrad, both GEMMs),
     # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers
     from paddleformers_amd import fp8_utils as U8
