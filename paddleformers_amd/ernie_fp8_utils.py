@@ -1,5 +1,7 @@
-"""Host mirror of the ERNIE token dispatcher's masked-layout FP8 expert node
-(cli/train/ernie_pretrain/models/moe/token_dispatcher/fp8_utils.py:56-784).
+"""Host mirror of the ERNIE token dispatcher's FP8 expert nodes
+(cli/train/ernie_pretrain/models/moe/token_dispatcher/fp8_utils.py:56-1437): the masked-layout
+ExpertsGroupGemmNode and the contiguous-layout ExpertsGroupGemmContiguousNode.  (ExpertsGroupGemmWLCHNode,
+:1439-1517, lays the rows out per expert-parallel rank and is not mirrored.)
 
 Masked layout: every expert owns a fixed capacity of `Mmax` rows of the flat `[E * Mmax, H]` activation
 tensor, of which the first `tokens_per_expert[e]` are valid; the grouped GEMMs leave the other rows of
@@ -25,7 +27,7 @@ from . import deep_gemm
 from . import functional as F8
 from .fp8_utils import FP8GroupGemmMlpFunctionNode
 
-__all__ = ["ExpertsGroupGemmNode", "fused_stack_transpose_quant", "split_group_gemm", "has_config"]
+__all__ = ["ExpertsGroupGemmNode", "ExpertsGroupGemmContiguousNode", "fused_stack_transpose_quant", "split_group_gemm", "has_config"]
 
 
 def _get_fp8_weight_and_scale(weight, stacked=False, transpose=False):
@@ -281,3 +283,207 @@ class ExpertsGroupGemmNode:
         self.bwd_gate_up_weight(do1, self.unzipped_tokens, expert_w1)
         self.reset_status()
         return dx
+
+
+class ExpertsGroupGemmContiguousNode:
+    """fp8_utils.py:787-1437.  The same expert MLP on the contiguous layout: rows sorted by expert, every
+    expert's segment a multiple of 128 rows (tokens_per_expert, a list of ints).  Switches read from
+    custom_map.config.fp8_fused_ops_configs: stack_quant, split_group_gemm, spaq (fused SwiGLU + quantize
+    with power-of-two scales), swiglu_probs_bwd, transpose_split_quant (fused, power-of-two scales).
+    dequant_input keeps the quantised input instead of the bf16 one and rebuilds it for the weight
+    gradient; a2a_async_fn(dx) -> (dx, task), when given to backward, is started right after dx is ready
+    and waited for at the end."""
+
+    def __init__(self, custom_map, recompute_fwd_gate_up=False, dequant_input=False, group=None,
+                 name="experts_group_gemm_contiguous_node"):
+        self.custom_map = custom_map
+        self.recompute_fwd_gate_up = recompute_fwd_gate_up
+        self.dequant_input = dequant_input
+        self.tokens_per_expert = None
+        self.m_indices = None
+        self.unzipped_probs = None
+        self.input = None
+        self.input_fp8 = None
+        self.input_scale = None
+        self.o1 = None
+        self.fp8_fused_ops_configs = custom_map.config.fp8_fused_ops_configs
+        self.is_split_group_gemm = has_config(self.fp8_fused_ops_configs, "split_group_gemm")
+        self.group = group
+        self.name = name
+
+    def reset_status(self):
+        self.tokens_per_expert = None
+        self.m_indices = None
+        self.unzipped_probs = None
+        self.input = None
+        self.input_fp8 = None
+        self.input_scale = None
+        self.o1 = None
+
+    def gen_m_indices(self, tokens_per_expert):
+        """fp8_utils.py:854-873: expert id of every row, int32."""
+        counts = torch.tensor([int(t) for t in tokens_per_expert], dtype=torch.int64)
+        return torch.repeat_interleave(torch.arange(len(counts), dtype=torch.int32), counts).cuda()
+
+    def _stack_quant(self) -> bool:
+        return has_config(self.fp8_fused_ops_configs, "stack_quant")
+
+    def _grouped(self, a_fp8, a_scale, w_quant, w_scale, out):
+        if numpy.prod(a_fp8.shape) != 0:
+            if self.is_split_group_gemm:
+                split_group_gemm(a_fp8, a_scale, w_quant, w_scale, self.tokens_per_expert, out)
+            else:
+                deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, a_scale), (w_quant, w_scale), out, self.m_indices)
+        return out
+
+    def fwd_gate_up(self, x, expert_w1, num_expert, tokens_per_expert, scale=None):
+        """fp8_utils.py:875-947.  x: bf16 [M, H]; e4m3 with its `scale` (needs dequant_input); or None to
+        reuse the cached quantised input."""
+        self.tokens_per_expert = tokens_per_expert
+        if not self.is_split_group_gemm:
+            self.m_indices = self.gen_m_indices(tokens_per_expert)
+        w1_t_quant, w1_t_scale = _quant_weights(expert_w1, True, self._stack_quant())
+        if x is None:
+            x_fp8, x_scale = self.input_fp8, self.input_scale
+            assert x_fp8 is not None and x_scale is not None
+        elif scale is not None:
+            x_fp8, x_scale = x, scale
+            assert self.dequant_input, "If a scale is provided, it indicates that a2a is using fp8. Dequant_input must be enabled."
+        else:
+            x_fp8, x_scale = F8.fp8_quant_blockwise(x, quant_method="1x128", input_transpose=False, output_scale_transpose=True)
+            x_scale = x_scale.T
+        o1 = torch.empty((x_fp8.shape[0], w1_t_quant.shape[1]), dtype=expert_w1[0].dtype, device=x_fp8.device)
+        self._grouped(x_fp8, x_scale, w1_t_quant, w1_t_scale, o1)
+        if self.dequant_input:
+            self.input_fp8 = x_fp8
+            self.input_scale = x_scale
+        else:
+            self.input = x
+        return o1
+
+    def fwd_swiglu(self, o1):
+        return F8.swiglu(o1)
+
+    def fwd_down(self, o1, unzipped_probs, expert_w2, num_expert):
+        """fp8_utils.py:953-1017: (o3 [M, H], probs [M, 1]).  `spaq` quantizes with power-of-two scales."""
+        w2_quant, w2_scale = _quant_weights(expert_w2, True, self._stack_quant())
+        o2_fp8, o2_scale = F8.fused_weighted_swiglu_act_quant(o1, unzipped_probs,
+                                                              using_pow2_scaling=has_config(self.fp8_fused_ops_configs, "spaq"))
+        unzipped_probs = unzipped_probs.unsqueeze(-1)
+        o3 = torch.empty((o2_fp8.shape[0], w2_quant.shape[1]), dtype=o1.dtype, device=o1.device)
+        self._grouped(o2_fp8, o2_scale, w2_quant, w2_scale, o3)
+        return o3, unzipped_probs
+
+    def bwd_down_input(self, expert_w2, unzipped_grad, o1):
+        """fp8_utils.py:1019-1094: (do1 [M, 2I], o2_s [M, I], probs_grad [M])."""
+        bw_w2_quant, bw_w2_scale = _quant_weights(expert_w2, False, self._stack_quant())
+        g_fp8, g_scale = F8.fp8_quant_blockwise(unzipped_grad, quant_method="1x128", input_transpose=False, output_scale_transpose=True)
+        do2_s = torch.empty((g_fp8.shape[0], bw_w2_quant.shape[1]), dtype=unzipped_grad.dtype, device=unzipped_grad.device)
+        self._grouped(g_fp8, g_scale.T, bw_w2_quant, bw_w2_scale, do2_s)
+        do1, probs_grad, o2_s = F8.fused_swiglu_weighted_bwd(o1, do2_s, self.unzipped_probs.squeeze(-1))
+        return do1, o2_s, probs_grad
+
+    def bwd_swiglu(self, o1, do2):
+        do1, _ = F8.swiglu_grad(o1, None, do2)
+        return do1
+
+    def bwd_gate_up_input(self, do1, expert_w1):
+        """fp8_utils.py:1100-1155: dx [M, H]."""
+        bw_w1_quant, bw_w1_scale = _quant_weights(expert_w1, False, self._stack_quant())
+        do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, quant_method="1x128", input_transpose=False, output_scale_transpose=True)
+        dx = torch.empty((do1_fp8.shape[0], bw_w1_quant.shape[1]), dtype=torch.bfloat16, device=do1.device)
+        self._grouped(do1_fp8, do1_scale.T, bw_w1_quant, bw_w1_scale, dx)
+        return dx
+
+    def fused_transpose_split_quant(self, x, tokens_per_expert, pow_2_scales):
+        """fp8_utils.py:1157-1180."""
+        return F8.fused_transpose_split_quant(x, None, tokens_per_expert, pow_2_scales)
+
+    def _wgrad(self, a, b, expert_w):
+        """fp8_utils.py:1182-1319: per expert, a_e^T . b_e into main_grad (or grad).  Without the
+        `transpose_split_quant` switch the reference transposes the whole tensor, quantizes it 1x128 with
+        plain scales and splits the scales per expert: the same values as the per-expert kernel without
+        power-of-two scales, since every segment is a multiple of 128 rows."""
+        pow2 = has_config(self.fp8_fused_ops_configs, "transpose_split_quant")
+        a_t, sa_t = self.fused_transpose_split_quant(a, self.tokens_per_expert, pow2)
+        b_t, sb_t = self.fused_transpose_split_quant(b, self.tokens_per_expert, pow2)
+        FP8GroupGemmMlpFunctionNode._expert_wgrads(a_t, sa_t, b_t, sb_t, expert_w, pow2)
+
+    def bwd_down_weight(self, do3, o2, expert_w2):
+        self._wgrad(o2, do3, expert_w2)
+
+    def bwd_gate_up_weight(self, do1, input_x, expert_w1):
+        self._wgrad(input_x, do1, expert_w1)
+
+    @torch.no_grad()
+    def forward(self, hs_out, unzipped_probs, tokens_per_expert, origin_token_per_experts, scale=None):
+        """fp8_utils.py:1321-1343."""
+        self.origin_token_per_experts = origin_token_per_experts
+        if hs_out.shape[0] == 0:
+            self.unzipped_probs = unzipped_probs.unsqueeze(-1)
+            return torch.zeros_like(hs_out)
+        expert_w1 = [x.up_gate_proj.weight for x in self.custom_map.experts if x is not None]
+        expert_w2 = [x.down_proj.weight for x in self.custom_map.experts if x is not None]
+        num_expert = len(expert_w1)
+        o1 = self.fwd_gate_up(hs_out, expert_w1, num_expert, tokens_per_expert, scale=scale)
+        if not self.recompute_fwd_gate_up:
+            self.o1 = o1
+        o3, unzipped_probs = self.fwd_down(o1, unzipped_probs, expert_w2, num_expert)
+        self.unzipped_probs = unzipped_probs
+        return o3
+
+    @torch.no_grad()
+    def backward(self, out_grad, a2a_async_fn=None):
+        """fp8_utils.py:1345-1436: (dx, probs_grad); zero rows still create the gradient accumulators."""
+        if out_grad.shape[0] == 0:
+            dx = torch.zeros_like(out_grad)
+            probs_grad = torch.zeros_like(self.unzipped_probs)
+            for expert in self.custom_map.experts:
+                if expert is None:
+                    continue
+                for w in (expert.down_proj.weight, expert.up_gate_proj.weight):
+                    if hasattr(w, "main_grad"):
+                        if w.main_grad is None:
+                            w.main_grad = torch.zeros(w.shape, dtype=torch.float32, device=w.device)
+                    elif w.grad is None:
+                        w.grad = torch.zeros(w.shape, dtype=torch.float32, device=w.device)
+            if a2a_async_fn:
+                dx, task = a2a_async_fn(dx)
+                task.wait()
+            return dx, probs_grad
+        expert_w2 = [x.down_proj.weight for x in self.custom_map.experts if x is not None]
+        expert_w1 = [x.up_gate_proj.weight for x in self.custom_map.experts if x is not None]
+        if self.recompute_fwd_gate_up:
+            o1 = self.fwd_gate_up(None if self.dequant_input else self.input, expert_w1, len(expert_w1), self.tokens_per_expert)
+        else:
+            o1 = self.o1
+        do1, o2_s, probs_grad = self.bwd_down_input(expert_w2, out_grad, o1)
+        del o1
+        if not self.recompute_fwd_gate_up:
+            self.o1 = None
+        if self.dequant_input:
+            input_x = F8.fused_act_dequant(self.input_fp8, self.input_scale)
+            self.input_scale = None
+        else:
+            input_x = self.input
+        task = None
+        if a2a_async_fn is None:
+            self.bwd_gate_up_weight(do1, input_x, expert_w1)
+            del input_x
+            if not self.dequant_input:
+                self.input = None
+            dx = self.bwd_gate_up_input(do1, expert_w1)
+            del do1
+            self.bwd_down_weight(out_grad, o2_s, expert_w2)
+        else:
+            dx = self.bwd_gate_up_input(do1, expert_w1)
+            dx, task = a2a_async_fn(dx)
+            self.bwd_gate_up_weight(do1, input_x, expert_w1)
+            del input_x
+            if not self.dequant_input:
+                self.input = None
+            del do1
+            self.bwd_down_weight(out_grad, o2_s, expert_w2)
+            task.wait()
+        self.reset_status()
+        return dx, probs_grad

@@ -199,3 +199,158 @@ def test_ernie_node_rejects_a_ragged_layout():
     tm = torch.tensor([128] * 3, dtype=torch.int32, device="cuda")
     with pytest.raises(ValueError):
         node.forward(G.to_torch_bf16(x[:-128 - 1]), torch.from_numpy(probs).cuda(), tm)
+
+
+# ---------------------------------------------------------------------------------------------
+# ExpertsGroupGemmContiguousNode
+# ---------------------------------------------------------------------------------------------
+
+_ALL_FUSED = {"stack_quant": True, "spaq": True, "swiglu_probs_bwd": True, "transpose_split_quant": True}
+
+
+class _W:
+    def __init__(self, w1, w2):
+        self.w1, self.w2 = w1, w2
+
+
+class _TMap:
+    def __init__(self, experts):
+        self.experts = experts
+
+
+def _contig_case(E, H, I, rows, seed):
+    w1 = [G.bf16_normal((H, 2 * I), seed=seed + e, std=0.03) for e in range(E)]
+    w2 = [G.bf16_normal((I, H), seed=seed + 100 + e, std=0.03) for e in range(E)]
+    M = sum(rows)
+    x = G.bf16_normal((M, H), seed=seed + 500)
+    dout = G.bf16_normal((M, H), seed=seed + 600, std=1e-3)
+    probs = np.random.default_rng(seed).random(M, dtype=np.float32) * 0.5 + 0.25
+    return w1, w2, x, probs, dout
+
+
+def _ernie_experts(w1, w2):
+    ex = []
+    for a, b in zip(w1, w2):
+        t1, t2 = G.to_torch_bf16(a), G.to_torch_bf16(b)
+        t1.main_grad = None
+        t2.main_grad = None
+        ex.append(_Expert(t1, t2))
+    return ex
+
+
+@pytest.mark.parametrize("dequant_input", [False, True])
+@pytest.mark.parametrize("recompute", [False, True])
+def test_ernie_contiguous_node_equals_the_transformers_node_when_every_switch_is_on(dequant_input, recompute):
+    """With stack_quant, spaq, swiglu_probs_bwd and transpose_split_quant the two classes ask for the same
+    operators with the same arguments: identical outputs and gradients."""
+    from paddleformers_amd.ernie_fp8_utils import ExpertsGroupGemmContiguousNode
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 3, 512, 384
+    rows = [256, 0, 384]
+    w1, w2, x, probs, dout = _contig_case(E, H, I, rows, seed=71)
+    ex = _ernie_experts(w1, w2)
+    node = ExpertsGroupGemmContiguousNode(_Map(ex, dict(_ALL_FUSED)), recompute_fwd_gate_up=recompute, dequant_input=dequant_input)
+    tp = torch.from_numpy(probs).cuda()
+    o3 = node.forward(G.to_torch_bf16(x), tp, rows, rows)
+    assert tuple(node.unzipped_probs.shape) == (sum(rows), 1)
+    dx, pg = node.backward(G.to_torch_bf16(dout))
+    assert node.o1 is None and node.m_indices is None           # backward resets the node
+
+    tex = []
+    for a, b in zip(w1, w2):
+        t1, t2 = G.to_torch_bf16(a), G.to_torch_bf16(b)
+        t1.main_grad = None
+        t2.main_grad = None
+        tex.append(_W(t1, t2))
+    ref = FP8GroupGemmMlpFunctionNode(_TMap(tex), recompute_fwd_gate_up=recompute)
+    r3 = ref.forward(G.to_torch_bf16(x), tp.unsqueeze(-1), rows)
+    rdx, rpg = ref.backward(G.to_torch_bf16(dout), tp.unsqueeze(-1), rows)
+    assert torch.equal(o3, r3) and torch.equal(dx, rdx) and torch.equal(pg, rpg)
+    for e in range(E):
+        if rows[e] == 0:
+            continue
+        assert torch.equal(ex[e].down_proj.weight.main_grad, tex[e].w2.main_grad)
+        g1, r1 = ex[e].up_gate_proj.weight.main_grad, tex[e].w1.main_grad
+        if dequant_input:
+            assert torch.equal(g1, r1)      # both transpose the dequantized FP8 copy of the input
+        else:
+            assert G.rel_fro(g1.cpu().numpy(), r1.cpu().numpy()) < 0.06     # this one transposes the bf16 input itself
+
+
+@pytest.mark.parametrize("cfg", [{}, {"split_group_gemm": True}, {"stack_quant": True, "transpose_split_quant": True}])
+def test_ernie_contiguous_node_against_fp32_moe(cfg):
+    from paddleformers_amd.ernie_fp8_utils import ExpertsGroupGemmContiguousNode
+
+    E, H, I = 3, 512, 256
+    rows = [128, 256, 0]
+    w1, w2, x, probs, dout = _contig_case(E, H, I, rows, seed=83)
+    ex = _ernie_experts(w1, w2)
+    node = ExpertsGroupGemmContiguousNode(_Map(ex, dict(cfg)))
+    tp = torch.from_numpy(probs).cuda()
+    o3 = node.forward(G.to_torch_bf16(x), tp, rows, rows)
+    calls = []
+
+    class _Task:
+        def wait(self):
+            calls.append("wait")
+
+    def a2a(t):
+        calls.append("start")
+        return t, _Task()
+
+    dx, pg = node.backward(G.to_torch_bf16(dout), a2a_async_fn=a2a)
+    assert calls == ["start", "wait"]
+    # the masked-layout helper of this file, with every expert's capacity equal to its segment, is the same MoE
+    off, refs = 0, []
+    for e, r in enumerate(rows):
+        refs.append((off, r))
+        off += r
+    xt = torch.tensor(O.bf16_bits_to_f32(x), requires_grad=True)
+    pt = torch.tensor(probs, requires_grad=True)
+    w1t = [torch.tensor(O.bf16_bits_to_f32(w), requires_grad=True) for w in w1]
+    w2t = [torch.tensor(O.bf16_bits_to_f32(w), requires_grad=True) for w in w2]
+    d = torch.tensor(O.bf16_bits_to_f32(dout))
+    outs = torch.zeros((sum(rows), H))
+    loss = 0.0
+    for e, (lo, r) in enumerate(refs):
+        if r == 0:
+            continue
+        h = xt[lo:lo + r] @ w1t[e]
+        y = (torch.nn.functional.silu(h[:, :I]) * h[:, I:] * pt[lo:lo + r, None]) @ w2t[e]
+        outs[lo:lo + r] = y.detach()
+        loss = loss + (y * d[lo:lo + r]).sum()
+    loss.backward()
+    assert G.rel_fro(o3.float().cpu().numpy(), outs.numpy()) < 0.08
+    assert G.rel_fro(dx.float().cpu().numpy(), xt.grad.numpy()) < 0.08
+    assert G.rel_fro(pg.cpu().numpy(), pt.grad.numpy()) < 0.08
+    for e, (lo, r) in enumerate(refs):
+        if r:
+            assert G.rel_fro(ex[e].up_gate_proj.weight.main_grad.cpu().numpy(), w1t[e].grad.numpy()) < 0.08
+            assert G.rel_fro(ex[e].down_proj.weight.main_grad.cpu().numpy(), w2t[e].grad.numpy()) < 0.08
+
+
+def test_ernie_contiguous_node_zero_rows_and_prequantized_input():
+    from paddleformers_amd import functional as F8
+    from paddleformers_amd.ernie_fp8_utils import ExpertsGroupGemmContiguousNode
+
+    E, H, I = 2, 256, 128
+    rows = [128, 128]
+    w1, w2, x, probs, dout = _contig_case(E, H, I, rows, seed=89)
+    ex = _ernie_experts(w1, w2)
+    node = ExpertsGroupGemmContiguousNode(_Map(ex, dict(_ALL_FUSED)))
+    o = node.forward(torch.zeros((0, H), dtype=torch.bfloat16, device="cuda"), torch.zeros((0,), device="cuda"), [0, 0], [0, 0])
+    assert tuple(o.shape) == (0, H)
+    dx, pg = node.backward(torch.zeros((0, H), dtype=torch.bfloat16, device="cuda"))
+    assert tuple(dx.shape) == (0, H) and tuple(pg.shape) == (0, 1)
+    assert all(e.up_gate_proj.weight.main_grad is not None and not e.up_gate_proj.weight.main_grad.any() for e in ex)
+    # an (fp8, scale) input needs dequant_input
+    xq, xs = F8.fp8_quant_blockwise(G.to_torch_bf16(x), quant_method="1x128", input_transpose=False, output_scale_transpose=False)
+    tp = torch.from_numpy(probs).cuda()
+    with pytest.raises(AssertionError):
+        node.forward(xq, tp, rows, rows, scale=xs)
+    node2 = ExpertsGroupGemmContiguousNode(_Map(ex, dict(_ALL_FUSED)), dequant_input=True)
+    a = node2.forward(xq, tp, rows, rows, scale=xs)
+    node3 = ExpertsGroupGemmContiguousNode(_Map(ex, dict(_ALL_FUSED)))
+    b = node3.forward(G.to_torch_bf16(x), tp, rows, rows)
+    assert torch.equal(a, b)
