@@ -129,3 +129,40 @@ def test_zipf_expert_counts_generator():
     assert (padded % 128 == 0).all() and (padded >= counts).all() and (padded - counts < 128).all()
     c2, _ = G.zipf_counts(8192, 32, 1.1, seed=3)
     assert np.array_equal(counts, c2)
+
+
+def test_ernie_and_inference_mirrors_host_logic_without_a_gpu():
+    """The host logic of the ERNIE wrappers and of the inference-style linear that needs no kernel: the
+    padding rule, the config switch lookup, the cached-weight lookup, the scale registration, the plain
+    linear on a wide weight; quantised work on CPU tensors raises instead of falling back."""
+    from paddleformers_amd import ernie_fp8_linear as EL
+    from paddleformers_amd import ernie_fp8_utils as EU
+    from paddleformers_amd import fp8_linear as FL
+    from paddleformers_amd import kernel as K8
+
+    for n in (1, 128, 300, 384, 512, 900):
+        exp = n if n % 512 == 0 else (n // 512 + 1) * 512
+        assert EL.padding(torch.ones((n, 4)), 0).shape[0] == exp and EL.padding(torch.ones((4, n)), 1).shape[1] == exp
+    assert EU.has_config({"spaq": True}, "spaq") and not EU.has_config({"spaq": False}, "spaq") and not EU.has_config({}, "spaq")
+
+    class W:
+        pass
+
+    w = W()
+    w.fp8_weight_stacked, w.fp8_scale_stacked = "q", "s"
+    w.fp8_weight_stacked_transpose, w.fp8_scale_stacked_transpose = "qt", "st"
+    assert EU.fused_stack_transpose_quant([w], transpose=False) == ("q", "s")
+    assert EU.fused_stack_transpose_quant([w], transpose=True) == ("qt", "st")
+
+    layer = FL.Linear(300, 200, bias=True, dtype=torch.float8_e4m3fn, device="cpu")
+    assert tuple(layer.weight_scale_inv.shape) == (3, 2) and layer.weight._scale is layer.weight_scale_inv
+    plain = FL.Linear(8, 4, bias=True, dtype=torch.float32, device="cpu")
+    assert not hasattr(plain, "weight_scale_inv")
+    x = torch.ones((2, 8))
+    assert torch.equal(plain(x), x @ plain.weight + plain.bias)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        layer(torch.ones((2, 300), dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        K8.act_quant(torch.zeros((4, 128), dtype=torch.bfloat16))
+    with pytest.raises(AssertionError):
+        K8.act_quant(torch.zeros((4, 100), dtype=torch.bfloat16))
