@@ -354,8 +354,35 @@ def bench_other_gemms(iters=10, warmup=3):
     del exm, gm1, gm2, xm, dm, nodem
     torch.cuda.empty_cache()
     # the fused FP8 MoE node end to end at config 5: forward + backward (dgrad and wgrad, both GEMMs),
-    # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers
+    # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers; then the same step
+    # with power-of-two scales throughout (use_ue8m0): forward and dgrad GEMMs on the block-scaled MFMA kernel
+    node_flop = 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H)
+    out["moe_node_config5_fwd_bwd"] = {"flop": node_flop, "ms": bench_moe_node(False, 3, 2)}
+    out["moe_node_config5_fwd_bwd_ue8m0"] = {"flop": node_flop, "ms": bench_moe_node(True, 3, 2)}
+    for v in out.values():
+        if "flop" in v:
+            v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)
+            v["frac_fp8_peak"] = round(v["TFLOPs"] / FP8_PEAK_TFLOPS, 4)
+        else:
+            v["GBps"] = round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)
+            v["frac_hbm"] = round(v["GBps"] / HBM_PEAK_GBS, 4)
+        v["ms"] = round(v["ms"], 4)
+    torch.cuda.empty_cache()
+    return out
+
+
+def bench_moe_node(ue8m0, iters, warmup):
+    """ms per forward + backward of FP8GroupGemmMlpFunctionNode at config 5 (E=128, H=4096, I=1408, 131072
+    routed rows, Zipf(1.0), segments padded to 128): cached stacked FP8 weights, weight gradients accumulated
+    into stacked fp32 buffers.  ue8m0: power-of-two scales throughout, GEMMs on the block-scaled MFMA kernel."""
+    import torch
+
     from paddleformers_amd import fp8_utils as U8
+
+    E, H, I, ROUTED = 128, 4096, 1408, 131072
+    _, padded = zipf_counts(ROUTED, E, 1.0, seed=5, n_empty=0)
+    Mp = int(padded.sum())
+    rows = [int(r) for r in padded]
 
     class _Ex:
         pass
@@ -372,10 +399,10 @@ def bench_other_gemms(iters=10, warmup=3):
         ex.w2 = (torch.randn((I, H), device="cuda") * 0.02).to(torch.bfloat16)
         ex.w1.main_grad, ex.w2.main_grad = g1[e], g2[e]
         exps.append(ex)
-    U8.fp8_quant_weight([ex.w1 for ex in exps], [ex.w2 for ex in exps], batch_mode=True)
+    U8.fp8_quant_weight([ex.w1 for ex in exps], [ex.w2 for ex in exps], batch_mode=True, using_pow2_scale=bool(ue8m0))
     mp = _Mp()
     mp.experts = exps
-    node = U8.FP8GroupGemmMlpFunctionNode(mp)
+    node = U8.FP8GroupGemmMlpFunctionNode(mp, use_ue8m0=bool(ue8m0))
     xin = torch.randn((Mp, H), device="cuda").to(torch.bfloat16)
     dout = (torch.randn((Mp, H), device="cuda") * 1e-3).to(torch.bfloat16)
     pr = torch.rand((Mp, 1), device="cuda")
@@ -384,30 +411,10 @@ def bench_other_gemms(iters=10, warmup=3):
         node.forward(xin, pr, rows)
         node.backward(dout, pr, rows, reset_status=True)
 
-    ms = time_kernel(fwd_bwd, [()], 3, 2)
-    out["moe_node_config5_fwd_bwd"] = {"flop": 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H), "ms": ms}
-    # the same step with power-of-two scales throughout (use_ue8m0): forward and dgrad GEMMs on the block-scaled MFMA kernel
-    for ex in exps:
-        for w in (ex.w1, ex.w2):
-            for name in ("fp8_weight_stacked", "fp8_scale_stacked", "fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose",
-                         "fp8_scale_is_pow2"):
-                if hasattr(w, name):
-                    delattr(w, name)
-    U8.fp8_quant_weight([ex.w1 for ex in exps], [ex.w2 for ex in exps], batch_mode=True, using_pow2_scale=True)
-    node = U8.FP8GroupGemmMlpFunctionNode(mp, use_ue8m0=True)
-    ms = time_kernel(fwd_bwd, [()], 3, 2)
-    out["moe_node_config5_fwd_bwd_ue8m0"] = {"flop": 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H), "ms": ms}
+    ms = time_kernel(fwd_bwd, [()], iters, warmup)
     del node, exps, g1, g2, xin, dout
-    for v in out.values():
-        if "flop" in v:
-            v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)
-            v["frac_fp8_peak"] = round(v["TFLOPs"] / FP8_PEAK_TFLOPS, 4)
-        else:
-            v["GBps"] = round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)
-            v["frac_hbm"] = round(v["GBps"] / HBM_PEAK_GBS, 4)
-        v["ms"] = round(v["ms"], 4)
     torch.cuda.empty_cache()
-    return out
+    return ms
 
 
 def cpu_baseline(H, I, rows=12288):
@@ -449,6 +456,9 @@ def main():
     ap.add_argument("--copy-yardstick", action="store_true",
                     help="also launch one plain 1 GiB copy (pf8::k_debug_copy) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings of the GEMM can be scaled by a kernel of known traffic")
+    ap.add_argument("--moe-node", choices=["fp32", "ue8m0"],
+                    help="run only the config 5 MoE node leg (forward + backward, --steps/--warmup iterations) with fp32 or "
+                         "UE8M0 scales and print its time: the run to profile for the node's per-kernel breakdown")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path uses no collectives and the run has a single MI355X; use --gpus 1",
@@ -465,6 +475,13 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
     torch.manual_seed(3)
+
+    if args.moe_node:
+        ms = bench_moe_node(args.moe_node == "ue8m0", args.steps, args.warmup)
+        flop = 3 * (2.0 * 131072 * 4096 * 2 * 1408 + 2.0 * 131072 * 1408 * 4096)
+        print(json.dumps({"leg": "moe_node_config5_fwd_bwd" + ("_ue8m0" if args.moe_node == "ue8m0" else ""), "steps": args.steps,
+                          "warmup": args.warmup, "ms": round(ms, 4), "TFLOPs": round(flop / ms / 1e9, 1)}))
+        return
 
     E, H, I, ROUTED = 32, 7168, 2048, 8192
     counts, padded = zipf_counts(ROUTED, E, 1.1, seed=3)
