@@ -184,6 +184,42 @@ def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_tra
             quantize_weights([w2])
 
 
+def fp8_quant_weight_all_layers(layers, quant_transpose=None, using_pow2_scale=False):
+    """What FP8QuantWeightCallback.on_step_begin (trainer/trainer_callback.py:725-765) asks for through
+    model.fp8_quant_weight(True, ...): the batch-mode caches of every MoE layer, here built by ONE launch
+    per weight shape instead of one (or two) per layer and list.  `layers` is a sequence of
+    (expert_w1_list, expert_w2_list); every list gets the attributes fp8_quant_weight(batch_mode=True)
+    attaches to its first weight, as views of the shared outputs, bit-identical to the per-layer calls.
+    Lists that already carry a cache are left alone."""
+    if quant_transpose not in (None, True, False):
+        raise ValueError("Invalid value for `quant_transpose`.")
+    groups = {}
+    for w1_list, w2_list in layers:
+        for lst in (w1_list, w2_list):
+            ws = [w for w in lst if w is not None]
+            if not ws or hasattr(ws[0], "fp8_weight_stacked") or hasattr(ws[0], "fp8_weight_stacked_transpose"):
+                continue
+            groups.setdefault((tuple(ws[0].shape), len(ws)), []).append(ws)
+    for ((R, Cc), E), lists in groups.items():
+        flat = [w for ws in lists for w in ws]
+        q = s = qt = st = None
+        if quant_transpose is None:
+            q, s, qt, st = F8.fused_stack_quant_both(flat, using_pow2_scale=using_pow2_scale)
+        elif quant_transpose is False:
+            q, s = F8.fused_stack_transpose_quant(flat, transpose=False, using_pow2_scale=using_pow2_scale)
+        else:
+            qt, st = F8.fused_stack_transpose_quant(flat, transpose=True, using_pow2_scale=using_pow2_scale)
+        for i, ws in enumerate(lists):
+            w0 = ws[0]
+            if q is not None:
+                w0.fp8_weight_stacked = q[i * E * R:(i + 1) * E * R]
+                w0.fp8_scale_stacked = s[i * E * R // 128:(i + 1) * E * R // 128]
+            if qt is not None:
+                w0.fp8_weight_stacked_transpose = qt[i * E * Cc:(i + 1) * E * Cc]
+                w0.fp8_scale_stacked_transpose = st[i * E * Cc // 128:(i + 1) * E * Cc // 128]
+            w0.fp8_scale_is_pow2 = bool(using_pow2_scale)
+
+
 def split_group_gemm(x_fp8, x_scale, w_fp8, w_scale, tokens_per_expert, gemm_out):
     """fp8_utils.py:853-870: the grouped GEMM as a loop of dense GEMMs, empty experts skipped."""
     start_idx = 0

@@ -261,6 +261,40 @@ def test_fp8_quant_weight_caches_what_fused_stack_quant_reads():
                            quant_transpose="both")
 
 
+@pytest.mark.parametrize("quant_transpose", [None, False, True])
+def test_fp8_quant_weight_all_layers_equals_the_per_layer_calls(quant_transpose):
+    """Every MoE layer's batch-mode cache from one launch per weight shape: same tensors as
+    fp8_quant_weight(batch_mode=True) layer by layer, and lists that are already cached are skipped."""
+    from paddleformers_amd import fp8_utils as U
+
+    E, H, I, L = 2, 256, 128, 3
+
+    def make(seed):
+        return ([G.to_torch_bf16(G.bf16_normal((H, 2 * I), seed=seed + e, std=0.02)) for e in range(E)],
+                [G.to_torch_bf16(G.bf16_normal((I, H), seed=seed + 50 + e, std=0.02)) for e in range(E)])
+
+    layers, refs = [make(600 + 100 * i) for i in range(L)], [make(600 + 100 * i) for i in range(L)]
+    for w1, w2 in refs:
+        U.fp8_quant_weight(w1, w2, batch_mode=True, quant_transpose=quant_transpose)
+    sentinel = object()
+    layers[1][1][0].fp8_weight_stacked = sentinel            # this list already has a cache
+    U.fp8_quant_weight_all_layers(layers, quant_transpose=quant_transpose)
+    assert layers[1][1][0].fp8_weight_stacked is sentinel and not hasattr(layers[1][1][0], "fp8_scale_stacked")
+    names = {None: ["fp8_weight_stacked", "fp8_scale_stacked", "fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose"],
+             False: ["fp8_weight_stacked", "fp8_scale_stacked"], True: ["fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose"]}[quant_transpose]
+    for li in range(L):
+        for k in (0, 1):
+            if (li, k) == (1, 1):
+                continue
+            got, ref = layers[li][k][0], refs[li][k][0]
+            for n in names:
+                a, b = getattr(got, n), getattr(ref, n)
+                assert a.shape == b.shape and torch.equal(a.view(torch.uint8) if a.dtype != torch.float32 else a,
+                                                          b.view(torch.uint8) if b.dtype != torch.float32 else b), (li, k, n)
+            assert got.fp8_scale_is_pow2 is False
+            assert not hasattr(layers[li][k][1], "fp8_weight_stacked")      # batch mode: only the first weight carries the cache
+
+
 # ---------------------------------------------------------------------------------------------
 # fused quant + transpose
 # ---------------------------------------------------------------------------------------------
