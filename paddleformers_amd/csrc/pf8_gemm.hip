@@ -17,6 +17,7 @@
 // 128(P) x 128(Q) x 128(K), each wavefront 64x64 = 4x4 MFMA tiles, operands staged through
 // registers into two 32 KB LDS stages).  LDS rows are 128 B with their 16-byte chunks XOR-swizzled
 // so that fragment reads (16 rows x 32 B per quarter-wave) are bank-conflict free.
+#include <atomic>
 #include <type_traits>
 
 #include "pf8_device.h"
@@ -866,10 +867,14 @@ using namespace pf8;
 #define PF8_ALIGNED16(p) ((reinterpret_cast<uintptr_t>(p) & 15u) == 0)
 
 static int ensure_lds_attr() {
-    // 64 KB of dynamic LDS needs the opt-in attribute once per kernel instantiation
-    static int done = 0;
-    if (done) return PF8_OK;
-    hipError_t e = hipSuccess;
+    // more than 64 KB of dynamic LDS needs the opt-in attribute, once per kernel instantiation and device
+    // (a bit per device; two threads racing here both set the same attributes, which is harmless)
+    static std::atomic<uint64_t> done{0};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return PF8_OK;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_wgrad<false>), hipFuncAttributeMaxDynamicSharedMemorySize, 69632);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_wgrad<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 69632);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
@@ -878,7 +883,7 @@ static int ensure_lds_attr() {
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
-    done = 1;
+    done.fetch_or(bit, std::memory_order_release);
     return PF8_OK;
 }
 

@@ -27,6 +27,7 @@
 //     the blocks of every expert (an odd one out gets a half-empty tile, padding blocks get none) and
 //     writes the list the GEMM walks.  Without a list the kernel walks aligned 256-row tiles and
 //     visits a tile that holds two experts twice, once per expert, each pass storing its own half.
+#include <atomic>
 #include <type_traits>
 
 #include "pf8_device.h"
@@ -465,11 +466,16 @@ using namespace pf8;
 static constexpr int E8_LDS_BYTES = 131072 + 4 * 16 * 272;
 
 static int launch_e8(const E8Args& a, int64_t max_q_tiles, hipStream_t st, const char* where) {
-    static int attr_done = 0;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_e8), hipFuncAttributeMaxDynamicSharedMemorySize, E8_LDS_BYTES);
+    // the LDS opt-in, once per device (a bit per device; a race sets the same attribute twice)
+    static std::atomic<uint64_t> attr_done{0};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, where, hipGetErrorString(e));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(attr_done.load(std::memory_order_acquire) & bit)) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_e8), hipFuncAttributeMaxDynamicSharedMemorySize, E8_LDS_BYTES);
         if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, where, hipGetErrorString(e));
-        attr_done = 1;
+        attr_done.fetch_or(bit, std::memory_order_release);
     }
     const int64_t T = ((a.Prows + 255) / 256) * max_q_tiles, per_xcd = (T + 7) / 8;
     int64_t w = pf8_effective_cus() / 8;
