@@ -82,6 +82,17 @@ def test_argument_validation_without_a_gpu(lib):
     assert lib.pf8_grouped_wgrad(aligned, aligned, aligned, aligned, rows, 2, 128, 128, aligned, 1, None) == -1
     # q/s must come as pairs
     assert lib.pf8_quant_128x128(aligned, 128, 128, aligned, None, None, None, 0, None) == -1
+    # the one-read row-wise + transposed quantizer: ragged segment, missing row-wise outputs, misaligned input
+    good = (C.c_int64 * 2)(128, 128)
+    assert lib.pf8_quant_and_transpose_split(aligned, rows, 2, 128, aligned, aligned, 0, aligned, aligned, 1, None) == -1
+    assert "multiples of 128" in _lib.last_error()
+    assert lib.pf8_quant_and_transpose_split(aligned, good, 2, 128, None, None, 0, aligned, aligned, 1, None) == -1
+    assert lib.pf8_quant_and_transpose_split(C.c_void_p(aligned.value + 2), good, 2, 128, aligned, aligned, 0, aligned, aligned, 1, None) == -1
+    assert lib.pf8_quant_and_transpose_split(aligned, good, 2, 100, aligned, aligned, 0, aligned, aligned, 1, None) == -1
+    # UE8M0 GEMM: N must be a multiple of 128 and at least 256, K at least 384
+    assert lib.pf8_gemm_nt_ue8m0(aligned, aligned, 128, aligned, aligned, 128, 128, 512, aligned, 128, None) == -1
+    assert lib.pf8_gemm_nt_ue8m0(aligned, aligned, 128, aligned, aligned, 128, 384, 256, aligned, 384, None) == -1
+    assert lib.pf8_gemm_nt_ue8m0(aligned, aligned, 128, aligned, aligned, 128, 320, 512, aligned, 320, None) == -1
 
 
 def test_cpu_tensors_raise_instead_of_falling_back():
