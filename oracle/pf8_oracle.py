@@ -400,11 +400,14 @@ def block_dequant(q: np.ndarray, scale: np.ndarray, scale_format: str, block_axe
 
 
 # ---------------------------------------------------------------------------------------------
-# moe_permute / moe_unpermute (numpy restatement).  PARITY UNPINNED: the operators live in the
-# paddlepaddle-gpu binary, the reference holds no test or fixture for them; the semantics below are
-# what its call sites rely on (cli/train/deepseek_v3_pretrain/moe_utils.py:141-261): expert-sorted
-# rows, token order kept inside an expert, zero rows up to a multiple of padding_alignment, a
-# [T, num_experts] row map with -1 for "not routed", fp32 summation in slot order on the way back.
+# moe_permute / moe_unpermute (numpy restatement).  The operators live in the paddlepaddle-gpu binary
+# and the reference holds no test or fixture for them.  Pinned: the row order and content of the
+# permutation and the scatter-add back, against the un-fused statement the reference keeps in plain
+# tensor operations (topk_to_permuted_indices / permute_fast / unpermute_fast,
+# cli/train/deepseek_v3_pretrain/moe_utils.py:57-130; tests/test_oracle_ops.py).  PARITY UNPINNED: what
+# only the fused operators define -- zero rows up to a multiple of padding_alignment, the
+# [T, num_experts] row map with -1 for "not routed", fp32 summation in slot order on the way back --
+# taken from what the call sites rely on (moe_utils.py:141-261).
 # ---------------------------------------------------------------------------------------------
 
 

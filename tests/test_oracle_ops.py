@@ -333,3 +333,32 @@ def test_moe_permute_unpermute_invariants():
     back, pb = O.moe_unpermute(ox, rowmap, rm, op, T, E)
     assert (O.bf16_bits_to_f32(back) == xv * (rm >= 0).sum(axis=1, keepdims=True)).all()
     assert (pb == np.where(rm >= 0, probs, 0)).all()
+
+
+def test_moe_permute_row_order_is_the_in_repo_permute_fast():
+    """cli/train/deepseek_v3_pretrain/moe_utils.py:57-88 states the un-fused permutation in plain tensor
+    operations: for expert 0, 1, ... the flat (token-major) positions of the routing map that name the
+    expert, in ascending order; token = position // topk; rows and probabilities are gathered in that order.
+    Without padding (alignment 1) the restated operator must give exactly that."""
+    rng = np.random.default_rng(1)
+    T, H, topk, E = 64, 8, 4, 6
+    rm = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    counts = [int((rm == e).sum()) for e in range(E)]
+    probs = rng.random(rm.shape).astype(np.float32)
+    x = O.f32_to_bf16_bits(rng.standard_normal((T, H)).astype(np.float32))
+    flat = rm.reshape(-1)
+    prob_idx = np.concatenate([np.nonzero(flat == e)[0] for e in range(E)])       # topk_to_permuted_indices
+    token_idx = prob_idx // topk
+    ox, rowmap, op, _ = O.moe_permute(x, None, rm, probs, E, counts, 1)
+    assert np.array_equal(ox, x[token_idx])                                     # permute_fast: index_select
+    assert np.array_equal(op[:, 0], probs.reshape(-1)[prob_idx])                # the probs gathered the same way
+    # the row map is the inverse of that order
+    for r, (t, p) in enumerate(zip(token_idx, prob_idx)):
+        assert rowmap[t, flat[p]] == r
+    # unpermute_fast (:90-130) scatter-adds the permuted rows back to their tokens: small integers make it exact
+    xi = rng.integers(-3, 4, size=(T, H)).astype(np.float32)
+    oxi, rowmap, opi, _ = O.moe_permute(O.f32_to_bf16_bits(xi), None, rm, probs, E, counts, 1)
+    back, _ = O.moe_unpermute(oxi, rowmap, rm, opi, T, E)
+    ref = np.zeros((T, H), np.float32)
+    np.add.at(ref, token_idx, O.bf16_bits_to_f32(oxi))
+    assert np.array_equal(O.bf16_bits_to_f32(back), ref)
