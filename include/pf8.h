@@ -45,6 +45,8 @@ const char* pf8_last_error(void);
  * compute units the GEMM grids are sized for (0 = all).  Returns the previous value. */
 int pf8_set_num_cus(int n);
 int pf8_get_num_cus(void);
+/* The budget in force on the current device: min(pf8_set_num_cus value, the device's compute units). */
+int pf8_effective_num_cus(void);
 
 /* fp8_quant_blockwise(x, quant_method="1x128", input_transpose=False, output_scale_transpose=...)
  * transformers/fp8_utils.py:262-268, 938-941; cli/train/deepseek_v3_pretrain/kernel.py:29-70.
@@ -137,8 +139,9 @@ int pf8_block_dequant(const uint8_t* q, const void* scale, int scale_format, int
  * expert's segment padded to a multiple of padding_alignment (zero rows), rowmap int32 [T,E] (row of
  * token t in expert e's segment, -1 = not routed; tokens keep their order inside a segment),
  * out_probs fp32 [Mpad] (0 on padding rows; NULL to skip), out_xs fp32 [Mpad,H/128] (with xs).
- * *overflow (device int32, cleared by the caller) is set when a token is routed to an expert whose
- * tokens_per_expert count is already used up; such copies are dropped. */
+ * *overflow (device int32, cleared by the caller): bit 0 is set when a token is routed to an expert whose
+ * tokens_per_expert count is already used up (such copies are dropped), bit 1 when an expert receives
+ * fewer tokens than its count says (the rows left over are written as zeros, like padding rows). */
 int pf8_moe_permute(const void* x, int x_is_fp8, const float* xs, const int32_t* routemap,
                     const float* probs, int64_t T, int64_t H, int topk, int E,
                     const int64_t* tokens_per_expert, int padding_alignment, void* out_x,
@@ -260,18 +263,6 @@ int pf8_gemm_nt_1d1d_f32_pow2(const uint8_t* a_t, const float* sa_t, const uint8
 int pf8_grouped_wgrad_pow2(const uint8_t* a_t, const float* sa_t, const uint8_t* b_t,
                            const float* sb_t, const int64_t* rows_per_expert, int E, int64_t Kin,
                            int64_t N, float* out, int accumulate, pf8_stream_t stream);
-
-/* Measurement hook: a plain device-to-device copy of nbytes (multiple of 16).  bench.py launches it
- * so that hardware traffic counters (FETCH_SIZE / WRITE_SIZE) can be scaled by a kernel whose
- * traffic is known. */
-int pf8_debug_copy(const void* src, void* dst, int64_t nbytes, pf8_stream_t stream);
-/* Self-test hook used by the GPU tests: converts n floats to e4m3 with the same device routine the
- * quantizers use (hardware OCP convert), so the codec can be swept exhaustively. */
-int pf8_debug_encode(const float* v, int64_t n, uint8_t* out, pf8_stream_t stream);
-/* Self-test hook: q[i] = e4m3(x[i] / s[i]) through the quantizers' fast-division path. */
-int pf8_debug_div_encode(const float* x, const float* s, int64_t n, uint8_t* out, pf8_stream_t stream);
-/* Self-test hook: out[i] = silu(x[i]) with the device restatement of the oracle's expf. */
-int pf8_debug_silu(const float* x, int64_t n, float* out, pf8_stream_t stream);
 
 #ifdef __cplusplus
 }

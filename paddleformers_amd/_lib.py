@@ -15,11 +15,12 @@ _lib = None
 
 _i64, _i32, _vp = C.c_int64, C.c_int, C.c_void_p
 
-# name -> argtypes; mirrors include/pf8.h one for one
+# name -> argtypes; mirrors include/pf8.h (and the self-test hooks of include/pf8_selftest.h) one for one
 SIGNATURES = {
     "pf8_version": [],
     "pf8_set_num_cus": [_i32],
     "pf8_get_num_cus": [],
+    "pf8_effective_num_cus": [],
     "pf8_quant_1x128": [_vp, _i64, _i64, _i64, _vp, _vp, _i32, _i32, _vp],
     "pf8_quant_128x128": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i32, _vp],
     "pf8_quant_transpose": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _vp],

@@ -15,7 +15,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libpf8.so")
 SOURCES = ["pf8_api.hip", "pf8_quant.hip", "pf8_gemm.hip", "pf8_gemm_e8.hip", "pf8_permute.hip", "pf8_norm.hip"]
-HEADERS = ["pf8_device.h", "pf8_host.h", os.path.join("..", "..", "include", "pf8.h")]
+HEADERS = ["pf8_device.h", "pf8_host.h", os.path.join("..", "..", "include", "pf8.h"),
+           os.path.join("..", "..", "include", "pf8_selftest.h")]
 
 FLAGS = [
     "--offload-arch=gfx950",

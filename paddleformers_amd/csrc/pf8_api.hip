@@ -7,7 +7,8 @@
 namespace {
 thread_local char g_err[512] = "";
 std::atomic<int> g_num_cus{0};
-std::atomic<int> g_dev_cus{-1};
+constexpr int MAX_DEVICES = 64;
+std::atomic<int> g_dev_cus[MAX_DEVICES];   // compute units of each device, 0 = not asked yet
 }  // namespace
 
 int pf8_fail(int code, const char* where, const char* msg) {
@@ -22,18 +23,25 @@ int pf8_check_launch(const char* where) {
     return PF8_ELAUNCH;
 }
 
-int pf8_effective_cus() {
-    int dev = g_dev_cus.load();
-    if (dev < 0) {
-        int d = 0, n = 0;
-        if (hipGetDevice(&d) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, d) != hipSuccess || n <= 0)
-            n = 256;
-        g_dev_cus.store(n);
-        dev = n;
+// compute units of the CURRENT device, asked once per device
+static int device_cus() {
+    int d = 0;
+    if (hipGetDevice(&d) != hipSuccess || d < 0) d = 0;
+    const int slot = d % MAX_DEVICES;
+    int n = g_dev_cus[slot].load(std::memory_order_relaxed);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, d) != hipSuccess || n <= 0) n = 256;
+        g_dev_cus[slot].store(n, std::memory_order_relaxed);
     }
-    int cap = g_num_cus.load();
+    return n;
+}
+int pf8_effective_cus() {
+    const int dev = device_cus(), cap = g_num_cus.load();
     return (cap > 0 && cap < dev) ? cap : dev;
+}
+bool pf8_cus_capped() {
+    const int cap = g_num_cus.load();
+    return cap > 0 && cap < device_cus();
 }
 
 extern "C" int pf8_version(void) { return 100; }
@@ -43,3 +51,4 @@ extern "C" int pf8_set_num_cus(int n) {
     return prev;
 }
 extern "C" int pf8_get_num_cus(void) { return g_num_cus.load(); }
+extern "C" int pf8_effective_num_cus(void) { return pf8_effective_cus(); }

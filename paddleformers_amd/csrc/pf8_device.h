@@ -45,35 +45,20 @@ __device__ __forceinline__ uint32_t row16_max(uint32_t v) {
     return v;
 }
 
-// 16-byte / 8-byte global accesses.  PF8_STREAMING=1 marks them non-temporal (streamed once).
-#ifndef PF8_STREAMING
-#define PF8_STREAMING 0
-#endif
+// 16-byte / 8-byte global accesses
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint4 ld16(const void* p) {
-#if PF8_STREAMING
-    u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-#else
     u32x4 v = *reinterpret_cast<const u32x4*>(p);
-#endif
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ void st16(void* p, uint4 o) {
     u32x4 v = {o.x, o.y, o.z, o.w};
-#if PF8_STREAMING
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
-#else
     *reinterpret_cast<u32x4*>(p) = v;
-#endif
 }
 __device__ __forceinline__ void st8(void* p, uint2 o) {
     u32x2 v = {o.x, o.y};
-#if PF8_STREAMING
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
-#else
     *reinterpret_cast<u32x2*>(p) = v;
-#endif
 }
 
 __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }

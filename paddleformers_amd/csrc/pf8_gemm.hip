@@ -50,18 +50,9 @@ struct GemmArgs {
     int pow2_scales;            // wgrad: every scale is a power of two (applied inside the MFMA)
 };
 
-#ifndef PF8_SWZ
-#define PF8_SWZ 2
-#endif
-__device__ __forceinline__ int swz_key(int row) {
-#if PF8_SWZ == 0
-    return (row >> 1) & 7;
-#elif PF8_SWZ == 1
-    return row & 7;
-#else
-    return (row & 7) ^ ((row >> 3) & 1);
-#endif
-}
+// 16-byte chunk c of LDS row `row` lives at chunk c ^ swz_key(row): the 16 rows a fragment read touches
+// then fall on 16 different bank groups of the 64-bank LDS
+__device__ __forceinline__ int swz_key(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 __device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ swz_key(row)) << 4); }
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -125,10 +116,12 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
     const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = (a.Qrows + BQ - 1) / BQ;
     const int64_t T = p_tiles * q_tiles;
     // consecutive workgroups go round-robin to the 8 XCDs: give every XCD a contiguous run of logical
-    // tiles, ordered in groups of 16 q-tiles x all p-tiles
+    // tiles, ordered in groups of 16 q-tiles x all p-tiles.  The grid normally holds one workgroup per
+    // tile; under a compute-unit budget it is smaller and a workgroup walks its XCD's run in strides.
     const int64_t per_xcd = (T + 7) / 8;
-    const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= T) return;
+    for (int64_t loc = blockIdx.x >> 3; loc < per_xcd; loc += gridDim.x >> 3) {
+    const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + loc;
+    if (logical >= T) break;
     constexpr int G = 16;
     const int64_t grp = logical / (G * p_tiles), rem = logical % (G * p_tiles);
     const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;
@@ -144,11 +137,11 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
     int e = 0, row_hi = BQ;
     if (a.group == GROUP_CONTIG) {
         e = a.m_indices[q0];
-        if (e < 0) return;
+        if (e < 0) continue;
     } else if (a.group == GROUP_MASKED) {
         e = blockIdx.y;
         const int64_t valid = a.masked_m[e];
-        if (q0 >= valid) return;
+        if (q0 >= valid) continue;
         row_hi = valid - q0 < BQ ? (int)(valid - q0) : BQ;
         qbase += (int64_t)e * a.Qrows * a.red;
         sqb += (int64_t)e * a.Qrows * KB;
@@ -305,6 +298,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
         } else if (col + 4 <= a.Prows) {
             *reinterpret_cast<uint2*>(dst) = make_uint2(v.x, v.y);
         }
+    }
+    __syncthreads();   // the staging rows are dead before the next tile's copies land on them
     }
 #undef PF8_DMA_P
 #undef PF8_DMA_Q
@@ -832,24 +827,28 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         // fit one round of compute units (dense M <= 2048 at N = 4096), +15% / +7% on the up+gate /
         // down GEMMs of 32 experts with a skewed 8192-row load, parity (0.92..1.06) elsewhere, where
         // its static tile assignment loses what the deeper pipeline gains.
-        // PF8_FWD_KERNEL=deep|wide overrides the choice (benchmarking).
-        static const char* force = getenv("PF8_FWD_KERNEL");
         const bool aligned = a.Prows % 256 == 0 && a.Qrows % 128 == 0 && a.red >= 384 && a.group != GROUP_MASKED;
         const int64_t cus = pf8_effective_cus();
-        bool deep = aligned && (T128 <= cus || (a.group == GROUP_CONTIG && a.red >= 2048 && T128 <= 10 * cus));
-        if (force && force[0] == 'd') deep = aligned;
-        if (force && force[0] == 'w') deep = false;
+        const bool deep = aligned && (T128 <= cus || (a.group == GROUP_CONTIG && a.red >= 2048 && T128 <= 10 * cus));
         if (deep) {
             // persistent: one workgroup per compute unit (or per tile of an XCD's run, if fewer)
             const int64_t per_xcd = (T128 + 7) / 8;
-            int64_t w = pf8_effective_cus() / 8;
+            int64_t w = cus / 8;
             if (w < 1) w = 1;
             if (w > per_xcd) w = per_xcd;
             dim3 gd((unsigned)(8 * w), 1);
             if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0>), gd, dim3(256), 147456, st, a);
             else hipLaunchKernelGGL((k_gemm_fwd_deep<1>), gd, dim3(256), 147456, st, a);
-        } else if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd128<0>), g128, dim3(256), 81920, st, a);
-        else hipLaunchKernelGGL((k_gemm_fwd128<1>), g128, dim3(256), 81920, st, a);
+        } else {
+            // under a compute-unit budget: two workgroups per budgeted unit, each walking several tiles
+            if (pf8_cus_capped()) {
+                int64_t w = 2 * cus / 8;
+                if (w < 1) w = 1;
+                if (8 * w < (int64_t)g128.x) g128.x = (unsigned)(8 * w);
+            }
+            if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd128<0>), g128, dim3(256), 81920, st, a);
+            else hipLaunchKernelGGL((k_gemm_fwd128<1>), g128, dim3(256), 81920, st, a);
+        }
     } else {
         const int64_t Tw = ((a.Prows + 127) / 128) * ((a.Qrows + 127) / 128);
         dim3 gw((unsigned)(((Tw + 7) / 8) * 8), grid.y);
@@ -889,16 +888,16 @@ static int ensure_lds_attr() {
 
 int pf8_launch_deep_ue8m0(const uint8_t* p, const uint8_t* q, const uint8_t* sp8, const uint8_t* sq8, int64_t ldsq, void* out,
                           int64_t Prows, int64_t Qrows, int64_t red, int E, const int32_t* m_indices, const int32_t* pair_list,
-                          hipStream_t stream, const char* where) {
+                          int cus, hipStream_t stream, const char* where) {
     if (Prows % 256 != 0 || Qrows % 128 != 0 || red % 128 != 0 || red < 384) return pf8_fail(PF8_EINVAL, where, "shape outside the persistent kernel's tiling");
     int rc = ensure_lds_attr();
     if (rc) return rc;
     GemmArgs g = {};
     g.p = p; g.q = q; g.sp = reinterpret_cast<const float*>(sp8); g.sq = reinterpret_cast<const float*>(sq8); g.out = out;
     g.Prows = Prows; g.Qrows = Qrows; g.red = red; g.ldo = Prows; g.sq_layout = 1; g.group = GROUP_CONTIG; g.E = E;
-    g.m_indices = m_indices; g.ldsq = ldsq; g.pair_list = pair_list; g.cus = pf8_effective_cus();
+    g.m_indices = m_indices; g.ldsq = ldsq; g.pair_list = pair_list; g.cus = cus;
     const int64_t T128 = (Prows / 256) * (Qrows / 128), per_xcd = (T128 + 7) / 8;
-    int64_t w = pf8_effective_cus() / 8;
+    int64_t w = cus / 8;
     if (w < 1) w = 1;
     if (w > per_xcd) w = per_xcd;
     hipLaunchKernelGGL((k_gemm_fwd_deep<1, 1>), dim3((unsigned)(8 * w)), dim3(256), 147456, stream, g);

@@ -465,7 +465,7 @@ using namespace pf8;
 
 static constexpr int E8_LDS_BYTES = 131072 + 4 * 16 * 272;
 
-static int launch_e8(const E8Args& a, int64_t max_q_tiles, hipStream_t st, const char* where) {
+static int launch_e8(const E8Args& a, int64_t max_q_tiles, int cus, hipStream_t st, const char* where) {
     // the LDS opt-in, once per device (a bit per device; a race sets the same attribute twice)
     static std::atomic<uint64_t> attr_done{0};
     int dev = 0;
@@ -478,7 +478,7 @@ static int launch_e8(const E8Args& a, int64_t max_q_tiles, hipStream_t st, const
         attr_done.fetch_or(bit, std::memory_order_release);
     }
     const int64_t T = ((a.Prows + 255) / 256) * max_q_tiles, per_xcd = (T + 7) / 8;
-    int64_t w = pf8_effective_cus() / 8;
+    int64_t w = cus / 8;
     if (w < 1) w = 1;
     if (w > per_xcd) w = per_xcd;
     hipLaunchKernelGGL(k_gemm_e8, dim3((unsigned)(8 * w)), dim3(256), E8_LDS_BYTES, st, a);
@@ -508,7 +508,7 @@ extern "C" int pf8_gemm_nt_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ld
     E8Args g = {};
     g.p = b; g.q = a; g.sp8 = sb; g.sq8 = sa; g.out = out;
     g.Prows = N; g.Qrows = M; g.red = K; g.ldo = ldo; g.ldsq = ldsa; g.grouped = 0;
-    return launch_e8(g, (M + 255) / 256, (hipStream_t)stream, __func__);
+    return launch_e8(g, (M + 255) / 256, pf8_effective_cus(), (hipStream_t)stream, __func__);
 }
 
 extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b,
@@ -526,18 +526,21 @@ extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint
     E8Args g = {};
     g.p = b; g.q = a; g.sp8 = sb; g.sq8 = sa; g.out = out;
     g.Prows = N; g.Qrows = Mtot; g.red = K; g.ldo = N; g.ldsq = ldsa; g.grouped = 1; g.m_indices = m_indices;
+    // the compute-unit budget is read once: both launches size their grids by it and both kernels weigh
+    // the expert load with it, so a pf8_set_num_cus from another thread cannot make them disagree
+    const int cus = pf8_effective_cus();
     if (items) {
         // both kernels are launched; each decides on entry, from the list's header, whether this expert
         // load is its own, and the other returns at once
         PF8_REQUIRE((reinterpret_cast<uintptr_t>(items) & 15u) == 0, "items must be 16-byte aligned");
         g.items = items;
-        g.cus = pf8_effective_cus();
+        g.cus = cus;
         g.force = N % 256 != 0;      // the 128x256-tile kernel takes whole 256-column tiles only
-        rc = launch_e8(g, Mtot / 128, (hipStream_t)stream, __func__);
+        rc = launch_e8(g, Mtot / 128, cus, (hipStream_t)stream, __func__);
         if (rc || g.force) return rc;
-        return pf8_launch_deep_ue8m0(b, a, sb, sa, ldsa, out, N, Mtot, K, E, m_indices, items, (hipStream_t)stream, __func__);
+        return pf8_launch_deep_ue8m0(b, a, sb, sa, ldsa, out, N, Mtot, K, E, m_indices, items, cus, (hipStream_t)stream, __func__);
     }
-    return launch_e8(g, (Mtot + 255) / 256, (hipStream_t)stream, __func__);
+    return launch_e8(g, (Mtot + 255) / 256, cus, (hipStream_t)stream, __func__);
 }
 
 extern "C" int pf8_grouped_items_build(const int32_t* m_indices, int64_t Mtot, int32_t* items, pf8_stream_t stream) {

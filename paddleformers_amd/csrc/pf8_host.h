@@ -5,18 +5,22 @@
 #include <stdint.h>
 
 #include "../../include/pf8.h"
+#include "../../include/pf8_selftest.h"
 
 // records the message for pf8_last_error() and returns `code`
 int pf8_fail(int code, const char* where, const char* msg);
 // hipGetLastError() -> PF8_OK or PF8_ELAUNCH (message recorded)
 int pf8_check_launch(const char* where);
-// compute units the GEMM grids may assume (pf8_set_num_cus, 0 = whole device)
+// compute units the GEMM grids may assume on the current device (pf8_set_num_cus, 0 = whole device)
 int pf8_effective_cus();
+// true when pf8_set_num_cus holds a budget below the current device's compute units
+bool pf8_cus_capped();
 
 // Launches the 128x256 persistent forward kernel on a contiguous-grouped GEMM whose scales are UE8M0
 // bytes (implemented next to that kernel; used by the UE8M0 entry point when a skewed expert load
 // makes 256-row tiles wasteful).  pair_list: DEVICE work-item list of the paired-tile kernel; this kernel
-// returns at once when that one takes the call (e8_paired_tiles_win).
+// returns at once when that one takes the call (e8_paired_tiles_win).  cus: the compute-unit budget, read ONCE by
+// the caller for both launches so that they reach the same verdict.
 int pf8_launch_deep_ue8m0(const uint8_t* p, const uint8_t* q, const uint8_t* sp8, const uint8_t* sq8, int64_t ldsq, void* out,
                           int64_t Prows, int64_t Qrows, int64_t red, int E, const int32_t* m_indices, const int32_t* pair_list,
-                          hipStream_t stream, const char* where);
+                          int cus, hipStream_t stream, const char* where);

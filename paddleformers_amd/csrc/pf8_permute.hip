@@ -19,7 +19,8 @@ struct PermuteArgs {
 template <int TOPK>   // compile-time top-k (a multiple of 4: the routing row is read as 16-byte words), 0 = generic
 __global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restrict__ routemap, int64_t T, int topk, PermuteArgs pa,
                                                         int32_t* __restrict__ rowmap, float* __restrict__ out_probs,
-                                                        int32_t* __restrict__ overflow) {
+                                                        int32_t* __restrict__ overflow, uint8_t* __restrict__ out_x, int64_t row_bytes,
+                                                        float* __restrict__ out_xs, int64_t scale_cols) {
     // every thread ranks J tokens per step (token = step base + j * 1024 + tid, so rank order is
     // j-major): the J x topk loads of a step are in flight together and a step costs one barrier
     constexpr int J = 4;
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restri
             const int64_t t = t0 + j * 1024 + tid;
             if (t < T) {
                 int64_t row = hit[j] ? base + before : -1;
-                if (row >= limit) { row = -1; *overflow = 1; }      // more routed rows than tokens_per_expert says
+                if (row >= limit) { row = -1; atomicOr(overflow, 1); }      // more routed rows than tokens_per_expert says
                 rowmap[t * E + e] = (int32_t)row;
             }
             base += total;
@@ -74,6 +75,18 @@ __global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restri
     }
     if (out_probs)
         for (int64_t r = limit + tid; r < pa.row_start[e + 1]; r += 1024) out_probs[r] = 0.0f;
+    // fewer routed rows than tokens_per_expert says: rows [base, limit) receive no token.  They are
+    // flagged and cleared here, so that nothing uninitialised flows into the quantizers and GEMMs.
+    if (base < limit) {
+        if (tid == 0) atomicOr(overflow, 2);
+        for (int64_t r = base; r < limit; ++r) {
+            uint4* dst = reinterpret_cast<uint4*>(out_x + r * row_bytes);
+            for (int64_t i = tid; i < row_bytes / 16; i += 1024) dst[i] = make_uint4(0, 0, 0, 0);
+            if (out_xs)
+                for (int64_t i = tid; i < scale_cols; i += 1024) out_xs[r * scale_cols + i] = 0.0f;
+            if (out_probs && tid == 0) out_probs[r] = 0.0f;
+        }
+    }
 }
 
 // One workgroup per padding row: zero the row of tokens (and of scales).
@@ -195,9 +208,10 @@ extern "C" int pf8_moe_permute(const void* x, int x_is_fp8, const float* xs, con
     hipStream_t st = (hipStream_t)stream;
     const int64_t scale_cols = xs ? H / 128 : 0;
     const bool rm16 = (reinterpret_cast<uintptr_t>(routemap) & 15u) == 0;
-    if (topk == 8 && rm16) hipLaunchKernelGGL(k_permute_rowmap<8>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
-    else if (topk == 4 && rm16) hipLaunchKernelGGL(k_permute_rowmap<4>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
-    else hipLaunchKernelGGL(k_permute_rowmap<0>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow);
+    // (the row-map kernel also clears the rows of an expert whose count overstates its routed tokens)
+    if (topk == 8 && rm16) hipLaunchKernelGGL(k_permute_rowmap<8>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow, (uint8_t*)out_x, row_bytes, out_xs, scale_cols);
+    else if (topk == 4 && rm16) hipLaunchKernelGGL(k_permute_rowmap<4>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow, (uint8_t*)out_x, row_bytes, out_xs, scale_cols);
+    else hipLaunchKernelGGL(k_permute_rowmap<0>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow, (uint8_t*)out_x, row_bytes, out_xs, scale_cols);
     int rc = pf8_check_launch(__func__);
     if (rc) return rc;
     if (max_pad > 0 && row_bytes > 0) {

@@ -67,7 +67,7 @@ def _ue8m0_kernel_shape(M: int, N: int, K: int, experts: int = 0) -> bool:
     if not (M % 128 == 0 and N % 128 == 0 and N >= 256 and K % 128 == 0 and K >= 384):
         return False
     if experts and N % 256 != 0:
-        cus = get_num_sms() or 256
+        cus = int(_lib.lib().pf8_effective_num_cus())
         p_tiles = (N + 255) // 256
         rounds_pair = -(-(M // 256 + experts) * p_tiles // cus)
         rounds_128 = -(-(M // 128) * p_tiles // cus)

@@ -588,7 +588,8 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
     expert_routemap_topk int32 [T, topk] (negative = unused slot); expert_prob_topk fp32 [T, topk].
     Returns (hidden_states_unzipped [Mpad, H], zipped_expertwise_rowmap int32 [T, num_experts],
     token_prob_unzipped fp32 [Mpad, 1], scale_unzipped fp32 [Mpad, H/128] or None).
-    A token routed to an expert beyond its `tokens_per_expert` count raises ValueError; that check
+    Counts that do not match the routing raise ValueError (a token routed to an expert beyond its
+    `tokens_per_expert` count is dropped; rows of an overstated count are written as zeros); that check
     reads a flag back from the device (one synchronisation), `validate=False` skips it.
     """
     if not do_gather:
@@ -627,8 +628,12 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
     cnt = (C.c_int64 * num_experts)(*counts)
     _lib.call("pf8_moe_permute", _p(x), int(is_fp8), _p(xs), _p(rm), _p(pr), T, H, topk, num_experts, cnt, a, _p(out_x), _p(rowmap),
               _p(out_p), _p(out_s), _p(overflow), _stream())
-    if validate and int(overflow.item()):
-        raise ValueError("expert_routemap_topk routes more tokens to an expert than tokens_per_expert allows")
+    if validate:
+        flags = int(overflow.item())
+        if flags & 1:
+            raise ValueError("expert_routemap_topk routes more tokens to an expert than tokens_per_expert allows")
+        if flags & 2:
+            raise ValueError("expert_routemap_topk routes fewer tokens to an expert than tokens_per_expert says")
     return out_x, rowmap, out_p, out_s
 
 

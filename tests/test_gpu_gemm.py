@@ -203,6 +203,66 @@ def test_grouped_contiguous_equals_per_expert_loop(dg, rows, lay):
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
 
 
+@pytest.fixture
+def few_cus(dg):
+    """A budget of eight compute units (deep_gemm.set_num_sms): the persistent kernel runs one workgroup per
+    XCD and the two-workgroup kernel sixteen workgroups, each walking several tiles."""
+    dg.set_num_sms(8)
+    yield
+    dg.set_num_sms(0)
+
+
+# K = 2048 with whole 256-column tiles: the persistent kernel, whose copy ring, next-tile scalar loads and
+# hand-counted waits run across 3-4 tile boundaries per workgroup; K = 512 or N = 384: the two-workgroup
+# kernel walking its XCD's run of tiles in strides
+@pytest.mark.parametrize("K,N", [(2048, 512), (512, 768), (1024, 384)])
+@pytest.mark.parametrize("rows", [[256, 0, 640, 128, 384, 512], [128] * 9 + [0, 768]])
+@pytest.mark.parametrize("lay", [0, 1])
+def test_grouped_contiguous_under_a_compute_unit_budget(dg, few_cus, K, N, rows, lay):
+    E = len(rows)
+    a, sa, b, sb, m_idx = _grouped_case(E, N, K, rows, seed=sum(rows) + K + N)
+    Mtot = a.shape[0]
+    tsa = torch.from_numpy(np.ascontiguousarray(sa.T)).cuda().t() if lay else torch.from_numpy(sa).cuda()
+    out = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dg.m_grouped_fp8_gemm_nt_contiguous((G.to_torch_fp8(a), tsa), (G.to_torch_fp8(b), torch.from_numpy(sb).cuda()), out,
+                                        torch.from_numpy(m_idx).cuda())
+    got = G.from_torch_bf16(out)
+    exp = O.grouped_gemm_nt_contiguous(a, sa, b, sb, m_idx)
+    assert G.rel_fro(_bf(got), _bf(exp)) <= BLOCK_FRO
+    start = 0
+    for e, r in enumerate(rows):
+        if r:
+            _elementwise_ok(_bf(got[start:start + r]), a[start:start + r], sa[start:start + r], b[e], sb[e], 0, f"expert {e}")
+        start += r
+
+
+def test_dense_and_masked_gemm_under_a_compute_unit_budget(dg, few_cus):
+    """The same budget on the dense call (32 tiles on 16 workgroups) and on the masked layout."""
+    M, N, K = 1024, 1024, 512
+    xa = G.bf16_normal((M, K), seed=71)
+    a, sa = _quant_act(xa, 0)
+    b, sb = _quant_w(G.bf16_normal((N, K), seed=72, std=0.02))
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dg.fp8_gemm_nt((G.to_torch_fp8(a), torch.from_numpy(sa).cuda()), (G.to_torch_fp8(b), torch.from_numpy(sb).cuda()), out)
+    _check(G.from_torch_bf16(out), a, sa, b, sb, "dense under a budget")
+    E, Mmax = 3, 512
+    masked = np.array([300, 0, 512], dtype=np.int32)
+    am = np.stack([_quant_act(G.bf16_normal((Mmax, K), seed=80 + e), 0)[0] for e in range(E)])
+    sam = np.stack([_quant_act(G.bf16_normal((Mmax, K), seed=80 + e), 0)[1] for e in range(E)])
+    bm = np.stack([_quant_w(G.bf16_normal((N, K), seed=90 + e, std=0.02))[0] for e in range(E)])
+    sbm = np.stack([_quant_w(G.bf16_normal((N, K), seed=90 + e, std=0.02))[1] for e in range(E)])
+    outm = torch.full((E, Mmax, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    dg.m_grouped_fp8_gemm_nt_masked((G.to_torch_fp8(am), torch.from_numpy(sam).cuda()), (G.to_torch_fp8(bm), torch.from_numpy(sbm).cuda()),
+                                    outm, torch.from_numpy(masked).cuda(), 300)
+    exp = O.grouped_gemm_nt_masked(am, sam, bm, sbm, masked)
+    got = G.from_torch_bf16(outm)
+    for e in range(E):
+        v = int(masked[e])
+        if v:
+            assert G.rel_fro(_bf(got[e, :v]), _bf(exp[e, :v])) <= BLOCK_FRO
+        assert (outm[e, v:] == 7.0).all()
+
+
 def test_grouped_contiguous_negative_index_skips_tile(dg):
     E, N, K = 2, 128, 256
     rows = [128, 128]
@@ -336,6 +396,11 @@ def test_grouped_wgrad_equals_per_expert_loop(dg):
     out0 = torch.full_like(base, float("nan"))
     F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, out0, accumulate=False)
     assert torch.equal(out0[1], torch.zeros_like(out0[1]))
+    # the grouped launch straight against the oracle's weight-gradient GEMM, expert by expert
+    for e, r in enumerate(rows):
+        if r:
+            exp = O.gemm_nt_1d1d_f32(G.from_torch_fp8(a_t[e]), sa_t[e].cpu().numpy(), G.from_torch_fp8(b_t[e]), sb_t[e].cpu().numpy())
+            assert G.rel_fro(out0[e].cpu().numpy(), exp) <= F32_FRO, f"expert {e} vs oracle"
     assert torch.allclose(out0[0], out[0] - base[0], rtol=1e-4, atol=1e-6)
     # the operands carry power-of-two scales (pow_2_scales=True above): scales inside the MFMA give the
     # same gradients, grouped launch and per-expert launches bit for bit
@@ -349,3 +414,9 @@ def test_grouped_wgrad_equals_per_expert_loop(dg):
         F8.fp8_gemm_blockwise(a=a_t[e], a_decode_scale=sa_t[e], b=b_t[e], b_decode_scale=sb_t[e], out=ref, accumulate=True, scales_pow2=True)
         assert torch.equal(outp[e], ref), f"expert {e}"
         assert G.rel_fro((outp[e] - base[e]).cpu().numpy(), (out[e] - base[e]).cpu().numpy()) <= 1e-4
+    outp0 = torch.full_like(base, float("nan"))
+    F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, outp0, accumulate=False, scales_pow2=True)
+    for e, r in enumerate(rows):
+        if r:
+            exp = O.gemm_nt_1d1d_f32(G.from_torch_fp8(a_t[e]), sa_t[e].cpu().numpy(), G.from_torch_fp8(b_t[e]), sb_t[e].cpu().numpy())
+            assert G.rel_fro(outp0[e].cpu().numpy(), exp) <= F32_FRO_MFMA_ACC, f"expert {e} vs oracle (scales inside the MFMA)"

@@ -213,6 +213,27 @@ def test_grouped_contiguous_ue8m0_vs_oracle(dg, request, rows, paired, cus):
         start += r
 
 
+# Sixteen K blocks and eight compute units: every persistent workgroup (paired 256-row tiles, and the 128-row-tile
+# kernel the list header may hand the call to) runs its copy ring across several tile boundaries, and the aligned
+# walk without a list makes a second pass over the tiles in which two experts meet.
+@pytest.mark.parametrize("rows", [[256, 0, 640, 128, 384, 512], [128] * 9 + [0, 768], [1024, 896]])
+@pytest.mark.parametrize("paired", [True, False])
+def test_grouped_contiguous_ue8m0_long_reduction_few_compute_units(dg, few_cus, rows, paired):
+    E, N, K = len(rows), 512, 2048
+    a, sa, b, sb, m_idx = _grouped_pow2_case(E, N, K, rows, seed=sum(rows) + 7 * E)
+    Mtot = a.shape[0]
+    out = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    _grouped_call(dg, a, sa, b, sb, m_idx, out, paired)
+    exp = O.grouped_gemm_nt_contiguous(a, sa, b, sb, m_idx)
+    got = G.from_torch_bf16(out)
+    assert G.rel_fro(_bf(got), _bf(exp)) <= BLOCK_FRO
+    start = 0
+    for e, r in enumerate(rows):
+        if r:
+            _elementwise_ok(_bf(got[start:start + r]), a[start:start + r], sa[start:start + r], b[e], sb[e], f"expert {e}")
+        start += r
+
+
 # 640 = two column tiles and a half: the wavefronts of the missing half compute on a copy of the first and
 # store nothing.  Through the raw C ABI, so that the block-scaled kernel runs whatever the load: with a
 # work-item list (paired 256-row tiles) and without (aligned tiles, two passes where experts meet).
@@ -365,7 +386,7 @@ def test_ue8m0_grouped_gemm_at_config5_size_agrees_with_the_fp32_scale_kernel(dg
     """128 experts with a Zipf(1.0) load over 131072 routed rows (segments of 2..190 blocks, 1083 blocks in
     all): here the cost estimate picks the paired 256-row tiles on the whole device, and the list builder
     walks two blocks per thread."""
-    from bench import zipf_counts
+    zipf_counts = G.zipf_counts
     from paddleformers_amd import deep_gemm as DG
     from paddleformers_amd import functional as F
 

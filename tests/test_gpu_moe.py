@@ -313,3 +313,132 @@ def test_moe_node_backward_fused_gradient_quantization_is_bit_identical(ue8m0):
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
     for ga, gb in zip(a[2] + a[3], b[2] + b[3]):
         assert torch.equal(ga, gb)
+
+
+# ---------------------------------------------------------------------------------------------
+# sub-batched forward / backward and deferred weight gradients
+# ---------------------------------------------------------------------------------------------
+
+
+def _split_list_prefix(counts, start, end):
+    """Rows of every expert that fall into [start, end): what the caller hands to a sub-batch
+    (cli/train/deepseek_v3_pretrain/moe_layer.py:838-851)."""
+    out, off = [], 0
+    for c in counts:
+        out.append(max(0, min(end, off + c) - max(start, off)))
+        off += c
+    return out
+
+
+@pytest.mark.parametrize("ue8m0", [False, True])
+def test_moe_node_subbatches_equal_the_one_shot_node(ue8m0):
+    """The caller's sub-batch loops (moe_layer.py:791-884, 936-982, 1054-1103): the quantised input is cut
+    into slices of a multiple of 128 rows that straddle experts, each slice goes through forward / backward
+    with its own m_indices slice.  Outputs, dx and probs_grad equal the one-shot node bit for bit; the fp32
+    weight gradients are sums split differently, so they agree to rounding."""
+    from paddleformers_amd import functional as F8
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
+
+    E, H, I = 4, 512, 384
+    rows = [384, 0, 256, 640]
+    M = sum(rows)
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=41)
+    dout = G.to_torch_bf16(G.bf16_normal((M, H), seed=43, std=1e-3))
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    xq, xs = F8.fp8_quant_blockwise(G.to_torch_bf16(x), quant_method="1x128", output_scale_transpose=False, using_pow2_scale=ue8m0)
+
+    def fresh_grads():
+        for ex in experts:
+            ex.w1.main_grad = torch.zeros_like(ex.w1, dtype=torch.float32)
+            ex.w2.main_grad = torch.zeros_like(ex.w2, dtype=torch.float32)
+
+    # one shot
+    fresh_grads()
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts), recompute_fwd_gate_up=True, use_ue8m0=ue8m0)
+    o3_ref = node.forward((xq, xs), tp, rows)
+    dx_ref, pg_ref = node.backward(dout, tp, rows)
+    g_ref = [(ex.w1.main_grad.clone(), ex.w2.main_grad.clone()) for ex in experts]
+
+    # sub-batched: 512-row slices (the last one 256), cutting through experts 0, 2 and 3
+    fresh_grads()
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts), recompute_fwd_gate_up=True, use_ue8m0=ue8m0)
+    m_indices = node.gen_m_indices(rows)
+    node.input_fp8, node.input_scale = xq, xs          # prepare_env_subbatch, moe_layer.py:774-780
+    node.fwd_subbatch = True
+    step = 512
+    parts = [(s, min(s + step, M)) for s in range(0, M, step)]
+    outs = [node.forward((xq[s:e], xs[s:e]), tp[s:e], rows, m_indices=m_indices[s:e]) for s, e in parts]
+    assert torch.equal(torch.cat(outs).view(torch.int16), o3_ref.view(torch.int16))
+    node.bwd_subbatch = True
+    dxs, pgs = [], []
+    for i, (s, e) in enumerate(parts):
+        dx, pg = node.backward(dout[s:e].contiguous(), tp[s:e].contiguous(), _split_list_prefix(rows, s, e),
+                               input_fp8_slice=xq[s:e].contiguous(), input_scale_slice=xs[s:e].contiguous(),
+                               m_indices=m_indices[s:e].contiguous(), reset_status=i == len(parts) - 1)
+        dxs.append(dx)
+        pgs.append(pg)
+    assert torch.equal(torch.cat(dxs).view(torch.int16), dx_ref.view(torch.int16))
+    assert torch.equal(torch.cat(pgs), pg_ref)
+    assert node.input_fp8 is None and node.m_indices is None        # the last part released the saved state
+    for ex, (r1, r2) in zip(experts, g_ref):
+        assert G.rel_fro(ex.w1.main_grad.cpu().numpy(), r1.cpu().numpy()) <= 5e-5 or not r1.any()
+        assert G.rel_fro(ex.w2.main_grad.cpu().numpy(), r2.cpu().numpy()) <= 5e-5 or not r2.any()
+        assert ex.w1.main_grad.any() == r1.any()
+
+
+@pytest.mark.parametrize("stacked", [False, True])
+def test_moe_node_deferred_weight_gradients_run_at_flush_on_another_stream(stacked):
+    """WeightGradStore.enabled (zero-bubble pipeline, fp8_utils.py:314-327): backward queues the weight-gradient
+    closures and returns; flush() runs them later, here on a second stream after the activations the node
+    held have been dropped.  main_grad ends up bit-identical to the immediate run."""
+    from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode, WeightGradStore
+
+    E, H, I = 3, 512, 256
+    rows = [256, 0, 384]
+    w1, w2, experts, x, probs = _make(E, H, I, rows, seed=51)
+    dout = G.to_torch_bf16(G.bf16_normal((sum(rows), H), seed=53, std=1e-3))
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+
+    def fresh_grads():
+        if stacked:
+            g1 = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
+            g2 = torch.zeros((E, I, H), dtype=torch.float32, device="cuda")
+            for e, ex in enumerate(experts):
+                ex.w1.main_grad, ex.w2.main_grad = g1[e], g2[e]
+        else:
+            for ex in experts:
+                ex.w1.main_grad = torch.zeros_like(ex.w1, dtype=torch.float32)
+                ex.w2.main_grad = torch.zeros_like(ex.w2, dtype=torch.float32)
+
+    fresh_grads()
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts))
+    node.forward(G.to_torch_bf16(x), tp, rows)
+    dx_ref, pg_ref = node.backward(dout, tp, rows)
+    ref = [(ex.w1.main_grad.clone(), ex.w2.main_grad.clone()) for ex in experts]
+
+    fresh_grads()
+    node = FP8GroupGemmMlpFunctionNode(_Map(experts))
+    node.forward(G.to_torch_bf16(x), tp, rows)
+    WeightGradStore.clear()
+    WeightGradStore.enabled = True
+    try:
+        dx, pg = node.backward(dout, tp, rows, reset_status=True)
+    finally:
+        WeightGradStore.enabled = False
+    assert torch.equal(dx, dx_ref) and torch.equal(pg, pg_ref)
+    for ex in experts:
+        assert not ex.w1.main_grad.any() and not ex.w2.main_grad.any()      # nothing has run yet
+    assert len(WeightGradStore._queue) == 2
+    # unrelated work reuses the allocator's freed blocks before the closures run
+    junk = [torch.randn((sum(rows), H), device="cuda") for _ in range(8)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        WeightGradStore.flush()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    del junk
+    assert not WeightGradStore._queue
+    for e, (ex, (r1, r2)) in enumerate(zip(experts, ref)):
+        assert torch.equal(ex.w1.main_grad, r1) and torch.equal(ex.w2.main_grad, r2), f"expert {e}"
+        assert bool(r1.any()) == (rows[e] > 0)

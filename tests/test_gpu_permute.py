@@ -97,6 +97,19 @@ def test_permute_rejects_inconsistent_counts_and_bad_arguments(F):
     short[int(np.argmax(counts))] -= 1
     with pytest.raises(ValueError, match="tokens_per_expert"):
         F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, short, 128)
+    # a count that overstates what the routing sends: flagged, and with the check skipped the rows no token
+    # lands on hold zeros (probability 0), like padding rows, not whatever the allocation held
+    big = int(np.argmax(counts))
+    over = list(counts)
+    over[big] += 3
+    with pytest.raises(ValueError, match="fewer tokens"):
+        F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, over, 128)
+    torch.full((E * 256, H), float("nan"), dtype=torch.bfloat16, device="cuda")     # poison what the allocator hands out next
+    ox, orow, op, _ = F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, over, 128, validate=False)
+    start = sum((c + 127) // 128 * 128 for c in over[:big])
+    assert not ox[start + counts[big]:start + over[big]].any() and not op[start + counts[big]:start + over[big]].any()
+    gx, _, gp, _ = F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, counts, 128)
+    assert torch.equal(ox[start:start + counts[big]], gx[start:start + counts[big]])
     with pytest.raises(ValueError):
         F.moe_permute(x, None, torch.from_numpy(rm).cuda(), None, E, counts[:-1], 128)
     with pytest.raises(RuntimeError):
