@@ -228,6 +228,21 @@ int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint8_t* sa, in
 int pf8_grouped_items_build(const int32_t* m_indices, int64_t Mtot, int32_t* items,
                             pf8_stream_t stream);
 
+/* pf8_grouped_gemm_nt_contiguous_ue8m0 for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments without `items`: the work-item list is built by the call itself, on `stream`, into a
+ * 131,088-byte array that is part of the library's device image (one copy per GPU, held until the process
+ * ends), and the GEMM then runs exactly as with a caller-built list, so `out` is bit-identical to
+ * pf8_grouped_items_build + pf8_grouped_gemm_nt_contiguous_ue8m0.  The call allocates and frees nothing.
+ * Mtot is limited to 1,048,576 rows (PF8_EINVAL beyond).  All calls on one GPU share that array: calls
+ * that may overlap on one GPU (different streams, different threads) race on it and must be serialised
+ * by the caller.  The first call on a device looks the array's address up (hipGetSymbolAddress); make
+ * that call outside any stream capture. */
+int pf8_grouped_gemm_nt_contiguous_ue8m0_noalloc(const uint8_t* a, const uint8_t* sa, int64_t ldsa,
+                                                 const uint8_t* b, const uint8_t* sb, int E, int64_t Mtot,
+                                                 int64_t N, int64_t K, const int32_t* m_indices,
+                                                 uint16_t* out, pf8_stream_t stream);
+
 /* fp32 scales that are powers of two -> UE8M0 exponent bytes, elementwise (any layout).  not_pow2,
  * when non-null, is a DEVICE int the kernel adds the number of scales to that are negative, zero,
  * non-finite or not a power of two (the caller zeroes it).  Scale side of `use_ue8m0`

@@ -543,6 +543,52 @@ extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0(const uint8_t* a, const uint
     return launch_e8(g, (Mtot + 255) / 256, cus, (hipStream_t)stream, __func__);
 }
 
+// ---------------------------------------------------------------------------------------------
+// The grouped UE8M0 GEMM for callers that cannot allocate: the work-item list lives in a file-scope
+// device array instead of a caller buffer.  Every GPU holds its own copy of the array at its own
+// address; the name `scratch` is only a host-side handle for hipGetSymbolAddress, which is asked once
+// per device (with that device current) and whose answer is what every launch passes on.
+// ---------------------------------------------------------------------------------------------
+static constexpr int64_t NOALLOC_MAX_BLOCKS = 8192;                 // 128-row blocks: 1,048,576 rows
+static __device__ __align__(256) int32_t scratch[4 + 4 * NOALLOC_MAX_BLOCKS];    // 131,088 bytes per GPU, held until the process ends
+
+static int noalloc_scratch(const char* where, int32_t** out) {
+    static std::atomic<int32_t*> ptrs[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, where, hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return pf8_fail(PF8_EINVAL, where, "device ordinal beyond 63");
+    int32_t* p = ptrs[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* sym = nullptr;
+        e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !sym) return pf8_fail(PF8_ELAUNCH, where, e != hipSuccess ? hipGetErrorString(e) : "hipGetSymbolAddress returned a null address");
+        p = static_cast<int32_t*>(sym);
+        ptrs[dev].store(p, std::memory_order_release);     // two threads racing here store the same address
+    }
+    *out = p;
+    return PF8_OK;
+}
+
+extern "C" int pf8_grouped_gemm_nt_contiguous_ue8m0_noalloc(const uint8_t* a, const uint8_t* sa, int64_t ldsa, const uint8_t* b,
+                                                            const uint8_t* sb, int E, int64_t Mtot, int64_t N, int64_t K,
+                                                            const int32_t* m_indices, uint16_t* out, pf8_stream_t stream) {
+    PF8_REQUIRE(Mtot >= 0 && Mtot % 128 == 0, "Mtot must be a non-negative multiple of 128");
+    PF8_REQUIRE(Mtot / 128 <= NOALLOC_MAX_BLOCKS, "Mtot beyond the 1,048,576 rows the built-in work-item list holds: build a list with pf8_grouped_items_build and call pf8_grouped_gemm_nt_contiguous_ue8m0");
+    if (Mtot == 0 || N == 0 || E == 0) return pf8_grouped_gemm_nt_contiguous_ue8m0(a, sa, ldsa, b, sb, E, Mtot, N, K, m_indices, nullptr, out, stream);
+    PF8_REQUIRE(m_indices, "null pointer");
+    int32_t* items = nullptr;
+    int rc = noalloc_scratch(__func__, &items);
+    if (rc) return rc;
+    // the list builder writes the header and every field of every item it counts, and the GEMM reads
+    // no further than that count: nothing in the array has to start at zero, stale items of an earlier,
+    // longer call are never looked at
+    hipLaunchKernelGGL(k_e8_build_items, dim3(1), dim3(1024), 0, (hipStream_t)stream, m_indices, Mtot / 128, items);
+    rc = pf8_check_launch(__func__);
+    if (rc) return rc;
+    return pf8_grouped_gemm_nt_contiguous_ue8m0(a, sa, ldsa, b, sb, E, Mtot, N, K, m_indices, items, out, stream);
+}
+
 extern "C" int pf8_grouped_items_build(const int32_t* m_indices, int64_t Mtot, int32_t* items, pf8_stream_t stream) {
     PF8_REQUIRE(Mtot >= 0 && Mtot % 128 == 0, "Mtot must be a non-negative multiple of 128");
     PF8_REQUIRE(items && (reinterpret_cast<uintptr_t>(items) & 15u) == 0, "items must be a 16-byte aligned buffer");
