@@ -26,12 +26,30 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 FP8_PEAK_TFLOPS = 5000.0
-# HBM bytes one launch of the up+gate grouped GEMM moves on this workload, from two rocprofv3 --pmc
-# runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
-# counter reads for the 1 GiB pf8::k_debug_copy launched with --copy-yardstick (FETCH_SIZE reads
-# 0.5 KiB per KiB copied -> factor 2.0; WRITE_SIZE reads 1.0 -> factor 1.0):
-#   868,055 KiB x 2.0 + 79,872 KiB x 1.0 = 1,815,982 KiB.   Summary: profiles/gemm_up_gate_config3_hbm_traffic.md
-GEMM_UP_GATE_TRAFFIC_BYTES = 1815982 * 1024
+# roofline.traffic is not something this run can measure (hardware counters need the profiler): it is
+# read from the committed summary of two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE,
+# KiB per dispatch, each scaled by what the same counter reads for the 1 GiB pf8::k_debug_copy launched
+# with --copy-yardstick).  The summary names the kernel it was taken on; when that is not the kernel this
+# run times, traffic is reported as null rather than as a stale figure.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gemm_up_gate_config3_hbm_traffic.md")
+
+
+def traffic_from_summary(kernel_name):
+    """HBM bytes per launch of `kernel_name` from the machine-readable line of the traffic summary
+    (`traffic-json: {...}`), or None when the summary is missing or belongs to another kernel."""
+    try:
+        for line in open(TRAFFIC_SUMMARY):
+            if line.startswith("traffic-json:"):
+                rec = json.loads(line[len("traffic-json:"):])
+                if rec.get("kernel") == kernel_name:
+                    return int(rec["bytes_per_launch"]), rec
+    except (OSError, ValueError, KeyError):
+        pass
+    return None, None
+
+
+# the kernel the up+gate grouped GEMM of the headline workload runs on (what rocprofv3 --kernel-trace names it)
+ROOFLINE_KERNEL = "pf8::k_gemm_fwd_deep<1, 0>"
 
 
 def zipf_counts(total, E, s, seed, n_empty=2, pad=128):
@@ -49,27 +67,54 @@ def zipf_counts(total, E, s, seed, n_empty=2, pad=128):
     return counts.astype(np.int64), (((counts + pad - 1) // pad) * pad).astype(np.int64)
 
 
-def time_kernel(fn, sets, iters, warmup):
-    """Median-free average time (ms) of fn(*sets[i % len(sets)]) over `iters` launches, with
-    HIP events on the launch stream."""
+def time_kernel(fn, sets, iters=50, warmup=10, batches=10):
+    """Times fn(*sets[i % len(sets)]) after `warmup` untimed launches: `batches` batches of back-to-back
+    launches (at least `iters` launches in all), one HIP event pair on the launch stream around each batch,
+    so that no event sits between two launches (recording one costs about 6 us of idle stream on this
+    machine, a third of the smaller kernels here).  Returns the median and the minimum over the batches of
+    the time per launch, and the mean over all launches, in ms; legs report the median."""
     import torch
 
+    per = max(1, -(-iters // batches))
     for i in range(warmup):
         fn(*sets[i % len(sets)])
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(iters):
-        fn(*sets[i % len(sets)])
-    e1.record()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(batches)]
+    k = warmup
+    for e0, e1 in ev:
+        e0.record()
+        for _ in range(per):
+            fn(*sets[k % len(sets)])
+            k += 1
+        e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    ts = sorted(e0.elapsed_time(e1) / per for e0, e1 in ev)
+    med = ts[batches // 2] if batches % 2 else 0.5 * (ts[batches // 2 - 1] + ts[batches // 2])
+    return {"ms": med, "ms_min": ts[0], "ms_mean": sum(ts) / batches, "launches": per * batches, "batches": batches}
 
 
-def bench_quantizers(iters=20, warmup=5):
-    """GB/s of the bandwidth-bound quantizers on BASELINE configs 1, 3 (SwiGLU) and 4.  Outputs are
-    pre-allocated and the C ABI is called directly, so the timed region holds kernels only; inputs
-    rotate over buffer sets larger than the 256 MB Infinity Cache."""
+def _finish(legs):
+    """bytes -> GB/s against the HBM peak, flop -> TFLOP/s against the dense FP8 peak (both on the median)."""
+    for v in legs.values():
+        if "flop" in v:
+            v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)
+            v["frac_fp8_peak"] = round(v["TFLOPs"] / FP8_PEAK_TFLOPS, 4)
+        else:
+            v["GBps"] = round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)
+            v["GBps_best"] = round(v["bytes"] / (v["ms_min"] * 1e-3) / 1e9, 1)
+            v["frac_hbm"] = round(v["GBps"] / HBM_PEAK_GBS, 4)
+        for k in ("ms", "ms_min", "ms_mean"):
+            if k in v:
+                v[k] = round(v[k], 5)
+    return legs
+
+
+def bench_quantizers(iters=60, warmup=10):
+    """GB/s of the bandwidth-bound quantizers on BASELINE configs 1, 3 (SwiGLU) and 4, with both scale rules,
+    next to a plain copy of matching size (the yardstick of what this memory system gives a kernel that
+    reads and writes once).  The C ABI is called directly on pre-allocated buffers, so the timed region
+    holds kernels only; inputs AND outputs rotate over buffer sets whose total exceeds the 256 MB Infinity
+    Cache several times, so neither reads nor write-allocations are served from it."""
     import ctypes as C
 
     import torch
@@ -80,8 +125,8 @@ def bench_quantizers(iters=20, warmup=5):
     vp = C.c_void_p
     st = vp(torch.cuda.current_stream().cuda_stream)
 
-    def mk(shape, n, std=1.0):
-        return [(torch.randn(shape, device="cuda", dtype=torch.float32) * std).to(torch.bfloat16) for _ in range(n)]
+    def bf(shape, std=1.0):
+        return (torch.randn(shape, device="cuda", dtype=torch.float32) * std).to(torch.bfloat16)
 
     def u8(*shape):
         return torch.empty(shape, dtype=torch.uint8, device="cuda")
@@ -89,48 +134,47 @@ def bench_quantizers(iters=20, warmup=5):
     def f32(*shape):
         return torch.empty(shape, dtype=torch.float32, device="cuda")
 
+    def p(t):
+        return vp(t.data_ptr()) if t is not None else None
+
+    def run(name, nbytes, nsets, make, call):
+        sets = [make() for _ in range(nsets)]
+        r = time_kernel(lambda *bufs: call(*bufs), sets, iters, warmup)
+        r["bytes"] = nbytes
+        r["buffer_sets"] = nsets
+        out[name] = r
+        del sets
+        torch.cuda.empty_cache()
+
+    # plain copies: the size of config 1's activation quantizer (89 MB moved) and of config 4's (477 MB)
+    for name, half in (("copy_yardstick_89MB", 44498944), ("copy_yardstick_477MB", 238551040)):
+        run(name, 2 * half, max(4, (1 << 30) // (2 * half)), lambda h=half: (u8(h).random_(0, 255), u8(h)),
+            lambda src, dst: _lib.call("pf8_debug_copy", p(src), p(dst), src.numel(), st))
     # C1a: 1x128 on [4096, 7168]
     M, K = 4096, 7168
-    xs, q, s = mk((M, K), 6), u8(M, K), f32(K // 128, M)
-    ms = time_kernel(lambda x: _lib.call("pf8_quant_1x128", vp(x.data_ptr()), M, K, K, vp(q.data_ptr()), vp(s.data_ptr()), 1, 0, st),
-                     [(x,) for x in xs], iters, warmup)
-    out["quant_1x128_4096x7168"] = {"bytes": 88997888, "ms": ms}
-    del xs, q, s
+    for pow2 in (0, 1):
+        run("quant_1x128_4096x7168" + ("_pow2" if pow2 else ""), 88997888, 8, lambda: (bf((M, K)), u8(M, K), f32(K // 128, M)),
+            lambda x, q, s_, pw=pow2: _lib.call("pf8_quant_1x128", p(x), M, K, K, p(q), p(s_), 1, pw, st))
     # C1b: 128x128 on [7168, 2048]
     R, Cc = 7168, 2048
-    ws, q, s = mk((R, Cc), 10, 0.02), u8(R, Cc), f32(R // 128, Cc // 128)
-    ms = time_kernel(lambda w: _lib.call("pf8_quant_128x128", vp(w.data_ptr()), R, Cc, vp(q.data_ptr()), vp(s.data_ptr()), None, None, 0, st),
-                     [(w,) for w in ws], iters, warmup)
-    out["quant_128x128_7168x2048"] = {"bytes": 44043776, "ms": ms}
-    del ws, q, s
+    for pow2 in (0, 1):
+        run("quant_128x128_7168x2048" + ("_pow2" if pow2 else ""), 44043776, 12, lambda: (bf((R, Cc), 0.02), u8(R, Cc), f32(R // 128, Cc // 128)),
+            lambda w, q, s_, pw=pow2: _lib.call("pf8_quant_128x128", p(w), R, Cc, p(q), p(s_), None, None, pw, st))
     # C3-q: fused SwiGLU + requant on [8192, 4096]
     M, I = 8192, 2048
-    os_, q, s = mk((M, 2 * I), 5), u8(M, I), f32(M, I // 128)
-    ms = time_kernel(lambda o: _lib.call("pf8_swiglu_weighted_quant", vp(o.data_ptr()), None, M, I, vp(q.data_ptr()), vp(s.data_ptr()), None, 0, 0, st),
-                     [(o,) for o in os_], iters, warmup)
-    out["swiglu_quant_8192x4096"] = {"bytes": 84443136 - 32768, "ms": ms}
-    ms = time_kernel(lambda o: _lib.call("pf8_swiglu_weighted_quant", vp(o.data_ptr()), None, M, I, vp(q.data_ptr()), vp(s.data_ptr()), None, 0, 1, st),
-                     [(o,) for o in os_], iters, warmup)
-    out["swiglu_quant_8192x4096_pow2"] = {"bytes": 84443136 - 32768, "ms": ms}
-    del os_, q, s
+    for pow2 in (0, 1):
+        run("swiglu_quant_8192x4096" + ("_pow2" if pow2 else ""), 84443136 - 32768, 8, lambda: (bf((M, 2 * I)), u8(M, I), f32(M, I // 128)),
+            lambda o, q, s_, pw=pow2: _lib.call("pf8_swiglu_weighted_quant", p(o), None, M, I, p(q), p(s_), None, 0, pw, st))
     # C4: fused quant + transpose on [16384, 7168]
     M, K = 16384, 7168
-    xs, q, s, qt, s2 = mk((M, K), 2), u8(M, K), f32(K // 128, M), u8(K, M), f32(M // 128, K)
-    ms = time_kernel(lambda x: _lib.call("pf8_quant_transpose", vp(x.data_ptr()), M, K, vp(q.data_ptr()), vp(s.data_ptr()), vp(qt.data_ptr()),
-                                         vp(s2.data_ptr()), 1, 0, st), [(x,) for x in xs], iters, warmup)
-    out["quant_transpose_16384x7168"] = {"bytes": 477102080, "ms": ms}
-    del xs, q, s, qt, s2
-    torch.cuda.empty_cache()
-    for v in out.values():
-        v["GBps"] = v["bytes"] / (v["ms"] * 1e-3) / 1e9
-        v["frac_hbm"] = v["GBps"] / HBM_PEAK_GBS
-        v["ms"] = round(v["ms"], 5)
-        v["GBps"] = round(v["GBps"], 1)
-        v["frac_hbm"] = round(v["frac_hbm"], 4)
-    return out
+    for pow2 in (0, 1):
+        run("quant_transpose_16384x7168" + ("_pow2" if pow2 else ""), 477102080, 3,
+            lambda: (bf((M, K)), u8(M, K), f32(K // 128, M), u8(K, M), f32(M // 128, K)),
+            lambda x, q, s_, qt, s2, pw=pow2: _lib.call("pf8_quant_transpose", p(x), M, K, p(q), p(s_), p(qt), p(s2), 1, pw, st))
+    return _finish(out)
 
 
-def bench_other_gemms(iters=10, warmup=3):
+def bench_other_gemms(iters=50, warmup=10):
     """Kernel-only timings of the other BASELINE GEMM workloads (random e4m3 bytes and scales):
     config 2 dense, config 5 forward grouped GEMMs and the config-5 weight gradient."""
     import numpy as np
@@ -139,95 +183,107 @@ def bench_other_gemms(iters=10, warmup=3):
     from paddleformers_amd import deep_gemm
     from paddleformers_amd import functional as F8
 
-    fp8 = torch.float8_e4m3fn
     out = {}
 
-    def rnd8(*shape):
-        return torch.randint(0, 120, shape, dtype=torch.uint8, device="cuda").view(fp8)
+    # operands are what the quantizers make of seeded Gaussian data (activations N(0,1) in 1x128 tiles,
+    # weights N(0,0.02) in 128x128 tiles), with exact scales or power-of-two scales as the leg needs
+    def qact(M, K, pow2=False):
+        x = torch.randn((M, K), device="cuda").to(torch.bfloat16)
+        q, s_ = F8.fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True, using_pow2_scale=pow2)
+        return q, s_                      # s_ [K/128, M]; its .T is the logical [M, K/128] the GEMMs take
+
+    def qweights(E, N, K, pow2=False):
+        q = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+        s_ = torch.empty((E, N // 128, K // 128), dtype=torch.float32, device="cuda")
+        for e in range(E):
+            w = (torch.randn((N, K), device="cuda") * 0.02).to(torch.bfloat16)
+            q[e], s_[e] = F8.fp8_quant_blockwise(w, quant_method="128x128", using_pow2_scale=pow2)
+        return q, s_
+
+    def e8(t):
+        return F8.scales_to_ue8m0(t, check=False)
+
+    def tkern(fn, n=iters, w=warmup):
+        return time_kernel(fn, [()], n, w)
 
     # config 2: [8192, 7168] x [4096, 7168]^T
     M, N, K = 8192, 4096, 7168
-    a, b = rnd8(M, K), rnd8(N, K)
-    sa, sb = torch.rand((K // 128, M), device="cuda"), torch.rand((N // 128, K // 128), device="cuda")
+    a, sa = qact(M, K)
+    b, sb = qweights(1, N, K)
     o = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
-    ms = time_kernel(lambda: deep_gemm.fp8_gemm_nt((a, sa.T), (b, sb), o), [()], iters, warmup)
-    out["dense_config2_8192x4096x7168"] = {"flop": 2.0 * M * N * K, "ms": ms}
-
-    def e8(*shape):     # UE8M0 exponent bytes around 2^0
-        return torch.randint(120, 131, shape, dtype=torch.uint8, device="cuda")
-
+    out["dense_config2_8192x4096x7168"] = dict(tkern(lambda: deep_gemm.fp8_gemm_nt((a, sa.T), (b[0], sb[0]), o)), flop=2.0 * M * N * K)
     # the same GEMM with power-of-two scales as exponent bytes: block-scaled MFMA kernel
-    ea, eb = e8(K // 128, M), e8(N // 128, K // 128)
-    ms = time_kernel(lambda: deep_gemm.fp8_gemm_nt((a, ea.T), (b, eb), o), [()], iters, warmup)
-    out["dense_config2_ue8m0"] = {"flop": 2.0 * M * N * K, "ms": ms}
+    a, sa = qact(M, K, True)
+    b, sb = qweights(1, N, K, True)
+    ea, eb = e8(sa), e8(sb[0])
+    out["dense_config2_ue8m0"] = dict(tkern(lambda: deep_gemm.fp8_gemm_nt((a, ea.T), (b[0], eb), o)), flop=2.0 * M * N * K)
     del a, b, o
     # config 3 forward GEMMs (32 experts, 8192 routed rows, Zipf 1.1, segments padded to 128) with UE8M0 scales
     E3, H3, I3 = 32, 7168, 2048
     _, padded3 = zipf_counts(8192, E3, 1.1, seed=3)
     M3 = int(padded3.sum())
     mi3 = torch.from_numpy(np.repeat(np.arange(E3, dtype=np.int32), padded3)).cuda()
-    a3, w13 = rnd8(M3, H3), rnd8(E3, 2 * I3, H3)
+    a3, sa3 = qact(M3, H3, True)
+    w13, sw13 = qweights(E3, 2 * I3, H3, True)
     o13 = torch.empty((M3, 2 * I3), dtype=torch.bfloat16, device="cuda")
-    ea3, ew13 = e8(H3 // 128, M3), e8(E3, 2 * I3 // 128, H3 // 128)
-    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a3, ea3.T), (w13, ew13), o13, mi3), [()], iters, warmup)
-    out["grouped_config3_up_gate_ue8m0"] = {"flop": 2.0 * 8192 * H3 * 2 * I3, "ms": ms, "padded_rows": M3}
+    ea3, ew13 = e8(sa3), e8(sw13)
+    out["grouped_config3_up_gate_ue8m0"] = dict(tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a3, ea3.T), (w13, ew13), o13, mi3)),
+                                                flop=2.0 * 8192 * H3 * 2 * I3, padded_rows=M3)
     del a3, w13, o13
-    a23, w23 = rnd8(M3, I3), rnd8(E3, H3, I3)
+    a23, sa23 = qact(M3, I3, True)
+    w23, sw23 = qweights(E3, H3, I3, True)
     o33 = torch.empty((M3, H3), dtype=torch.bfloat16, device="cuda")
-    ea23, ew23 = e8(I3 // 128, M3), e8(E3, H3 // 128, I3 // 128)
-    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a23, ea23.T), (w23, ew23), o33, mi3), [()], iters, warmup)
-    out["grouped_config3_down_ue8m0"] = {"flop": 2.0 * 8192 * I3 * H3, "ms": ms, "padded_rows": M3}
+    ea23, ew23 = e8(sa23), e8(sw23)
+    out["grouped_config3_down_ue8m0"] = dict(tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a23, ea23.T), (w23, ew23), o33, mi3)),
+                                             flop=2.0 * 8192 * I3 * H3, padded_rows=M3)
     del a23, w23, o33
     # config 5 forward: E=128, H=4096, I=1408, 131072 routed rows, Zipf(1.0)
     E, H, I, ROUTED = 128, 4096, 1408, 131072
     counts, padded = zipf_counts(ROUTED, E, 1.0, seed=5, n_empty=0)
     Mp = int(padded.sum())
     mi = torch.from_numpy(np.repeat(np.arange(E, dtype=np.int32), padded)).cuda()
-    a = rnd8(Mp, H)
-    sa = torch.rand((H // 128, Mp), device="cuda")
-    w1, s1 = rnd8(E, 2 * I, H), torch.rand((E, 2 * I // 128, H // 128), device="cuda")
-    o1 = torch.empty((Mp, 2 * I), dtype=torch.bfloat16, device="cuda")
-    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa.T), (w1, s1), o1, mi), [()], iters, warmup)
-    out["grouped_config5_up_gate"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms, "padded_rows": Mp}
-    ea5, ew5 = e8(H // 128, Mp), e8(E, 2 * I // 128, H // 128)
-    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, ea5.T), (w1, ew5), o1, mi), [()], iters, warmup)
-    out["grouped_config5_up_gate_ue8m0"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms, "padded_rows": Mp}
-    del w1, o1, ea5, ew5
-    a2, sa2 = rnd8(Mp, I), torch.rand((Mp, I // 128), device="cuda")
-    w2, s2 = rnd8(E, H, I), torch.rand((E, H // 128, I // 128), device="cuda")
-    o3 = torch.empty((Mp, H), dtype=torch.bfloat16, device="cuda")
-    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a2, sa2), (w2, s2), o3, mi), [()], iters, warmup)
-    out["grouped_config5_down"] = {"flop": 2.0 * ROUTED * I * H, "ms": ms, "padded_rows": Mp}
-    ea5, ew5 = e8(I // 128, Mp), e8(E, H // 128, I // 128)
-    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a2, ea5.T), (w2, ew5), o3, mi), [()], iters, warmup)
-    out["grouped_config5_down_ue8m0"] = {"flop": 2.0 * ROUTED * I * H, "ms": ms, "padded_rows": Mp}
-    del a2, w2, o3, ea5, ew5
+    for pow2, tag in ((False, ""), (True, "_ue8m0")):
+        a, sa = qact(Mp, H, pow2)
+        w1, s1 = qweights(E, 2 * I, H, pow2)
+        o1 = torch.empty((Mp, 2 * I), dtype=torch.bfloat16, device="cuda")
+        sa_l, s1_l = (e8(sa).T, e8(s1)) if pow2 else (sa.T, s1)
+        out["grouped_config5_up_gate" + tag] = dict(tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa_l), (w1, s1_l), o1, mi)),
+                                                    flop=2.0 * ROUTED * H * 2 * I, padded_rows=Mp)
+        del a, w1, o1
+        a2, sa2 = qact(Mp, I, pow2)
+        w2, s2 = qweights(E, H, I, pow2)
+        o3 = torch.empty((Mp, H), dtype=torch.bfloat16, device="cuda")
+        sa2_l, s2_l = (e8(sa2).T, e8(s2)) if pow2 else (sa2.T, s2)
+        out["grouped_config5_down" + tag] = dict(tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a2, sa2_l), (w2, s2_l), o3, mi)),
+                                                 flop=2.0 * ROUTED * I * H, padded_rows=Mp)
+        del a2, w2, o3
+    torch.cuda.empty_cache()
     # config 5 weight gradient dW1[e] [H, 2I] += x_e^T . do1_e, all experts in one launch
     rows = [int(r) for r in padded]
     x = torch.randn((Mp, H), device="cuda").to(torch.bfloat16)
     d = (torch.randn((Mp, 2 * I), device="cuda") * 1e-3).to(torch.bfloat16)
-    ms_q = time_kernel(lambda: F8.fused_transpose_split_quant(x, None, rows, True), [()], 5, 2)
-    out["transpose_split_quant_config5_x"] = {"bytes": Mp * H * 3 + (Mp // 128) * H * 4, "ms": ms_q}
+    ms_q = time_kernel(lambda: F8.fused_transpose_split_quant(x, None, rows, True), [()], 20, 3)
+    out["transpose_split_quant_config5_x"] = dict(ms_q, bytes=Mp * H * 3 + (Mp // 128) * H * 4)
     a_t, sa_t = F8.fused_transpose_split_quant(x, None, rows, True)
     b_t, sb_t = F8.fused_transpose_split_quant(d, None, rows, True)
     del x, d
     g = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
-    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True), [()], 5, 2)
-    out["grouped_wgrad_config5_dw1"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms}
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True), [()], 20, 3)
+    out["grouped_wgrad_config5_dw1"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
     # the operands above carry power-of-two scales (pow_2_scales=True): scales applied inside the MFMA
-    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True, scales_pow2=True), [()], 5, 2)
-    out["grouped_wgrad_config5_dw1_pow2"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms}
-    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=False, scales_pow2=True), [()], 5, 2)
-    out["grouped_wgrad_config5_dw1_pow2_overwrite"] = {"flop": 2.0 * ROUTED * H * 2 * I, "ms": ms}
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True, scales_pow2=True), [()], 20, 3)
+    out["grouped_wgrad_config5_dw1_pow2"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=False, scales_pow2=True), [()], 20, 3)
+    out["grouped_wgrad_config5_dw1_pow2_overwrite"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
     del a_t, sa_t, b_t, sb_t, g
     torch.cuda.empty_cache()
     # per-step weight requantization of config 3's up+gate experts: both orientations from one read
     Ew, Hw, Iw = 32, 7168, 2048
     ws = [(torch.randn((Hw, 2 * Iw), device="cuda") * 0.02).to(torch.bfloat16) for _ in range(Ew)]
-    ms = time_kernel(lambda: F8.fused_stack_quant_both(ws), [()], 5, 2)
-    out["stack_quant_both_config3_w1"] = {"bytes": Ew * Hw * 2 * Iw * 4 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4, "ms": ms}
-    ms = time_kernel(lambda: (F8.fused_stack_transpose_quant(ws, False), F8.fused_stack_transpose_quant(ws, True)), [()], 5, 2)
-    out["stack_quant_two_calls_config3_w1"] = {"bytes": Ew * Hw * 2 * Iw * 6 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4, "ms": ms}
+    ms = time_kernel(lambda: F8.fused_stack_quant_both(ws), [()], 20, 3)
+    out["stack_quant_both_config3_w1"] = dict(ms, bytes=Ew * Hw * 2 * Iw * 4 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4)
+    ms = time_kernel(lambda: (F8.fused_stack_transpose_quant(ws, False), F8.fused_stack_transpose_quant(ws, True)), [()], 20, 3)
+    out["stack_quant_two_calls_config3_w1"] = dict(ms, bytes=Ew * Hw * 2 * Iw * 6 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4)
     del ws
     torch.cuda.empty_cache()
     # checkpoint load: block-FP8 [32, 4096, 7168] (128x128 blocks, UE8M0 scales) -> bf16
@@ -236,8 +292,8 @@ def bench_other_gemms(iters=10, warmup=3):
     dq = CD.get_checkpoint_dequantizer("fp8_block").configure_formats("e4m3", "ue8m0").configure_geometry((1, 2), (128, 128))
     qw = torch.randint(0, 120, (Ew, 2 * Iw, Hw), dtype=torch.uint8, device="cuda")
     sc = torch.randint(110, 130, (Ew, 2 * Iw // 128, Hw // 128), dtype=torch.uint8, device="cuda")
-    ms = time_kernel(lambda: dq.dequantize({"qweight": qw, "scale": sc}, torch.bfloat16), [()], 5, 2)
-    out["block_dequant_config3_w1"] = {"bytes": Ew * 2 * Iw * Hw * 3 + sc.numel(), "ms": ms}
+    ms = time_kernel(lambda: dq.dequantize({"qweight": qw, "scale": sc}, torch.bfloat16), [()], 20, 3)
+    out["block_dequant_config3_w1"] = dict(ms, bytes=Ew * 2 * Iw * Hw * 3 + sc.numel())
     del qw, sc
     torch.cuda.empty_cache()
     # config 5 token reordering either side of the expert MLP: 16384 tokens x top-8 over 128 experts
@@ -248,11 +304,11 @@ def bench_other_gemms(iters=10, warmup=3):
     rm_t = torch.from_numpy(rm_np).cuda()
     pr_t = torch.rand((Tt, tk), device="cuda")
     xt = torch.randn((Tt, Ht), device="cuda").to(torch.bfloat16)
-    ms = time_kernel(lambda: F8.moe_permute(xt, None, rm_t, pr_t, Et, cnts, 128, validate=False), [()], 5, 2)
+    ms = time_kernel(lambda: F8.moe_permute(xt, None, rm_t, pr_t, Et, cnts, 128, validate=False), [()], 20, 3)
     ux, rowmap, up, _ = F8.moe_permute(xt, None, rm_t, pr_t, Et, cnts, 128)
-    out["moe_permute_config5"] = {"bytes": Tt * Ht * 2 + ux.numel() * 2, "ms": ms}
-    ms = time_kernel(lambda: F8.moe_unpermute(ux, rowmap, rm_t, up, Tt, Et), [()], 5, 2)
-    out["moe_unpermute_config5"] = {"bytes": Tt * tk * Ht * 2 + Tt * Ht * 2, "ms": ms}
+    out["moe_permute_config5"] = dict(ms, bytes=Tt * Ht * 2 + ux.numel() * 2)
+    ms = time_kernel(lambda: F8.moe_unpermute(ux, rowmap, rm_t, up, Tt, Et), [()], 20, 3)
+    out["moe_unpermute_config5"] = dict(ms, bytes=Tt * tk * Ht * 2 + Tt * Ht * 2)
     del xt, ux, rowmap, up
     torch.cuda.empty_cache()
     # the RMSNorm the dense FP8 MLP recomputes: forward and backward on [16384, 7168] bf16
@@ -260,48 +316,51 @@ def bench_other_gemms(iters=10, warmup=3):
     xn = torch.randn((Mn, Hn), device="cuda").to(torch.bfloat16)
     wn = torch.randn((Hn,), device="cuda").to(torch.bfloat16)
     dn = torch.randn((Mn, Hn), device="cuda").to(torch.bfloat16)
-    ms = time_kernel(lambda: F8.fused_rms_norm_ext(xn, wn, 1e-6), [()], 5, 2)
-    out["rms_norm_fwd_16384x7168"] = {"bytes": Mn * Hn * 4 + Mn * 4, "ms": ms}
+    ms = time_kernel(lambda: F8.fused_rms_norm_ext(xn, wn, 1e-6), [()], 20, 3)
+    out["rms_norm_fwd_16384x7168"] = dict(ms, bytes=Mn * Hn * 4 + Mn * 4)
     _, ivn = F8.fused_rms_norm_ext(xn, wn, 1e-6)
-    ms = time_kernel(lambda: F8.fused_rms_norm_ext_grad(xn, wn, ivn, dn, 1e-6), [()], 5, 2)
-    out["rms_norm_bwd_16384x7168"] = {"bytes": Mn * Hn * 6 + Mn * 4 + Hn * 4, "ms": ms}
+    ms = time_kernel(lambda: F8.fused_rms_norm_ext_grad(xn, wn, ivn, dn, 1e-6), [()], 20, 3)
+    out["rms_norm_bwd_16384x7168"] = dict(ms, bytes=Mn * Hn * 6 + Mn * 4 + Hn * 4)
     del xn, dn, ivn
     torch.cuda.empty_cache()
     # dequantizers on a [16384, 7168] activation / a [7168, 4096] weight
-    qa = rnd8(Mn, Hn)
-    sa_d = torch.rand((Hn // 128, Mn), device="cuda")
-    ms = time_kernel(lambda: F8.fused_act_dequant(qa, sa_d.T), [()], 5, 2)
-    out["act_dequant_16384x7168"] = {"bytes": Mn * Hn * 3 + Mn * (Hn // 128) * 4, "ms": ms}
-    qw2, sw2 = rnd8(Hn, 4096), torch.rand((Hn // 128, 4096 // 128), device="cuda")
-    ms = time_kernel(lambda: F8.weight_dequant(qw2, sw2), [()], 5, 2)
-    out["weight_dequant_7168x4096"] = {"bytes": Hn * 4096 * 3 + sw2.numel() * 4, "ms": ms}
+    qa, sa_d = qact(Mn, Hn)
+    ms = time_kernel(lambda: F8.fused_act_dequant(qa, sa_d.T), [()], 20, 3)
+    out["act_dequant_16384x7168"] = dict(ms, bytes=Mn * Hn * 3 + Mn * (Hn // 128) * 4)
+    qw2, sw2 = qweights(1, Hn, 4096)
+    qw2, sw2 = qw2[0], sw2[0]
+    ms = time_kernel(lambda: F8.weight_dequant(qw2, sw2), [()], 20, 3)
+    out["weight_dequant_7168x4096"] = dict(ms, bytes=Hn * 4096 * 3 + sw2.numel() * 4)
     del qa, sa_d, qw2, sw2
     # SwiGLU backward of the MoE node at config 5: o1 [Mp, 2I], do2_s [Mp, I] -> do1, o2_s, probs_grad
     o1b = torch.randn((Mp, 2 * I), device="cuda").to(torch.bfloat16)
     d2b = (torch.randn((Mp, I), device="cuda") * 1e-3).to(torch.bfloat16)
     prb = torch.rand((Mp, 1), device="cuda")
-    ms = time_kernel(lambda: F8.fused_swiglu_weighted_bwd(o1b, d2b, prb), [()], 5, 2)
-    out["swiglu_bwd_config5"] = {"bytes": Mp * I * 12 + Mp * 8, "ms": ms}
+    ms = time_kernel(lambda: F8.fused_swiglu_weighted_bwd(o1b, d2b, prb), [()], 20, 3)
+    out["swiglu_bwd_config5"] = dict(ms, bytes=Mp * I * 12 + Mp * 8)
     del o1b, d2b, prb
     # dense weight gradient of config 2: dW [7168, 4096] = x^T [7168, 8192] . dy^T [4096, 8192]^T, fp32 out
     Mw, Kw, Nw = 8192, 7168, 4096
-    xt_q, dyt_q = rnd8(Kw, Mw), rnd8(Nw, Mw)
-    sxt = torch.exp2(torch.randint(-3, 3, (Mw // 128, Kw), device="cuda").float())
-    sdy = torch.exp2(torch.randint(-3, 3, (Mw // 128, Nw), device="cuda").float())
+    xw = torch.randn((Mw, Kw), device="cuda").to(torch.bfloat16)
+    dyw = (torch.randn((Mw, Nw), device="cuda") * 1e-3).to(torch.bfloat16)
+    (xt_q,), (sxt,) = F8.fused_transpose_split_quant(xw, None, [Mw], True)       # x^T [Kw, Mw], scales [Mw/128, Kw], powers of two
+    (dyt_q,), (sdy,) = F8.fused_transpose_split_quant(dyw, None, [Mw], True)
+    del xw, dyw
     dwd = torch.zeros((Kw, Nw), dtype=torch.float32, device="cuda")
     ms = time_kernel(lambda: F8.fp8_gemm_blockwise(xt_q, sxt, dyt_q, sdy, out=dwd, accumulate=True), [()], iters, warmup)
-    out["wgrad_dense_config2"] = {"flop": 2.0 * Mw * Kw * Nw, "ms": ms}
+    out["wgrad_dense_config2"] = dict(ms, flop=2.0 * Mw * Kw * Nw)
     ms = time_kernel(lambda: F8.fp8_gemm_blockwise(xt_q, sxt, dyt_q, sdy, out=dwd, accumulate=True, scales_pow2=True), [()], iters, warmup)
-    out["wgrad_dense_config2_pow2"] = {"flop": 2.0 * Mw * Kw * Nw, "ms": ms}
+    out["wgrad_dense_config2_pow2"] = dict(ms, flop=2.0 * Mw * Kw * Nw)
     del xt_q, dyt_q, sxt, sdy, dwd
     # masked grouped GEMM (fixed capacity per expert): 32 experts x 512 rows, 256..512 of them valid
     Em, Cm, Km, Nm = 32, 512, 7168, 4096
-    am, bm = rnd8(Em, Cm, Km), rnd8(Em, Nm, Km)
-    sam, sbm = torch.rand((Em, Cm, Km // 128), device="cuda"), torch.rand((Em, Nm // 128, Km // 128), device="cuda")
+    am, sam = F8.fp8_quant_blockwise(torch.randn((Em * Cm, Km), device="cuda").to(torch.bfloat16), quant_method="1x128")
+    am, sam = am.view(Em, Cm, Km), sam.view(Em, Cm, Km // 128)
+    bm, sbm = qweights(Em, Nm, Km)
     mm = torch.from_numpy(np.random.default_rng(7).integers(256, Cm + 1, Em).astype(np.int32)).cuda()
     om = torch.empty((Em, Cm, Nm), dtype=torch.bfloat16, device="cuda")
     ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_masked((am, sam), (bm, sbm), om, mm, Cm), [()], iters, warmup)
-    out["grouped_masked_32x512"] = {"flop": 2.0 * float(mm.sum().item()) * Km * Nm, "ms": ms}
+    out["grouped_masked_32x512"] = dict(ms, flop=2.0 * float(mm.sum().item()) * Km * Nm)
     del am, bm, sam, sbm, om
     torch.cuda.empty_cache()
     # the masked-layout expert node (fixed capacity per expert) end to end: 32 experts x 512 rows, 256..512 valid
@@ -347,28 +406,20 @@ def bench_other_gemms(iters=10, warmup=3):
         nodem.forward(xm, prm, mm)
         nodem.backward(dm, mm, None, Cm)
 
-    ms = time_kernel(fwd_bwd_masked, [()], 3, 2)
+    ms = time_kernel(fwd_bwd_masked, [()], 20, 3)
     valid_rows = float(mm.sum().item())
-    out["ernie_masked_node_32x512_fwd_bwd"] = {"flop": 2 * (2.0 * valid_rows * Hm * 2 * Im + 2.0 * valid_rows * Im * Hm)
-                                               + (2.0 * Em * Cm * Hm * 2 * Im + 2.0 * Em * Cm * Im * Hm), "ms": ms}
+    out["ernie_masked_node_32x512_fwd_bwd"] = dict(ms, flop=2 * (2.0 * valid_rows * Hm * 2 * Im + 2.0 * valid_rows * Im * Hm)
+                                               + (2.0 * Em * Cm * Hm * 2 * Im + 2.0 * Em * Cm * Im * Hm))
     del exm, gm1, gm2, xm, dm, nodem
     torch.cuda.empty_cache()
     # the fused FP8 MoE node end to end at config 5: forward + backward (dgrad and wgrad, both GEMMs),
     # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers; then the same step
     # with power-of-two scales throughout (use_ue8m0): forward and dgrad GEMMs on the block-scaled MFMA kernel
     node_flop = 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H)
-    out["moe_node_config5_fwd_bwd"] = {"flop": node_flop, "ms": bench_moe_node(False, 3, 2)}
-    out["moe_node_config5_fwd_bwd_ue8m0"] = {"flop": node_flop, "ms": bench_moe_node(True, 3, 2)}
-    for v in out.values():
-        if "flop" in v:
-            v["TFLOPs"] = round(v.pop("flop") / (v["ms"] * 1e-3) / 1e12, 1)
-            v["frac_fp8_peak"] = round(v["TFLOPs"] / FP8_PEAK_TFLOPS, 4)
-        else:
-            v["GBps"] = round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)
-            v["frac_hbm"] = round(v["GBps"] / HBM_PEAK_GBS, 4)
-        v["ms"] = round(v["ms"], 4)
+    out["moe_node_config5_fwd_bwd"] = dict(bench_moe_node(False, 20, 3), flop=node_flop)
+    out["moe_node_config5_fwd_bwd_ue8m0"] = dict(bench_moe_node(True, 20, 3), flop=node_flop)
     torch.cuda.empty_cache()
-    return out
+    return _finish(out)
 
 
 def bench_moe_node(ue8m0, iters, warmup):
@@ -452,7 +503,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-quant", action="store_true")
+    ap.add_argument("--no-quant", action="store_true", help="skip the quantizer and other-GEMM legs")
+    ap.add_argument("--quant-only", action="store_true", help="run only the quantizer legs (GB/s) and print them")
     ap.add_argument("--copy-yardstick", action="store_true",
                     help="also launch one plain 1 GiB copy (pf8::k_debug_copy) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings of the GEMM can be scaled by a kernel of known traffic")
@@ -476,8 +528,11 @@ def main():
     torch.cuda.set_device(0)
     torch.manual_seed(3)
 
+    if args.quant_only:
+        print(json.dumps({"quant": bench_quantizers()}))
+        return
     if args.moe_node:
-        ms = bench_moe_node(args.moe_node == "ue8m0", args.steps, args.warmup)
+        ms = bench_moe_node(args.moe_node == "ue8m0", args.steps, args.warmup)["ms"]
         flop = 3 * (2.0 * 131072 * 4096 * 2 * 1408 + 2.0 * 131072 * 1408 * 4096)
         print(json.dumps({"leg": "moe_node_config5_fwd_bwd" + ("_ue8m0" if args.moe_node == "ue8m0" else ""), "steps": args.steps,
                           "warmup": args.warmup, "ms": round(ms, 4), "TFLOPs": round(flop / ms / 1e9, 1)}))
@@ -547,13 +602,17 @@ def main():
         del src, dst
 
     names = ["quant_x", "gemm_up_gate", "swiglu_requant", "gemm_down"]
-    kms = {n: sum(ev[k][i].elapsed_time(ev[k][i + 1]) for k in range(args.steps)) / args.steps for i, n in enumerate(names)}
+    per = {n: sorted(ev[k][i].elapsed_time(ev[k][i + 1]) for k in range(args.steps)) for i, n in enumerate(names)}
+    kms = {n: sum(v) / len(v) for n, v in per.items()}              # mean over the timed steps (what `value` is built from)
+    kmed = {n: v[len(v) // 2] for n, v in per.items()}
+    kmin = {n: v[0] for n, v in per.items()}
 
     flops_up = 2.0 * ROUTED * H * 2 * I
     flops_down = 2.0 * ROUTED * I * H
     flops = flops_up + flops_down
     value = flops / (ms_per_step * 1e-3) / 1e12
     ach = flops_up / (kms["gemm_up_gate"] * 1e-3) / 1e12
+    traffic, traffic_rec = traffic_from_summary(ROOFLINE_KERNEL)
 
     res = {
         "metric": "FP8 MoE grouped-GEMM TFLOP/s + block-quant GB/s on 1 MI355X (% of peak)",
@@ -576,15 +635,19 @@ def main():
         },
         "frac_fp8_peak": round(value / FP8_PEAK_TFLOPS, 4),
         "kernel_ms": {k: round(v, 4) for k, v in kms.items()},
+        "kernel_ms_median": {k: round(v, 4) for k, v in kmed.items()},
+        "kernel_ms_min": {k: round(v, 4) for k, v in kmin.items()},
         "roofline": {
-            "kernel": "pf8::k_gemm_fwd_deep<1, 0> (up+gate grouped GEMM)",
+            "kernel": ROOFLINE_KERNEL + " (up+gate grouped GEMM)",
             "bound": "mfma",
             "achieved": round(ach, 2),
             "peak": FP8_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(ach / FP8_PEAK_TFLOPS, 4),
-            "traffic": GEMM_UP_GATE_TRAFFIC_BYTES,
+            "traffic": traffic,
+            "traffic_source": None if traffic_rec is None else {k: traffic_rec[k] for k in ("commit", "command") if k in traffic_rec},
             "algorithmic_bytes": int(w1q[counts > 0].numel() + Mpad * H + Mpad * 2 * I * 2),
+            "launch_ms": round(kms["gemm_up_gate"], 4),
         },
     }
     if not args.no_quant:

@@ -487,6 +487,38 @@ PF8O_API void pf8o_grouped_gemm_nt_masked(const uint8_t* a, const float* sa, con
 PF8O_API void pf8o_e4m3_encode_array(const float* v, int64_t n, uint8_t* out) {
     for (int64_t i = 0; i < n; ++i) out[i] = pf8o_e4m3_encode(v[i]);
 }
+/* Checker for the device kernels' division-free quantizer step.  The formulation is q = x / s with an
+ * IEEE divide per element (kernel.py:45-47); the kernels instead form y = 1/s once per tile and take
+ *     q0 = x * y;  r = fma(-q0, s, x);  q = fma(r, y, q0)
+ * per element.  Every quantizer input is a bf16 value and s = amax/448 of a bf16 amax, a finite set:
+ * this walks ALL pairs (amax > 0 a finite bf16 magnitude, 0 <= x <= amax a bf16 magnitude; the device
+ * copies the sign of x onto the result, which is what makes negative inputs, -0 included, symmetric) whose scale is at least min_scale (smaller ones take the divide on the device as well) and
+ * counts, in out[0..2]: pairs visited, pairs whose e4m3 CODE differs between the two ways, pairs whose
+ * fp32 quotient differs (those are quotients far below the e4m3 grid, where the residual underflows). */
+PF8O_API void pf8o_check_reciprocal_division(int pow2, float min_scale, int64_t* out) {
+    int64_t total = 0, bad_code = 0, bad_q = 0;
+#pragma omp parallel for schedule(dynamic, 64) reduction(+ : total, bad_code, bad_q)
+    for (int ab = 1; ab < 0x7F80; ++ab) {
+        const float amax = pf8o_bf16_to_f32((uint16_t)ab);
+        const float s = scale_from_amax(amax, pow2);
+        if (!(s >= min_scale)) continue;
+        volatile float yv = 1.0f / s;
+        const float y = yv;
+        for (int xb = 0; xb <= ab; ++xb) {
+            const float x = pf8o_bf16_to_f32((uint16_t)xb);
+            volatile float qv = x / s;
+            const float q = qv;
+            const float q0 = x * y;
+            const float r = fmaf(-q0, s, x);
+            const float q1 = fmaf(r, y, q0);
+            total++;
+            if (pf8o_e4m3_encode(q1) != pf8o_e4m3_encode(q)) bad_code++;
+            if (memcmp(&q1, &q, 4) != 0) bad_q++;
+        }
+    }
+    out[0] = total; out[1] = bad_code; out[2] = bad_q;
+}
+
 PF8O_API void pf8o_div_encode_array(const float* x, const float* s, int64_t n, uint8_t* out) {
     for (int64_t i = 0; i < n; ++i) out[i] = pf8o_e4m3_encode(x[i] / s[i]);
 }

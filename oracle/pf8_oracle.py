@@ -156,6 +156,14 @@ def f32_to_bf16_array(v):
     return _array_fn("pf8o_f32_to_bf16_array", v, np.uint16)
 
 
+def check_reciprocal_division(pow2=False, min_scale=1.0e-30):
+    """Exhaustive sweep of the reciprocal-and-residual division over every (bf16 amax, bf16 x <= amax) pair:
+    returns (pairs, pairs whose e4m3 code differs from the IEEE divide's, pairs whose fp32 quotient differs)."""
+    out = np.zeros(3, np.int64)
+    lib().pf8o_check_reciprocal_division(int(pow2), C.c_float(min_scale), _p(out))
+    return int(out[0]), int(out[1]), int(out[2])
+
+
 def div_encode_array(x, s):
     """e4m3_encode(x / s) element-wise with IEEE fp32 division."""
     x = np.ascontiguousarray(x, dtype=np.float32).ravel()

@@ -78,37 +78,39 @@ __device__ __forceinline__ uint32_t amax_bits8(uint4 w) {
 
 struct TileScale {
     float s;      // decode scale stored next to the bytes
-    float r_lo;   // reciprocal of s nudged down by 2^-20 (relative)
-    float r_hi;   // reciprocal of s nudged up by 2^-20
-    bool slow;    // tile must take the IEEE division path (scale too small for a finite reciprocal)
-    bool exact;   // s is a power of two: r_lo == r_hi == 1/s exactly, and v * r_lo IS the correctly rounded v / s
+    float y;      // its correctly rounded reciprocal (IEEE 1/s); exact when s is a power of two
+    bool slow;    // scale too small for a finite, normal reciprocal: the tile takes the IEEE division
+    bool exact;   // s is a power of two: v * y IS the correctly rounded v / s
 };
 
-// s = amax/448 (IEEE divide), amax == 0 -> 1; pow2: decode scale rounded up to a power of two.
+// Scales below this have no usable reciprocal (1/s overflows or s is subnormal): such tiles divide.
+constexpr float kMinFastScale = 1.0e-30f;
+
+// 1/s of a power of two s = 2^k, k in [-126, 126] (what the pow2 rule below yields), by exponent arithmetic
+__device__ __forceinline__ float pow2_recip(float s) { return u2f(0x7F000000u - f2u(s)); }
+
 __device__ __forceinline__ TileScale make_scale_from(float s) {
     TileScale t;
     t.s = s;
-    const float r = __builtin_amdgcn_rcpf(s);
-    t.r_lo = r * 0.99999904632568359375f;   // 1 - 2^-20
-    t.r_hi = r * 1.00000095367431640625f;   // 1 + 2^-20
-    t.slow = !(s >= 1.0e-30f);
+    t.slow = !(s >= kMinFastScale);
+    t.y = 1.0f / (t.slow ? 1.0f : s);
     t.exact = false;
     return t;
 }
-// 1/s of a power of two s = 2^k, k in [-126, 126] (what the pow2 rule below yields), by exponent arithmetic
-__device__ __forceinline__ float pow2_recip(float s) { return u2f(0x7F000000u - f2u(s)); }
-__device__ __forceinline__ TileScale make_scale(uint32_t amax_bits, bool pow2) {
-    float amax = u2f(amax_bits);
-    float s = amax / 448.0f;
+// s = amax/448 (IEEE divide), amax == 0 -> 1; pow2: decode scale rounded up to a power of two.
+__device__ __forceinline__ float scale_of(uint32_t amax_bits, bool pow2) {
+    float s = u2f(amax_bits) / 448.0f;
     if (pow2) s = u2f((f2u(s) + 0x007FFFFFu) & 0x7F800000u);
-    if (amax_bits == 0u) s = 1.0f;
+    return amax_bits == 0u ? 1.0f : s;
+}
+__device__ __forceinline__ TileScale make_scale(uint32_t amax_bits, bool pow2) {
+    const float s = scale_of(amax_bits, pow2);
     if (pow2) {
         // dividing by a power of two is multiplying by its (exact) reciprocal: the product is the
-        // correctly rounded quotient, so one conversion per element and no bracket to check.  (With
-        // the bracket every exact e4m3 tie, one bf16 value in 32, would take the division path.)
+        // correctly rounded quotient, one multiply and one conversion per element
         TileScale t;
         t.s = s;
-        t.r_lo = t.r_hi = pow2_recip(s);
+        t.y = pow2_recip(s);
         t.slow = false;
         t.exact = true;
         return t;
@@ -128,86 +130,51 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 }
 
 // Quantise 8 values of one tile: bytes == e4m3_rne(v / s) with v / s the correctly rounded fp32
-// quotient.  Fast path: the quotient is bracketed by v*r_lo and v*r_hi (the reciprocal is good to
-// 1 ulp, the nudges are 2^-20, so the bracket holds with a wide margin); rounding is monotone, so
-// where both ends convert to the same e4m3 code that is the code of the exact quotient.  Where they
-// differ a rounding boundary lies inside the 2^-19-wide bracket and that ELEMENT is redone with the
-// IEEE division.  This is not rare: s = amax/448 carries an fp32 rounding error, so every element
-// for which 448 v / amax is an exact e4m3 tie in real arithmetic (bf16 inputs make these common,
-// about one element in a thousand) sits 2^-24 from a boundary.  Most wavefronts therefore visit
-// the fallback for one or two elements, and it is written to cost one division, not eight.
-__device__ __forceinline__ uint32_t nonzero_bytes(uint32_t d) {   // 0x80 in every byte of d that is not zero
-    return (((d & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | d) & 0x80808080u;
+// quotient, without dividing per element.  With y = RN(1/s) (one IEEE division per tile):
+//     q0 = v * y;   r = fma(-q0, s, v);   q = fma(r, y, q0)
+// q0 is within an ulp or two of the quotient, the residual r = v - q0 s is exact in fp32, and the
+// corrected q rounds to the same e4m3 code as the IEEE quotient.  That is not taken on faith: the
+// inputs of every quantizer here are bf16 values and s = amax/448 of a bf16 amax, a finite set, and
+// the CPU test suite walks ALL (amax, v) pairs of it (522 million, |v| <= amax, s >= kMinFastScale),
+// comparing the codes of this sequence with those of the division; it also holds on 2.5e9 random
+// pairs of an arbitrary fp32 scale and a bf16 value.  (The fp32 quotients themselves differ only
+// where the residual underflows, quotients below 2^-27, which encode as zero either way.)
+// One input needs care: v = -0 gives q0 = -0, r = +0 and q = (+0) + (-0) = +0, while -0 / s is -0 (code
+// 0x80).  The quotient always carries the sign of v (s > 0), so the sign is copied over (one v_bfi_b32).
+__device__ __forceinline__ float div_by_recip(float v, float s, float y) {
+    const float q0 = v * y;
+    const float r = __builtin_fmaf(-q0, s, v);
+    return __builtin_copysignf(__builtin_fmaf(r, y, q0), v);
 }
-__device__ __forceinline__ void quant8_fix(const float (&v)[8], float s, uint2& lo, const uint2 hi) {
-    const uint32_t dx = lo.x ^ hi.x, dy = lo.y ^ hi.y;
-    if (__builtin_expect((dx | dy) != 0u, 0)) {
-        const uint32_t zx = nonzero_bytes(dx), zy = nonzero_bytes(dy);
-        if (__builtin_popcount(zx) + __builtin_popcount(zy) == 1) {
-            // the usual case, one element: pick it without branching on its index
-            const int idx = zx ? (__builtin_ctz(zx) >> 3) : 4 + (__builtin_ctz(zy) >> 3);
-            const float a = (idx & 1) ? v[1] : v[0], b = (idx & 1) ? v[3] : v[2];
-            const float c = (idx & 1) ? v[5] : v[4], d = (idx & 1) ? v[7] : v[6];
-            const float e = (idx & 2) ? b : a, f = (idx & 2) ? d : c;
-            const float qv = ((idx & 4) ? f : e) / s;
-            const uint32_t code = cvt_e4m3_lo(qv, qv, 0u) & 0xFFu;
-            const int sh = 8 * (idx & 3);
-            const uint32_t keep = ~(0xFFu << sh), put = code << sh;
-            if (idx & 4) lo.y = (lo.y & keep) | put;
-            else lo.x = (lo.x & keep) | put;
-        } else {
-            // a tile whose amax makes exact ties common (e.g. amax = 448 * 2^k: one value in eight)
-            lo.x = pack4_e4m3(v[0] / s, v[1] / s, v[2] / s, v[3] / s);
-            lo.y = pack4_e4m3(v[4] / s, v[5] / s, v[6] / s, v[7] / s);
-        }
-    }
-}
-__device__ __forceinline__ uint2 quant8_exact(const float (&v)[8], float r) {
+__device__ __forceinline__ uint2 quant8_exact(const float (&v)[8], float y) {
     uint2 o;
-    o.x = pack4_e4m3(v[0] * r, v[1] * r, v[2] * r, v[3] * r);
-    o.y = pack4_e4m3(v[4] * r, v[5] * r, v[6] * r, v[7] * r);
+    o.x = pack4_e4m3(v[0] * y, v[1] * y, v[2] * y, v[3] * y);
+    o.y = pack4_e4m3(v[4] * y, v[5] * y, v[6] * y, v[7] * y);
+    return o;
+}
+__device__ __forceinline__ uint2 quant8_divide(const float (&v)[8], float s) {
+    uint2 o;
+    o.x = pack4_e4m3(v[0] / s, v[1] / s, v[2] / s, v[3] / s);
+    o.y = pack4_e4m3(v[4] / s, v[5] / s, v[6] / s, v[7] / s);
+    return o;
+}
+// 8 values against a scale and its reciprocal; `slow` tiles (tiny scales) divide
+__device__ __forceinline__ uint2 quant8_r(const float (&v)[8], float s, float y, bool slow) {
+    if (__builtin_expect(slow, 0)) return quant8_divide(v, s);
+    uint2 o;
+    o.x = pack4_e4m3(div_by_recip(v[0], s, y), div_by_recip(v[1], s, y), div_by_recip(v[2], s, y), div_by_recip(v[3], s, y));
+    o.y = pack4_e4m3(div_by_recip(v[4], s, y), div_by_recip(v[5], s, y), div_by_recip(v[6], s, y), div_by_recip(v[7], s, y));
     return o;
 }
 __device__ __forceinline__ uint2 quant8(const float (&v)[8], const TileScale& t) {
-    if (t.exact) return quant8_exact(v, t.r_lo);
-    uint2 lo, hi;
-    const float r_lo = t.slow ? 0.0f : t.r_lo, r_hi = t.slow ? __builtin_inff() : t.r_hi;   // slow: every element differs
-    lo.x = pack4_e4m3(v[0] * r_lo, v[1] * r_lo, v[2] * r_lo, v[3] * r_lo);
-    lo.y = pack4_e4m3(v[4] * r_lo, v[5] * r_lo, v[6] * r_lo, v[7] * r_lo);
-    hi.x = pack4_e4m3(v[0] * r_hi, v[1] * r_hi, v[2] * r_hi, v[3] * r_hi);
-    hi.y = pack4_e4m3(v[4] * r_hi, v[5] * r_hi, v[6] * r_hi, v[7] * r_hi);
-    quant8_fix(v, t.s, lo, hi);
-    return lo;
+    if (t.exact) return quant8_exact(v, t.y);
+    return quant8_r(v, t.s, t.y, t.slow);
 }
 
-// ---- quantizers that hold several tiles per lane: scales for up to four tiles in one pass ----
 // value of lane Q of every quad, for all four lanes of the quad (folds into the consuming VALU op)
 template <int Q>
 __device__ __forceinline__ float quad_bcast(float v) {
     return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v), Q * 0x55, 0xF, 0xF, false));
-}
-// Reciprocal pair of a scale; a scale too small for a finite reciprocal gets (0, inf), which makes
-// the two conversions of any element disagree and sends the tile down the division path.
-__device__ __forceinline__ void scale_recips(float s, float& r_lo, float& r_hi) {
-    const float r = __builtin_amdgcn_rcpf(s);
-    const bool ok = s >= 1.0e-30f;
-    r_lo = ok ? r * 0.99999904632568359375f : 0.0f;          // 1 - 2^-20
-    r_hi = ok ? r * 1.00000095367431640625f : __builtin_inff();   // 1 + 2^-20
-}
-__device__ __forceinline__ float scale_of(uint32_t amax_bits, bool pow2) {
-    float s = u2f(amax_bits) / 448.0f;
-    if (pow2) s = u2f((f2u(s) + 0x007FFFFFu) & 0x7F800000u);
-    return amax_bits == 0u ? 1.0f : s;
-}
-// 8 values against a reciprocal pair; elements whose two conversions differ are redone by division
-__device__ __forceinline__ uint2 quant8_r(const float (&v)[8], float r_lo, float r_hi, float s) {
-    uint2 lo, hi;
-    lo.x = pack4_e4m3(v[0] * r_lo, v[1] * r_lo, v[2] * r_lo, v[3] * r_lo);
-    lo.y = pack4_e4m3(v[4] * r_lo, v[5] * r_lo, v[6] * r_lo, v[7] * r_lo);
-    hi.x = pack4_e4m3(v[0] * r_hi, v[1] * r_hi, v[2] * r_hi, v[3] * r_hi);
-    hi.y = pack4_e4m3(v[4] * r_hi, v[5] * r_hi, v[6] * r_hi, v[7] * r_hi);
-    quant8_fix(v, s, lo, hi);
-    return lo;
 }
 
 __device__ __forceinline__ void unpack8(uint4 w, float (&v)[8]) {

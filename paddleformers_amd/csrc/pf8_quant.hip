@@ -18,11 +18,11 @@ namespace pf8 {
 
 // grid.x = column chunks of 16 tiles, grid.y = groups of 4 rows; every lane issues its four 16-byte
 // loads before any arithmetic, so a wavefront is one load phase, one compute phase, one store phase.
-// The kernel is bound by the vector ALU, not by memory (the bracketing quantizer costs about 20
-// ALU cycles per element), so the bookkeeping around it is kept off the vector pipe:
+// The arithmetic has to hide behind the memory stream, so the bookkeeping around it is kept off the
+// vector pipe:
 //   * the row is wave-uniform: every address is a scalar base plus one 32-bit lane offset;
 //   * the scales of a lane group's four tiles are computed in ONE pass (lane q of every quad takes
-//     tile q; the IEEE divide and the reciprocal run once, not four times) and come back through
+//     tile q; the IEEE divides for the scale and for its reciprocal run once, not four times) and come back through
 //     quad-broadcast DPP operands.
 template <int LAYOUT, int U>
 __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict__ x, int64_t M, int64_t m0, int KB, int64_t ldx,
@@ -49,9 +49,9 @@ __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict_
     const int ql = l & 3;
     const uint32_t am_sel = ql == 0 ? am[0] : ql == 1 ? am[1] : ql == 2 ? am[2] : am[3];
     const float sc = scale_of(am_sel, pow2 != 0);       // lane q of a quad: scale of tile q
-    float r_lo, r_hi;
-    scale_recips(sc, r_lo, r_hi);
-    if (pow2) r_lo = pow2_recip(sc);                    // exact: one conversion per element, nothing to check
+    // its reciprocal: exponent arithmetic for a power of two, else ONE IEEE division per tile
+    const bool slow = !(sc >= kMinFastScale);
+    const float y = pow2 ? pow2_recip(sc) : 1.0f / (slow ? 1.0f : sc);
     if (l < 4) {
         const int kb = kb0 + 4 * l + g;
         if (kb < KB) {
@@ -63,16 +63,17 @@ __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict_
     uint2 o[4];
     if (pow2) {
         float v[8];
-        unpack8(w[0], v); o[0] = quant8_exact(v, quad_bcast<0>(r_lo));
-        unpack8(w[1], v); o[1] = quant8_exact(v, quad_bcast<1>(r_lo));
-        unpack8(w[2], v); o[2] = quant8_exact(v, quad_bcast<2>(r_lo));
-        unpack8(w[3], v); o[3] = quant8_exact(v, quad_bcast<3>(r_lo));
+        unpack8(w[0], v); o[0] = quant8_exact(v, quad_bcast<0>(y));
+        unpack8(w[1], v); o[1] = quant8_exact(v, quad_bcast<1>(y));
+        unpack8(w[2], v); o[2] = quant8_exact(v, quad_bcast<2>(y));
+        unpack8(w[3], v); o[3] = quant8_exact(v, quad_bcast<3>(y));
     } else {
         float v[8];
-        unpack8(w[0], v); o[0] = quant8_r(v, quad_bcast<0>(r_lo), quad_bcast<0>(r_hi), quad_bcast<0>(sc));
-        unpack8(w[1], v); o[1] = quant8_r(v, quad_bcast<1>(r_lo), quad_bcast<1>(r_hi), quad_bcast<1>(sc));
-        unpack8(w[2], v); o[2] = quant8_r(v, quad_bcast<2>(r_lo), quad_bcast<2>(r_hi), quad_bcast<2>(sc));
-        unpack8(w[3], v); o[3] = quant8_r(v, quad_bcast<3>(r_lo), quad_bcast<3>(r_hi), quad_bcast<3>(sc));
+        const float s0 = quad_bcast<0>(sc), s1 = quad_bcast<1>(sc), s2 = quad_bcast<2>(sc), s3 = quad_bcast<3>(sc);
+        unpack8(w[0], v); o[0] = quant8_r(v, s0, quad_bcast<0>(y), !(s0 >= kMinFastScale));
+        unpack8(w[1], v); o[1] = quant8_r(v, s1, quad_bcast<1>(y), !(s1 >= kMinFastScale));
+        unpack8(w[2], v); o[2] = quant8_r(v, s2, quad_bcast<2>(y), !(s2 >= kMinFastScale));
+        unpack8(w[3], v); o[3] = quant8_r(v, s3, quad_bcast<3>(y), !(s3 >= kMinFastScale));
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u)
@@ -363,7 +364,7 @@ __device__ __forceinline__ void load_patch_packed(const TileSrc& src, int64_t ro
 //   SPLIT=true : qt / st packed per expert               (transpose-split-quant), source bf16 or e4m3
 // pow2: bit 0 = power-of-two scales for the transposed copy, bit 1 = for the row-scaled copy.
 // Per element the kernel spends one masked copy, two packed-u16 max (row and column amax), one
-// unpack and two bracketing conversions; the 128 row scales and 128 column scales are each computed
+// unpack and two reciprocal-based quantizations; the 128 row scales and 128 column scales are each computed
 // once (threads 0..127 / 128..255) and handed round through LDS instead of sixteen times over.
 template <bool SPLIT, int LAYOUT>
 __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M, int64_t K, uint8_t* __restrict__ q,
@@ -372,7 +373,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
     __shared__ uint32_t lds_t[128 * LDT];      // transposed byte tile
     __shared__ uint32_t lds_cm[4 * 64];        // per-wave packed column maxima
     __shared__ uint32_t lds_rm[128];           // row maxima
-    __shared__ float4 lds_sc[256];             // (s, r_lo, r_hi, slow) for rows 0..127, columns 128..255
+    __shared__ float4 lds_sc[256];             // (s, 1/s, -, slow) for rows 0..127, columns 128..255
     const int tid = threadIdx.x, g = tid >> 4, l = tid & 15, wave = tid >> 6, lane = tid & 63;
     const int64_t tc = blockIdx.x, tr = blockIdx.y;
     const int64_t row0 = tr * 128, col0 = tc * 128;
@@ -417,7 +418,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
         }
         if (tid >= 128 || want_rows) {
             const TileScale t = make_scale(am, (pow2 & (tid < 128 ? 2 : 1)) != 0);
-            lds_sc[tid] = make_float4(t.s, t.r_lo, t.r_hi, t.slow ? 1.0f : 0.0f);
+            lds_sc[tid] = make_float4(t.s, t.y, 0.0f, t.slow ? 1.0f : 0.0f);
         }
     }
     __syncthreads();
@@ -429,7 +430,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float4 f = lds_sc[8 * g + i];
-            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f; t.exact = (pow2 & 2) != 0;
+            TileScale t; t.s = f.x; t.y = f.y; t.slow = f.w != 0.0f; t.exact = (pow2 & 2) != 0;
             const int64_t r = row0 + 8 * g + i;
             float v[8];
             unpack8(w[i], v);
@@ -454,7 +455,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
         for (int h = 0; h < 2; ++h) {
             const int j = 2 * k + h;
             const float4 f = lds_sc[128 + 8 * l + j];
-            TileScale t; t.s = f.x; t.r_lo = f.y; t.r_hi = f.z; t.slow = f.w != 0.0f; t.exact = (pow2 & 1) != 0;
+            TileScale t; t.s = f.x; t.y = f.y; t.slow = f.w != 0.0f; t.exact = (pow2 & 1) != 0;
             cs[j] = t.s;
             lds_put_col(lds_t, l, g, j, h == 0 ? quant8(lo, t) : quant8(hi, t));
         }
