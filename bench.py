@@ -581,15 +581,28 @@ def main():
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2q, w2s), o3, m_idx)
         if evs: evs[4].record()
 
+    # W warm-up steps, then EXACTLY K timed steps between two synchronisations: `value`.  No event is
+    # recorded inside them: recording one idles the stream for about 6 us on this machine, and five per
+    # step would charge the step 4-5% for its own instrumentation.
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
-        step(ev[k])
+        step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    # the same K steps once more with an event between the kernels: the per-kernel times and the
+    # duration of the roofline kernel (each carries the cost of one event record, reported below)
+    for k in range(args.steps):
+        step(ev[k])
+    torch.cuda.synchronize()
+    eo = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
+    for e in eo:
+        e.record()
+    torch.cuda.synchronize()
+    event_overhead_ms = sorted(eo[i].elapsed_time(eo[i + 1]) for i in range(20))[10]
 
     if args.copy_yardstick:
         import ctypes as C
@@ -637,6 +650,7 @@ def main():
         "kernel_ms": {k: round(v, 4) for k, v in kms.items()},
         "kernel_ms_median": {k: round(v, 4) for k, v in kmed.items()},
         "kernel_ms_min": {k: round(v, 4) for k, v in kmin.items()},
+        "event_record_ms": round(event_overhead_ms, 4),
         "roofline": {
             "kernel": ROOFLINE_KERNEL + " (up+gate grouped GEMM)",
             "bound": "mfma",
