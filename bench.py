@@ -174,7 +174,7 @@ def bench_quantizers(iters=60, warmup=10):
     return _finish(out)
 
 
-def bench_other_gemms(iters=50, warmup=10):
+def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     """Kernel-only timings of the other BASELINE GEMM workloads (random e4m3 bytes and scales):
     config 2 dense, config 5 forward grouped GEMMs and the config-5 weight gradient."""
     import numpy as np
@@ -262,21 +262,23 @@ def bench_other_gemms(iters=50, warmup=10):
     rows = [int(r) for r in padded]
     x = torch.randn((Mp, H), device="cuda").to(torch.bfloat16)
     d = (torch.randn((Mp, 2 * I), device="cuda") * 1e-3).to(torch.bfloat16)
-    ms_q = time_kernel(lambda: F8.fused_transpose_split_quant(x, None, rows, True), [()], 20, 3)
+    ms_q = time_kernel(lambda: F8.fused_transpose_split_quant(x, None, rows, True), [()], min(iters, 20), min(warmup, 3))
     out["transpose_split_quant_config5_x"] = dict(ms_q, bytes=Mp * H * 3 + (Mp // 128) * H * 4)
     a_t, sa_t = F8.fused_transpose_split_quant(x, None, rows, True)
     b_t, sb_t = F8.fused_transpose_split_quant(d, None, rows, True)
     del x, d
     g = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
-    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True), [()], 20, 3)
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True), [()], min(iters, 20), min(warmup, 3))
     out["grouped_wgrad_config5_dw1"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
     # the operands above carry power-of-two scales (pow_2_scales=True): scales applied inside the MFMA
-    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True, scales_pow2=True), [()], 20, 3)
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True, scales_pow2=True), [()], min(iters, 20), min(warmup, 3))
     out["grouped_wgrad_config5_dw1_pow2"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
-    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=False, scales_pow2=True), [()], 20, 3)
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=False, scales_pow2=True), [()], min(iters, 20), min(warmup, 3))
     out["grouped_wgrad_config5_dw1_pow2_overwrite"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
     del a_t, sa_t, b_t, sb_t, g
     torch.cuda.empty_cache()
+    if gemm_only:       # the legs a profiler run of the GEMM kernels wants: config 2, 3 (UE8M0), 5 forward and weight gradient
+        return _finish(out)
     # per-step weight requantization of config 3's up+gate experts: both orientations from one read
     Ew, Hw, Iw = 32, 7168, 2048
     ws = [(torch.randn((Hw, 2 * Iw), device="cuda") * 0.02).to(torch.bfloat16) for _ in range(Ew)]
@@ -505,6 +507,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-quant", action="store_true", help="skip the quantizer and other-GEMM legs")
     ap.add_argument("--quant-only", action="store_true", help="run only the quantizer legs (GB/s) and print them")
+    ap.add_argument("--gemm-legs-only", action="store_true",
+                    help="run only the config 2 / 3 (UE8M0) / 5 GEMM and weight-gradient legs and print them")
+    ap.add_argument("--leg-iters", type=int, default=0, help="launches per leg for --quant-only / --gemm-legs-only (profiler runs want few)")
     ap.add_argument("--copy-yardstick", action="store_true",
                     help="also launch one plain 1 GiB copy (pf8::k_debug_copy) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings of the GEMM can be scaled by a kernel of known traffic")
@@ -529,7 +534,11 @@ def main():
     torch.manual_seed(3)
 
     if args.quant_only:
-        print(json.dumps({"quant": bench_quantizers()}))
+        print(json.dumps({"quant": bench_quantizers(args.leg_iters, min(10, args.leg_iters)) if args.leg_iters else bench_quantizers()}))
+        return
+    if args.gemm_legs_only:
+        it = args.leg_iters or 50
+        print(json.dumps({"other_gemm": bench_other_gemms(it, min(10, it), gemm_only=True)}))
         return
     if args.moe_node:
         ms = bench_moe_node(args.moe_node == "ue8m0", args.steps, args.warmup)["ms"]

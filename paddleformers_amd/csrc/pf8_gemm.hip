@@ -825,11 +825,12 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         // The persistent deep-pipeline kernel wins where the operand stream, not the matrix pipe, sets
         // the pace.  Measured on MI355X against the two-workgroup kernel: +14..24% when all tiles
         // fit one round of compute units (dense M <= 2048 at N = 4096), +15% / +7% on the up+gate /
-        // down GEMMs of 32 experts with a skewed 8192-row load, parity (0.92..1.06) elsewhere, where
-        // its static tile assignment loses what the deeper pipeline gains.
+        // down GEMMs of 32 experts with a skewed 8192-row load, +10% on the dense 8192 x 4096 x 7168
+        // product (four rounds); beyond ten rounds of tiles its static tile assignment loses what the
+        // deeper pipeline gains.
         const bool aligned = a.Prows % 256 == 0 && a.Qrows % 128 == 0 && a.red >= 384 && a.group != GROUP_MASKED;
         const int64_t cus = pf8_effective_cus();
-        const bool deep = aligned && (T128 <= cus || (a.group == GROUP_CONTIG && a.red >= 2048 && T128 <= 10 * cus));
+        const bool deep = aligned && (T128 <= cus || (a.red >= 2048 && T128 <= 10 * cus));
         if (deep) {
             // persistent: one workgroup per compute unit (or per tile of an XCD's run, if fewer)
             const int64_t per_xcd = (T128 + 7) / 8;
