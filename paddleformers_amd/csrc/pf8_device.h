@@ -209,8 +209,22 @@ __device__ __forceinline__ float expf_fixed(float x) {
     return __builtin_ldexpf(y, (int)n);
 }
 
-// silu(g) = g / (1 + exp(-g)), IEEE division
-__device__ __forceinline__ float silu_exact(float g) { return g / (1.0f + expf_fixed(-g)); }
+// silu(g) = g / (1 + exp(-g)) with the correctly rounded quotient, without the IEEE division sequence.
+// Numerator and denominator are both scaled by 1/8 (exact: g is a bf16 value, the denominator is at least
+// 1), which keeps the denominator below 2^125 where v_rcp_f32 still returns a normal number (the
+// exponential clamps at exp(88.5) = 2.7e38).  Then y = rcp refined by one Newton step, q0 = g' y,
+// r = fma(-q0, den', g'), q = fma(r, y, q0), and the sign of g is copied over (g = -0).  g is always a bf16
+// value in this library: the GPU test suite compares this routine with the CPU checker's division on every
+// one of the 65,536 bf16 inputs, bit for bit.
+__device__ __forceinline__ float silu_exact(float g) {
+    const float den = __builtin_fmaf(expf_fixed(-g), 0.125f, 0.125f);     // (1 + exp(-g)) / 8, same rounding
+    const float g8 = g * 0.125f;
+    float y = __builtin_amdgcn_rcpf(den);
+    y = __builtin_fmaf(__builtin_fmaf(-den, y, 1.0f), y, y);
+    const float q0 = g8 * y;
+    const float r = __builtin_fmaf(-q0, den, g8);
+    return __builtin_copysignf(__builtin_fmaf(r, y, q0), g);
+}
 
 // Contiguous-grouped GEMM with UE8M0 scales: which of the two kernels takes an expert load, from the
 // work-item list's header {paired 256-row items, 128-row blocks}.  Rounds of tiles per compute unit,
