@@ -3,7 +3,9 @@
 
 One "step" = one forward pass of the DeepSeek-V3-shaped FP8 MoE expert MLP over one batch of
 synthetic routed tokens (BASELINE config 3, one GPU's local share):
-    1x128 quant of X -> up+gate grouped GEMM -> fused SwiGLU + 1x128 requant -> down grouped GEMM.
+    1x128 quant of X -> up+gate grouped GEMM -> fused SwiGLU + 1x128 requant -> down grouped GEMM
+(the four launches of the reference's node; the form with the SwiGLU quantizer inside the GEMM's epilogue is timed
+beside it and reported as `swiglu_in_gemm_epilogue_ms_per_step`).
 Expert weights are quantised once before the timed region (the reference re-quantises them once
 per optimizer step in a callback, outside the MoE forward); that kernel is reported separately.
 
@@ -49,7 +51,7 @@ def traffic_from_summary(kernel_name):
 
 
 # the kernel the up+gate grouped GEMM of the headline workload runs on (what rocprofv3 --kernel-trace names it)
-ROOFLINE_KERNEL = "pf8::k_gemm_fwd_deep<1, 0>"
+ROOFLINE_KERNEL = "pf8::k_gemm_fwd_deep<1, 0, 0>"
 
 
 def zipf_counts(total, E, s, seed, n_empty=2, pad=128):
@@ -590,6 +592,25 @@ def main():
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2q, w2s), o3, m_idx)
         if evs: evs[4].record()
 
+    def step_one_launch():
+        """The same forward with SwiGLU and the requantization in the up+gate GEMM's epilogue (one launch, bit-identical
+        o2; the bf16 o1 is never written: what the node does when recompute_fwd_gate_up makes o1 disposable)."""
+        xq, xs = F8.fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True)
+        o2q, o2s = deep_gemm.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((xq, xs.T), (w1q, w1s), m_idx, None, using_pow2_scaling=True)
+        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2q, w2s), o3, m_idx)
+
+    # First the comparison leg: the same forward with the SwiGLU quantizer in the GEMM's epilogue, timed like the
+    # headline (W warm-up steps, K timed steps).  It runs first on purpose: after idle or memory-bound work (the setup
+    # above) this GPU needs some 15 ms of matrix load before its clocks settle, and a 25-step window that starts cold
+    # reads 5-14% slow (measured: 0.64-0.69 ms against 0.60 ms for the same step); whatever leg runs first pays that.
+    for _ in range(args.warmup):
+        step_one_launch()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for k in range(args.steps):
+        step_one_launch()
+    torch.cuda.synchronize()
+    ms_one_launch = (time.perf_counter() - t2) * 1e3 / args.steps
     # W warm-up steps, then EXACTLY K timed steps between two synchronisations: `value`.  No event is
     # recorded inside them: recording one idles the stream for about 6 us on this machine, and five per
     # step would charge the step 4-5% for its own instrumentation.
@@ -660,6 +681,7 @@ def main():
         "kernel_ms_median": {k: round(v, 4) for k, v in kmed.items()},
         "kernel_ms_min": {k: round(v, 4) for k, v in kmin.items()},
         "event_record_ms": round(event_overhead_ms, 4),
+        "swiglu_in_gemm_epilogue_ms_per_step": round(ms_one_launch, 4),
         "roofline": {
             "kernel": ROOFLINE_KERNEL + " (up+gate grouped GEMM)",
             "bound": "mfma",

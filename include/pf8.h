@@ -201,6 +201,22 @@ int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_lay
                                    const float* sb, int E, int64_t Mtot, int64_t N, int64_t K,
                                    const int32_t* m_indices, uint16_t* out, pf8_stream_t stream);
 
+/* The up+gate grouped GEMM with the activation quantizer of the down projection in its epilogue: the two calls of
+ * FP8GroupGemmMlpFunctionNode.forward -- deep_gemm.m_grouped_fp8_gemm_nt_contiguous (transformers/fp8_utils.py:949-954)
+ * and fused_weighted_swiglu_act_quant(o1, probs, using_pow2_scaling) (:981-987; un-fused definition ernie
+ * token_dispatcher/fp8_utils.py:996-1004) -- as one launch.  a, sa, m_indices as in pf8_grouped_gemm_nt_contiguous;
+ * b e4m3 [E, 2I, K] with every expert's gate rows first and its up rows after them (the stacked [H, 2I] weight
+ * transposed, as fused_stack_transpose_quant(..., transpose=True) writes it), sb fp32 [E, 2I/128, K/128]; probs fp32
+ * [Mtot] or NULL.  Outputs: q e4m3 [Mtot, I] and s fp32 [Mtot, I/128] of
+ * quant_1x128( bf16( bf16(silu(o1[:, :I]) * o1[:, I:]) * probs ) ), bit-identical to the two separate calls, and,
+ * when o1 is not NULL, the bf16 GEMM result o1 [Mtot, 2I] itself (the node keeps it for backward unless
+ * recompute_fwd_gate_up is set, :1263-1267).  Mtot and I multiples of 128, K a multiple of 128 and >= 384; other shapes
+ * return PF8_EINVAL (make the two calls). */
+int pf8_grouped_gemm_swiglu_quant_nt_contiguous(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b,
+                                                const float* sb, int E, int64_t Mtot, int64_t I, int64_t K,
+                                                const int32_t* m_indices, const float* probs, uint16_t* o1,
+                                                uint8_t* q, float* s, int pow2, pf8_stream_t stream);
+
 /* The same two GEMMs with power-of-two scales held as UE8M0 exponent bytes (scale = 2^(byte-127)),
  * the form `use_ue8m0` selects for deep_gemm (transformers/configuration_utils.py:454-459; byte
  * format quantization/checkpoint_dequant.py:121-131).  Both operands must have been quantized with

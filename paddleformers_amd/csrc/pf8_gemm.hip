@@ -48,6 +48,13 @@ struct GemmArgs {
     const int32_t* pair_list;   // UE8M0 forward: when set, the kernel runs only if the paired-tile kernel declines
     int cus;                    //   (header of its work-item list, compute units both assume)
     int pow2_scales;            // wgrad: every scale is a power of two (applied inside the MFMA)
+    // fused up+gate -> SwiGLU -> 1x128 requantization (k_gemm_fwd_deep<.., .., 1>): P holds [gate rows | up rows],
+    // Prows = 2 * inter; `out` (bf16 [Qrows, 2 inter]) may be null
+    int64_t inter;              // I: columns of the quantized activation
+    const float* probs;         // per-row factor or null
+    uint8_t* q2;                // e4m3 [Qrows, inter]
+    float* s2;                  // fp32 [Qrows, inter / 128]
+    int pow2_out;               // scale rule of the requantization
 };
 
 // 16-byte chunk c of LDS row `row` lives at chunk c ^ swz_key(row): the 16 rows a fragment read touches
@@ -339,7 +346,15 @@ __device__ __forceinline__ void dma16_s(uint32_t voff, const uint8_t* sbase, uin
 // the kernel is the same, a scale is decoded where the block's factors are formed.
 __device__ __forceinline__ float e8m0_to_f32(uint32_t b) { return u2f(b ? b << 23 : 0x00400000u); }
 
-template <int SQL, int SF = 0>
+// FUSE = 1: the up+gate GEMM of the MoE MLP with SwiGLU, the probability factor and the 1x128 requantization in its
+// epilogue.  A tile's 256 weight rows are 128 gate rows and the 128 up rows of the same output columns (two row ranges
+// of the stacked [gate | up] weight, nothing is re-laid out), so the wavefront pair (wq, 0) / (wq, 1) holds gate and up
+// of the same 64 x 128 outputs.  Both round to bf16 (that IS o1, stored as well when the caller wants it), meet in the
+// LDS staging rows, and each wavefront turns 16 rows per pass into e4m3 bytes and one scale per row: a row of 128
+// outputs is the 16 lanes of a DPP row, exactly the tile of the standalone SwiGLU quantizer, whose arithmetic is
+// restated operation for operation (bf16(silu(g) * u), bf16(. * p), amax, scale, quotient), so bytes and scales are
+// bit-identical to the un-fused pair of launches.
+template <int SQL, int SF = 0, int FUSE = 0>
 __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     using ST = typename std::conditional<SF == 1, uint8_t, float>::type;
     if (SF == 1 && a.pair_list && e8_paired_tiles_win(a.pair_list, a.Prows / 256, a.cus)) return;
@@ -355,6 +370,10 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
 
     const int64_t p_tiles = a.Prows / 256, q_tiles = a.Qrows / BQ;
     const int64_t T = p_tiles * q_tiles;
+    // FUSE: tile p takes weight rows [128 p, 128 p + 128) (gate) and inter + the same (up)
+    const int64_t p_rows_per_tile = FUSE ? 128 : 256;
+    const int64_t up_off = FUSE ? a.inter * a.red : 128 * a.red;      // bytes from a tile's first half to its second
+    const int64_t IB = FUSE ? a.inter / 128 : 0;
     // consecutive workgroups go round-robin to the 8 XCDs: every XCD owns a contiguous run of
     // logical tiles (groups of 16 q-tiles x all p-tiles), walked W tiles at a time by its W workgroups
     const int64_t per_xcd = (T + 7) / 8;
@@ -382,9 +401,9 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     if (grouped) ce = __builtin_amdgcn_readfirstlane(a.m_indices[cq * BQ]);
     int c_rows = ce < 0 ? 0 : BQ;          // rows of the tile that are stored (none for a padding tile)
     if (ce < 0) ce = 0;
-    const uint8_t* c_ptile = a.p + ((int64_t)ce * a.Prows + cp * 256) * a.red;
+    const uint8_t* c_ptile = a.p + ((int64_t)ce * a.Prows + cp * p_rows_per_tile) * a.red;
     const uint8_t* c_qtile = a.q + cq * BQ * a.red;
-    const ST* c_spb = sp_base + ((int64_t)ce * PB + cp * 2 + wp) * KB;
+    const ST* c_spb = sp_base + ((int64_t)ce * PB + (FUSE ? cp + wp * IB : cp * 2 + wp)) * KB;
     const ST* c_sq0 = SQL == 0 ? sq_base + (cq * BQ + wq * 64) * KB : sq_base + cq * BQ + wq * 64;
     const uint8_t* n_ptile = c_ptile;
     const uint8_t* n_qtile = c_qtile;
@@ -415,7 +434,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
 
 #define PF8_COPY(i_, pt_, qt_, stage_)                                                                 \
     do {                                                                                               \
-        if ((i_) < 8) dma16_s(c_off, (pt_) + (i_) * copy_step, lds_base + (stage_) * STAGE + ((i_) * 4 + wave) * 1024); \
+        if ((i_) < 4) dma16_s(c_off, (pt_) + (i_) * copy_step, lds_base + (stage_) * STAGE + ((i_) * 4 + wave) * 1024); \
+        else if ((i_) < 8) dma16_s(c_off, (pt_) + up_off + ((i_) - 4) * copy_step, lds_base + (stage_) * STAGE + ((i_) * 4 + wave) * 1024); \
         else dma16_s(c_off, (qt_) + ((i_) - 8) * copy_step, lds_base + (stage_) * STAGE + Q_OFS + (((i_) - 8) * 4 + wave) * 1024); \
     } while (0)
 #define PF8_LOAD_S(sq_, sp_)                                                                           \
@@ -462,9 +482,9 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                 if (n_valid) {
                     n_rows = ne < 0 ? 0 : BQ;
                     const int e = ne < 0 ? 0 : ne;
-                    n_ptile = a.p + ((int64_t)e * a.Prows + np * 256) * a.red;
+                    n_ptile = a.p + ((int64_t)e * a.Prows + np * p_rows_per_tile) * a.red;
                     n_qtile = a.q + nq * BQ * a.red;
-                    n_spb = sp_base + ((int64_t)e * PB + np * 2 + wp) * KB;
+                    n_spb = sp_base + ((int64_t)e * PB + (FUSE ? np + wp * IB : np * 2 + wp)) * KB;
                     n_sq0 = SQL == 0 ? sq_base + (nq * BQ + wq * 64) * KB : sq_base + nq * BQ + wq * 64;
                 } else {
                     // past the last tile the copies and scale loads re-read this tile's first blocks:
@@ -544,7 +564,68 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         // block's barrier with its fragment reads returned, and no copy targets the stage before the
         // next block starts.  Each wavefront stages 32 of its 64 rows at a time in a private slice
         // (LDS operations of one wavefront execute in order) and stores whole 256-byte rows.
-        {
+        if (FUSE) {
+            constexpr int EP_LD = 272;                   // 128 bf16 per row + 16 B pad
+            const int last = cur == 0 ? 2 : cur - 1;
+            uint8_t* ep0 = lds + last * STAGE;
+            uint8_t* ep = ep0 + wave * (32 * EP_LD);                             // this wavefront's rows: gate (wp = 0) or up (wp = 1)
+            const uint8_t* ep_g = ep0 + (wq * 2) * (32 * EP_LD);                 // the pair's gate rows
+            const uint8_t* ep_u = ep0 + (wq * 2 + 1) * (32 * EP_LD);             // the pair's up rows
+            uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
+            const int er = lane >> 4, ec = lane & 15;
+            const int64_t col = (wp ? a.inter : 0) + cp * 128 + ec * 8;          // column of o1
+            const bool has_p = a.probs != nullptr;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int qh = 0; qh < 2; ++qh) {
+                    const int qs = half * 2 + qh;
+#pragma unroll
+                    for (int ps = 0; ps < NPS; ++ps) {
+                        uint2 o;
+                        o.x = pack_bf16(acc[ps][qs][0], acc[ps][qs][1]);
+                        o.y = pack_bf16(acc[ps][qs][2], acc[ps][qs][3]);
+                        *reinterpret_cast<uint2*>(ep + (qh * 16 + li) * EP_LD + (ps * 16 + 4 * kg) * 2) = o;
+                    }
+                }
+                if (outb) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int rl = er + 4 * i;
+                        const int64_t row = cq * BQ + wq * 64 + half * 32 + rl;
+                        const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
+                        if (c_rows) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
+                    }
+                }
+                __syncthreads();      // the pair's gate and up rows are both staged
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int rl = wp * 16 + it * 4 + er;                         // this wavefront's 16 of the pass's 32 rows
+                    const int64_t row = cq * BQ + wq * 64 + half * 32 + rl;
+                    const uint4 wg = *reinterpret_cast<const uint4*>(ep_g + rl * EP_LD + ec * 16);
+                    const uint4 wu = *reinterpret_cast<const uint4*>(ep_u + rl * EP_LD + ec * 16);
+                    const float pr = has_p ? a.probs[row] : 1.0f;
+                    float gv[8], uv[8], v[8];
+                    unpack8(wg, gv);
+                    unpack8(wu, uv);
+                    uint32_t am = 0;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        float y = round_bf16(silu_exact(gv[i]) * uv[i]);
+                        if (has_p) y = round_bf16(y * pr);
+                        v[i] = y;
+                        am = umax(am, f2u(y) & 0x7FFFFFFFu);
+                    }
+                    const TileScale t = make_scale(row16_max(am), a.pow2_out != 0);
+                    const uint2 o = quant8(v, t);
+                    if (c_rows) {
+                        st8(a.q2 + row * a.inter + cp * 128 + ec * 8, o);
+                        if (ec == 0) a.s2[row * IB + cp] = t.s;
+                    }
+                }
+                if (half == 0) __syncthreads();      // everyone has read the first pass's rows before they are overwritten
+            }
+        } else {
             constexpr int EP_LD = 272;                   // 128 bf16 per row + 16 B pad
             const int last = cur == 0 ? 2 : cur - 1;
             uint8_t* ep = lds + last * STAGE + wave * (32 * EP_LD);
@@ -882,6 +963,8 @@ static int ensure_lds_attr() {
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
     done.fetch_or(bit, std::memory_order_release);
     return PF8_OK;
@@ -945,6 +1028,38 @@ extern "C" int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa,
     const int64_t tiles = ((N + 127) / 128) * (Mtot / 128);
     PF8_REQUIRE(tiles <= 0x7FFFFFFF, "too many tiles");
     return launch_gemm(g, MODE_FWD, dim3((unsigned)tiles), (hipStream_t)stream, __func__);
+}
+
+extern "C" int pf8_grouped_gemm_swiglu_quant_nt_contiguous(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b,
+                                                           const float* sb, int E, int64_t Mtot, int64_t I, int64_t K,
+                                                           const int32_t* m_indices, const float* probs, uint16_t* o1, uint8_t* q,
+                                                           float* s, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(E >= 0 && Mtot >= 0 && I >= 0 && K >= 0, "negative shape");
+    PF8_REQUIRE(K % 128 == 0 && K >= 384, "K must be a multiple of 128 and at least 384");
+    PF8_REQUIRE(I % 128 == 0, "I must be a multiple of 128");
+    PF8_REQUIRE(Mtot % 128 == 0, "Mtot must be a multiple of 128 (expert segments are padded to 128 rows)");
+    if (Mtot == 0 || I == 0 || E == 0) return PF8_OK;
+    PF8_REQUIRE(a && sa && b && sb && q && s && m_indices, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(a) && PF8_ALIGNED16(b) && PF8_ALIGNED16(o1) && (reinterpret_cast<uintptr_t>(q) & 7u) == 0,
+                "a, b, o1 must be 16-byte aligned and q 8-byte aligned");
+    PF8_REQUIRE(sa_layout == 0 || sa_layout == 1, "sa_layout must be 0 or 1");
+    PF8_REQUIRE(K <= (1ll << 24) && I <= (1ll << 24), "shape too large");
+    int rc = ensure_lds_attr();
+    if (rc) return rc;
+    GemmArgs g = {};
+    g.p = b; g.q = a; g.sp = sb; g.sq = sa; g.out = o1;
+    g.Prows = 2 * I; g.Qrows = Mtot; g.red = K; g.ldo = 2 * I; g.sq_layout = sa_layout; g.group = GROUP_CONTIG; g.E = E;
+    g.m_indices = m_indices;
+    g.inter = I; g.probs = probs; g.q2 = q; g.s2 = s; g.pow2_out = pow2;
+    const int64_t T128 = (I / 128) * (Mtot / 128), per_xcd = (T128 + 7) / 8;
+    PF8_REQUIRE(T128 <= 0x7FFFFFFF, "too many tiles");
+    int64_t w = pf8_effective_cus() / 8;
+    if (w < 1) w = 1;
+    if (w > per_xcd) w = per_xcd;
+    dim3 gd((unsigned)(8 * w), 1);
+    if (sa_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0, 0, 1>), gd, dim3(256), 147456, (hipStream_t)stream, g);
+    else hipLaunchKernelGGL((k_gemm_fwd_deep<1, 0, 1>), gd, dim3(256), 147456, (hipStream_t)stream, g);
+    return pf8_check_launch(__func__);
 }
 
 extern "C" int pf8_grouped_gemm_nt_masked(const uint8_t* a, const float* sa, const uint8_t* b, const float* sb, int E, int64_t Mmax,

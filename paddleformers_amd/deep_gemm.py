@@ -200,6 +200,57 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
     return out
 
 
+def swiglu_quant_fusable(Mtot: int, N: int, K: int, a_scale: Optional[torch.Tensor] = None,
+                         b_scale: Optional[torch.Tensor] = None) -> bool:
+    """Shapes and scale kinds m_grouped_fp8_gemm_nt_contiguous_swiglu_quant takes: fp32 scales, whole 128-row and
+    128-column tiles of both halves, at least three K blocks."""
+    if (a_scale is not None and _is_ue8m0(a_scale)) or (b_scale is not None and _is_ue8m0(b_scale)):
+        return False
+    return Mtot > 0 and Mtot % 128 == 0 and N % 256 == 0 and N > 0 and K % 128 == 0 and K >= 384
+
+
+def m_grouped_fp8_gemm_nt_contiguous_swiglu_quant(a, b, m_indices: torch.Tensor, probs: Optional[torch.Tensor] = None,
+                                                  using_pow2_scaling: bool = False, out: Optional[torch.Tensor] = None):
+    """The up+gate grouped GEMM of the MoE MLP with fused_weighted_swiglu_act_quant in its epilogue: one launch for
+    transformers/fp8_utils.py:949-954 followed by :981-987.  a [Mtot, K] + sa, b [E, 2I, K] (gate rows, then up rows)
+    + sb [E, 2I/128, K/128], fp32 scales; probs fp32 [Mtot] (or [Mtot, 1]) or None.  Returns (q [Mtot, I] e4m3,
+    s [Mtot, I/128] fp32), bit-identical to m_grouped_fp8_gemm_nt_contiguous + fused_weighted_swiglu_act_quant;
+    `out` (bf16 [Mtot, 2I], optional) also receives the GEMM result o1.  No counterpart of its own in the reference."""
+    (ta, sa), (tb, sb) = _check_pair(a, "a"), _check_pair(b, "b")
+    _dev(m_indices, "m_indices")
+    Mtot, K = ta.shape
+    if tb.dim() != 3:
+        raise ValueError("b must be [E, 2I, K]")
+    E, N, K2 = tb.shape
+    if K != K2 or not swiglu_quant_fusable(Mtot, N, K, sa, sb):
+        raise ValueError("shape or scale kind outside the fused kernel: Mtot % 128 == 0, 2I % 256 == 0, K % 128 == 0, K >= 384, fp32 scales")
+    I = N // 2
+    if m_indices.dtype != torch.int32 or m_indices.numel() != Mtot:
+        raise ValueError("m_indices must be int32 with one entry per row")
+    if out is not None:
+        _dev(out, "out")
+        if tuple(out.shape) != (Mtot, N) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+            raise ValueError(f"out must be a contiguous bfloat16 [{Mtot}, {N}] tensor")
+    if probs is not None:
+        _dev(probs, "probs")
+        probs = probs.reshape(-1)
+        if probs.numel() != Mtot:
+            raise ValueError("probs must have one entry per row")
+        probs = probs.float().contiguous()
+    ta = ta if ta.is_contiguous() else ta.contiguous()
+    tb = tb if tb.is_contiguous() else tb.contiguous()
+    m_indices = m_indices if m_indices.is_contiguous() else m_indices.contiguous()
+    sa, lay = _scale_layout_of(sa, Mtot, K // 128, "a scale")
+    if tuple(sb.shape) != (E, N // 128, K // 128) or sb.dtype != torch.float32:
+        raise ValueError(f"b scale must be float32 [{E}, {N // 128}, {K // 128}]")
+    sb = sb if sb.is_contiguous() else sb.contiguous()
+    q = torch.empty((Mtot, I), dtype=FP8, device=ta.device)
+    s = torch.empty((Mtot, I // 128), dtype=torch.float32, device=ta.device)
+    _lib.call("pf8_grouped_gemm_swiglu_quant_nt_contiguous", _p(ta), _p(sa), lay, _p(tb), _p(sb), E, Mtot, I, K, _p(m_indices),
+              _p(probs), _p(out), _p(q), _p(s), int(bool(using_pow2_scaling)), _stream())
+    return q, s
+
+
 def m_grouped_fp8_gemm_nt_masked(a, b, out: torch.Tensor, masked_m: torch.Tensor, expected_m: int):
     """Grouped GEMM with a fixed capacity per expert.
 

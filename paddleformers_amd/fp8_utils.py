@@ -604,6 +604,12 @@ class FP8GroupGemmMlpFunctionNode:
         # backward quantizes out_grad and do1 twice each (row-wise for the dgrad GEMM, transposed per expert
         # for the wgrad GEMM); with this set both come from one read of the gradient, bit-identical
         self.fuse_bwd_quant = True
+        # forward may run the up+gate grouped GEMM with SwiGLU, the probability factor and the 1x128 requantization in
+        # its epilogue (one launch, bit-identical to the two calls of fp8_utils.py:949-954 and :981-987).  Measured on
+        # config 3 the one launch takes as long as the two (SwiGLU is bound by the vector ALU and the persistent GEMM
+        # has nothing to hide it behind), so what it buys is memory: with recompute_fwd_gate_up the bf16 o1 is never
+        # written.  None = on exactly then; True / False force it.
+        self.fuse_swiglu_epilogue = None
         self._group_items = None
         self.m_indices = None
         self.input = None
@@ -849,6 +855,12 @@ class FP8GroupGemmMlpFunctionNode:
         expert_w1 = [x.w1 for x in self.experts if x is not None]
         expert_w2 = [x.w2 for x in self.experts if x is not None]
         num_expert = len(expert_w1)
+        in_scale = hs_out[1] if isinstance(hs_out, tuple) else (self.input_scale if hs_out is None else None)
+        fuse = self.recompute_fwd_gate_up if self.fuse_swiglu_epilogue is None else self.fuse_swiglu_epilogue
+        if (fuse and not self.is_split_group_gemm and not self.use_ue8m0
+                and (in_scale is None or in_scale.dtype == torch.float32)
+                and deep_gemm.swiglu_quant_fusable(shape[0], expert_w1[0].shape[1], shape[1])):
+            return self._forward_fused(hs_out, unzipped_probs, expert_w1, expert_w2, num_expert, tokens_per_expert, m_indices)
         o1 = self.fwd_gate_up(hs_out, expert_w1, num_expert, tokens_per_expert, m_indices)
         if not self.recompute_fwd_gate_up:
             self.o1 = o1
@@ -856,6 +868,38 @@ class FP8GroupGemmMlpFunctionNode:
         else:
             clear_o1 = True
         return self.fwd_down(o1, unzipped_probs, expert_w2, num_expert, tokens_per_expert, clear_o1=clear_o1, m_indices=m_indices)
+
+    def _forward_fused(self, x, unzipped_probs, expert_w1, expert_w2, num_expert, tokens_per_expert, m_indices=None):
+        """fwd_gate_up + the quantizer half of fwd_down as one launch, then the down GEMM.  Same cached state as the
+        two methods leave behind (m_indices, input_fp8 / input_scale, o1 unless recomputed).  The caller has checked
+        that the fused kernel takes the shapes."""
+        if self.m_indices is None:
+            self.m_indices = self.gen_m_indices(tokens_per_expert)
+        w1_t_quant, w1_t_scale = self._stacked(expert_w1, True, num_expert)
+        if x is None:
+            x_fp8, x_scale = self.input_fp8, self.input_scale
+            assert x_fp8 is not None and x_scale is not None
+        elif isinstance(x, tuple):
+            x_fp8, x_scale = x
+            x_scale = x_scale.t().contiguous().t()
+        else:
+            x_fp8, x_scale = F8.fp8_quant_blockwise(x, output_scale_transpose=True, quant_method="1x128", input_transpose=False)
+            x_scale = x_scale.T
+        Mtot, K = x_fp8.shape
+        keep_o1 = not self.recompute_fwd_gate_up
+        o1 = torch.empty([Mtot, w1_t_quant.shape[1]], dtype=expert_w1[0].dtype, device=x_fp8.device) if keep_o1 else None
+        o2_fp8, o2_scale = deep_gemm.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant(
+            (x_fp8, x_scale), (w1_t_quant, w1_t_scale), self.m_indices if m_indices is None else m_indices,
+            unzipped_probs.squeeze(-1), using_pow2_scaling=True, out=o1)
+        if m_indices is None:
+            self.input_fp8 = x_fp8
+            self.input_scale = x_scale
+        if keep_o1:
+            self.o1 = o1
+        w2_quant, w2_scale = self._stacked(expert_w2, True, num_expert)
+        o3 = torch.empty([Mtot, w2_quant.shape[1]], dtype=expert_w1[0].dtype, device=x_fp8.device)
+        self._grouped_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, o3, m_indices if self.fwd_subbatch else self.m_indices)
+        return o3
 
     @torch.no_grad()
     def backward(self, out_grad, unzipped_probs, tokens_per_expert, input_fp8_slice=None, input_scale_slice=None, m_indices=None,

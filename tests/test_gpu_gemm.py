@@ -429,3 +429,66 @@ def test_grouped_wgrad_equals_per_expert_loop(dg):
         if r:
             exp = O.gemm_nt_1d1d_f32(G.from_torch_fp8(a_t[e]), sa_t[e].cpu().numpy(), G.from_torch_fp8(b_t[e]), sb_t[e].cpu().numpy())
             assert G.rel_fro(outp0[e].cpu().numpy(), exp) <= F32_FRO_MFMA_ACC, f"expert {e} vs oracle (scales inside the MFMA)"
+
+
+# ---------------------------------------------------------------------------------------------
+# up+gate grouped GEMM with SwiGLU and the requantization in its epilogue
+# ---------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("rows,K,I", [([128, 0, 256, 128], 512, 256), ([256, 0, 640, 128, 384, 512], 2048, 384), ([128] * 5, 384, 128)])
+@pytest.mark.parametrize("lay", [0, 1])
+@pytest.mark.parametrize("with_probs,pow2,few", [(True, True, False), (False, False, False), (True, False, True)])
+def test_grouped_gemm_swiglu_quant_equals_the_two_launches(dg, request, rows, K, I, lay, with_probs, pow2, few):
+    """q, s and o1 of the one-launch form are bit-identical to m_grouped_fp8_gemm_nt_contiguous followed by
+    fused_weighted_swiglu_act_quant, and equal the oracle chain: o1 within the GEMM bars, bytes and scales of the
+    requantization exact given o1.  `few`: eight compute units, so every workgroup walks several tiles."""
+    from paddleformers_amd import functional as F8
+
+    if few:
+        request.getfixturevalue("few_cus")
+    E, N = len(rows), 2 * I
+    a, sa, b, sb, m_idx = _grouped_case(E, N, K, rows, seed=sum(rows) + K + I)
+    Mtot = a.shape[0]
+    probs = np.random.default_rng(3).random(Mtot, dtype=np.float32) * 0.5 + 0.25 if with_probs else None
+    ta, tb, tm = G.to_torch_fp8(a), G.to_torch_fp8(b), torch.from_numpy(m_idx).cuda()
+    tsa = torch.from_numpy(np.ascontiguousarray(sa.T)).cuda().t() if lay else torch.from_numpy(sa).cuda()
+    tsb = torch.from_numpy(sb).cuda()
+    tp = None if probs is None else torch.from_numpy(probs).cuda()
+    o1_two = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dg.m_grouped_fp8_gemm_nt_contiguous((ta, tsa), (tb, tsb), o1_two, tm)
+    q_two, s_two = F8.fused_weighted_swiglu_act_quant(o1_two, tp, using_pow2_scaling=pow2)
+    o1 = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    q, s = dg.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((ta, tsa), (tb, tsb), tm, tp, using_pow2_scaling=pow2, out=o1)
+    assert torch.equal(o1.view(torch.int16), o1_two.view(torch.int16))
+    assert torch.equal(q.view(torch.uint8), q_two.view(torch.uint8)) and torch.equal(s, s_two)
+    q_no, s_no = dg.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((ta, tsa), (tb, tsb), tm, tp, using_pow2_scaling=pow2)
+    assert torch.equal(q_no.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s_no, s)
+    # against the oracle: the GEMM, then the requantization of the GPU's own o1
+    exp = O.grouped_gemm_nt_contiguous(a, sa, b, sb, m_idx)
+    got = G.from_torch_bf16(o1)
+    assert G.rel_fro(_bf(got), _bf(exp)) <= BLOCK_FRO
+    eq, es = O.swiglu_weighted_quant(got, probs, 0, pow2)
+    assert np.array_equal(G.from_torch_fp8(q), eq) and np.array_equal(s.cpu().numpy(), es)
+
+
+def test_grouped_gemm_swiglu_quant_skips_padding_tiles_and_rejects_other_shapes(dg):
+    E, K, I = 2, 512, 128
+    rows = [128, 128]
+    a, sa, b, sb, m_idx = _grouped_case(E, 2 * I, K, rows, seed=77)
+    m_idx[128:] = -1
+    ta, tb = G.to_torch_fp8(a), G.to_torch_fp8(b)
+    o1 = torch.full((256, 2 * I), 7.0, dtype=torch.bfloat16, device="cuda")
+    q, s = dg.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((ta, torch.from_numpy(sa).cuda()), (tb, torch.from_numpy(sb).cuda()),
+                                                            torch.from_numpy(m_idx).cuda(), None, out=o1)
+    assert (o1[128:] == 7.0).all() and not (o1[:128] == 7.0).all()
+    eq, es = O.swiglu_weighted_quant(G.from_torch_bf16(o1[:128]), None, 0, False)
+    assert np.array_equal(G.from_torch_fp8(q[:128]), eq) and np.array_equal(s[:128].cpu().numpy(), es)
+    with pytest.raises(ValueError):      # two K blocks only
+        dg.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((ta[:, :256].contiguous(), torch.from_numpy(sa[:, :2].copy()).cuda()),
+                                                         (tb[:, :, :256].contiguous(), torch.from_numpy(sb[:, :, :2].copy()).cuda()),
+                                                         torch.from_numpy(m_idx).cuda(), None)
+    with pytest.raises(ValueError):      # UE8M0 scales take the two launches
+        dg.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((ta, torch.ones((256, 4), dtype=torch.uint8, device="cuda")),
+                                                         (tb, torch.ones((E, 2, 4), dtype=torch.uint8, device="cuda")),
+                                                         torch.from_numpy(m_idx).cuda(), None)

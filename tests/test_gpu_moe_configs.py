@@ -52,7 +52,7 @@ class _Recorder:
         from paddleformers_amd import functional as F8
 
         self._stack = contextlib.ExitStack()
-        for mod, names in ((F8, self.F8_NAMES), (deep_gemm, ["m_grouped_fp8_gemm_nt_contiguous"])):
+        for mod, names in ((F8, self.F8_NAMES), (deep_gemm, ["m_grouped_fp8_gemm_nt_contiguous", "m_grouped_fp8_gemm_nt_contiguous_swiglu_quant"])):
             for name in names:
                 orig = getattr(mod, name)
 
@@ -204,16 +204,27 @@ def _build(E, H, I, routed, zipf_s, seed, n_empty, ue8m0=False):
 
 
 def _check_forward(rec, node, x, probs, rows, pow2_in, tag):
+    """Checks every launch of one recorded forward; returns o1."""
     qx = rec.named("fp8_quant_blockwise")
     gemms = rec.named("m_grouped_fp8_gemm_nt_contiguous")
     sw = rec.named("fused_weighted_swiglu_act_quant")
-    assert len(qx) == 1 and len(gemms) == 2 and len(sw) == 1, [c[0] for c in rec.calls]
+    fused = rec.named("m_grouped_fp8_gemm_nt_contiguous_swiglu_quant")
     xq, xs = qx[0][3]
     _check_quant_rows(x, xq, xs, rows, pow2_in, f"{tag} quant(X)")
-    _check_grouped_gemm(gemms[0], rows, f"{tag} up+gate")
+    if fused:
+        # one launch for up+gate GEMM, SwiGLU and requantization: its o1 output is checked like the GEMM's own
+        assert len(qx) == 1 and len(gemms) == 1 and not sw, [c[0] for c in rec.calls]
+        _, fargs, fkw, (o2q, o2s) = fused[0]
+        o1 = fkw["out"]
+        assert o1 is not None and fkw["using_pow2_scaling"] is True
+        _check_grouped_gemm(("gemm", (fargs[0], fargs[1], o1, fargs[2]), {}, None), rows, f"{tag} up+gate (fused launch)")
+        gemms = [None, gemms[0]]
+    else:
+        assert len(qx) == 1 and len(gemms) == 2 and len(sw) == 1, [c[0] for c in rec.calls]
+        _check_grouped_gemm(gemms[0], rows, f"{tag} up+gate")
+        o1 = sw[0][1][0]
+        o2q, o2s = sw[0][3]
     # SwiGLU + requant (power-of-two scales) of the GPU's own o1, bit-exact on the slabs
-    o1 = sw[0][1][0]
-    o2q, o2s = sw[0][3]
     for lo, _, label in _slab_tiles(rows):
         eq, es = O.swiglu_weighted_quant(G.from_torch_bf16(o1[lo:lo + 128]), probs[lo:lo + 128, 0].cpu().numpy(), 0, True)
         msg = G.mismatch_report(G.from_torch_fp8(o2q[lo:lo + 128]), eq, f"{tag} o2 bytes, {label}")
@@ -224,16 +235,31 @@ def _check_forward(rec, node, x, probs, rows, pow2_in, tag):
     return o1
 
 
-def test_config3_forward_at_full_size():
+@pytest.mark.parametrize("fused", [True, False])
+def test_config3_forward_at_full_size(fused):
     """32 experts, hidden 7168, intermediate 2048, 8192 routed rows, Zipf(1.1), two empty experts (the
-    benchmark's workload): quant -> up+gate -> SwiGLU+requant -> down."""
+    benchmark's workload): quant -> up+gate -> SwiGLU+requant -> down, with the middle two as one launch
+    (the node's default) and as two."""
     torch.backends.cuda.matmul.allow_tf32 = False
     node, experts, x, probs, rows, counts, _ = _build(32, 7168, 2048, 8192, 1.1, seed=3, n_empty=2)
+    node.fuse_swiglu_epilogue = fused
     assert (counts == 0).sum() >= 2 and sum(rows) == 9984
     with _Recorder() as rec:
         o3 = node.forward(x, probs, rows)
     assert tuple(o3.shape) == (sum(rows), 7168)
-    _check_forward(rec, node, x, probs, rows, False, "config 3")
+    assert bool(rec.named("m_grouped_fp8_gemm_nt_contiguous_swiglu_quant")) == fused
+    _check_forward(rec, node, x, probs, rows, False, "config 3" + (" fused" if fused else ""))
+    if fused:
+        # the one-launch forward is the two-launch forward, bit for bit, with and without o1 being kept
+        o1_fused = node.o1
+        node.fuse_swiglu_epilogue = False
+        o3_two = node.forward(None, probs, rows)
+        assert torch.equal(o3.view(torch.int16), o3_two.view(torch.int16))
+        assert torch.equal(o1_fused.view(torch.int16), node.o1.view(torch.int16))
+        node.fuse_swiglu_epilogue, node.recompute_fwd_gate_up = True, True
+        node.o1 = None
+        o3_no_o1 = node.forward(None, probs, rows)
+        assert node.o1 is None and torch.equal(o3.view(torch.int16), o3_no_o1.view(torch.int16))
     # rows of padding stay exactly zero through the whole pipeline (zero input rows, zero probabilities)
     off = 0
     for e, r in enumerate(rows):
