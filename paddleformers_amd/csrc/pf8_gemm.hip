@@ -375,7 +375,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     const int64_t up_off = FUSE ? a.inter * a.red : 128 * a.red;      // bytes from a tile's first half to its second
     const int64_t IB = FUSE ? a.inter / 128 : 0;
     // consecutive workgroups go round-robin to the 8 XCDs: every XCD owns a contiguous run of
-    // logical tiles (groups of 16 q-tiles x all p-tiles), walked W tiles at a time by its W workgroups
+    // logical tiles (groups of q-tiles x all p-tiles, see below), walked W tiles at a time by its W workgroups
     const int64_t per_xcd = (T + 7) / 8;
     const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, W = gridDim.x >> 3;
     const int64_t KB = a.red / 128;
@@ -383,10 +383,61 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     const int64_t q_rows_total = a.Qrows;
     const bool grouped = a.group == GROUP_CONTIG;
 
+    // Grouped layout with at most 256 row tiles: the row tiles are cut into groups that never span two experts
+    // (at most 12 tiles each), and the tiles of a group are walked q fastest, p slowest.  The 32 workgroups of an
+    // XCD then work on one or two weight strips of ONE expert at a time and on the few activation strips of that
+    // group, instead of on 16 activation strips that belong to a dozen experts.  Measured on config 3 (32 experts,
+    // Zipf load) against groups of 16 row tiles cut without regard to experts: the L2s miss 1.33 GB instead of
+    // 1.74 GB per up+gate launch (hit rate 64% against 53%) and 0.74 GB instead of 0.96 GB on the down GEMM; the
+    // launches get 3% and 2% shorter.  seg_tab[q] = first tile of q's group | tiles in it << 16.
+    __shared__ uint32_t seg_tab[256];
+    __shared__ int seg_wave_max[4];
+    const bool ordered = grouped && q_tiles <= 256;
+    if (ordered) {
+        constexpr int CAP = 12;
+        const int t = tid, qt = (int)q_tiles;
+        // expert of tile t and of its neighbours; every padding tile counts as expert -1, tiles past the end as -2
+        auto expert_of = [&](int i) -> int {
+            if (i < 0) return -3;
+            if (i >= qt) return -2;
+            const int e = a.m_indices[(int64_t)i * BQ];
+            return e < 0 ? -1 : e;
+        };
+        const int e_me = expert_of(t), e_prev = expert_of(t - 1), e_next = expert_of(t + 1);
+        int v = (t < qt && e_me != e_prev) ? t : 0;            // first tile of a run of one expert
+#pragma unroll
+        for (int dlt = 1; dlt < 64; dlt <<= 1) {
+            const int o = __shfl_up(v, dlt, 64);
+            if (lane >= dlt && o > v) v = o;
+        }
+        if (lane == 63) seg_wave_max[wave] = v;
+        __syncthreads();
+        for (int w = 0; w < wave; ++w) v = seg_wave_max[w] > v ? seg_wave_max[w] : v;
+        const int run_start = v;
+        if (t < qt && e_me != e_next) seg_tab[run_start] = (uint32_t)(t - run_start + 1);
+        __syncthreads();
+        const int run_len = t < qt ? (int)seg_tab[run_start] : 0;
+        __syncthreads();
+        if (t < qt) {
+            const int gs = run_start + (t - run_start) / CAP * CAP;
+            const int left = run_start + run_len - gs;
+            seg_tab[t] = (uint32_t)gs | (uint32_t)(left < CAP ? left : CAP) << 16;
+        }
+        __syncthreads();
+    }
+
     auto tile_coords = [&](int64_t n, int64_t& q_tile, int64_t& p_tile) -> bool {
         constexpr int G = 16;
         const int64_t loc = slot + n * W, logical = xcd * per_xcd + loc;
         if (loc >= per_xcd || logical >= T) return false;
+        if (ordered) {
+            const uint32_t sg = (uint32_t)__builtin_amdgcn_readfirstlane((int)seg_tab[(int)(logical / p_tiles)]);
+            const int gs = (int)(sg & 0xFFFFu), gl = (int)(sg >> 16);
+            const int j = (int)(logical - (int64_t)gs * p_tiles);
+            p_tile = j / gl;
+            q_tile = gs + j % gl;
+            return true;
+        }
         const int64_t grp = logical / (G * p_tiles), rem = logical % (G * p_tiles);
         const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;
         q_tile = grp * G + rem % gq;
