@@ -1,4 +1,4 @@
-"""The Paddle binding printed in INTEGRATION.md, executed as written.
+"""The Paddle binding shipped as paddleformers_amd/paddle_backend.py, executed as written.
 
 Paddle is not installed, so the dozen `paddle.*` names the binding uses (dtypes, `empty`, the stream accessor, the
 `incubate.nn.functional` namespace, `Tensor.strides` / `Tensor.astype`) are provided here on top of torch tensors.  What this
@@ -8,7 +8,6 @@ byte for byte with the package's own binding of the same entry point.
 from __future__ import annotations
 
 import os
-import re
 import sys
 import types
 
@@ -49,8 +48,7 @@ def _fake_paddle():
 
 @pytest.fixture(scope="module")
 def stub():
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
-    code = re.search(r"```python\n(.*?)```", text, re.S).group(1)
+    code = open(os.path.join(ROOT, "paddleformers_amd", "paddle_backend.py")).read()
     assert "..." not in code, "the binding must be written out in full"
     assert 'ctypes.CDLL("libpf8.so")' in code
     code = code.replace('ctypes.CDLL("libpf8.so")', f"ctypes.CDLL({L.LIB_PATH!r})")   # the in-tree build, by path
@@ -62,7 +60,7 @@ def stub():
     sys.modules["paddle"] = _fake_paddle()
     ns = {"__name__": "pf8_backend"}
     try:
-        exec(compile(code, "INTEGRATION.md:pf8_backend", "exec"), ns)
+        exec(compile(code, "paddle_backend.py", "exec"), ns)
         ns["install"]()
         yield types.SimpleNamespace(**ns)
     finally:
