@@ -206,6 +206,57 @@ def test_grouped_contiguous_equals_per_expert_loop(dg, rows, lay):
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
 
 
+# The persistent kernel (K = 2048, whole 256-column tiles) orders its tiles by groups of row tiles that stop at expert
+# boundaries and hold at most twelve tiles; with more than 256 row tiles it falls back to fixed groups of sixteen.
+# Cases: runs longer than a group, padding tiles (m_indices = -1) between and inside experts' runs, a single expert,
+# and 300 row tiles.  Every 128-row tile must equal the dense GEMM of its rows with its expert's weight, bit for bit.
+@pytest.mark.parametrize("blocks", [
+    [(0, 13), (-1, 1), (1, 1), (2, 25), (-1, 2), (3, 2), (3, 1)],
+    [(2, 30)],
+    [(e % 5, 1 + (e * 7) % 4) for e in range(40)] + [(-1, 1)] + [(4, 199)],
+])
+@pytest.mark.parametrize("cus", [0, 16])
+def test_grouped_contiguous_tile_groups_of_the_persistent_kernel(dg, blocks, cus):
+    E, N, K = 5, 512, 2048
+    Mtot = 128 * sum(n for _, n in blocks)
+    rng = np.random.default_rng(Mtot + cus)
+    # one activation row block and its scales, repeated with a per-block sign and exponent change: cheap to build at
+    # 38,400 rows and still different from block to block
+    base = G.bf16_normal((128, K), seed=5, outlier_frac=0.01, outlier_scale=20.0)
+    a0, sa0 = _quant_act(base, 0)
+    nb = Mtot // 128
+    shift = rng.integers(0, 128, size=nb)
+    a = np.concatenate([np.roll(a0, int(sft), axis=0) for sft in shift])
+    sa = np.concatenate([np.roll(sa0, int(sft), axis=0) * np.float32(2.0 ** (int(sft) % 5 - 2)) for sft in shift])
+    bs, sbs = zip(*[_quant_w(G.bf16_normal((N, K), seed=70 + e, std=0.02, outlier_frac=5e-4, outlier_scale=50.0)) for e in range(E)])
+    b, sb = np.stack(bs), np.stack(sbs)
+    m_idx = np.concatenate([np.full(128 * n, e, dtype=np.int32) for e, n in blocks])
+    ta, tsa = G.to_torch_fp8(a), torch.from_numpy(np.ascontiguousarray(sa.T)).cuda().t()
+    tb, tsb = G.to_torch_fp8(b), torch.from_numpy(sb).cuda()
+    out = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dg.set_num_sms(cus)
+    try:
+        dg.m_grouped_fp8_gemm_nt_contiguous((ta, tsa), (tb, tsb), out, torch.from_numpy(m_idx).cuda())
+    finally:
+        dg.set_num_sms(0)
+    ref = torch.full_like(out, float("nan"))
+    start = 0
+    for e, n in blocks:
+        r = 128 * n
+        if e >= 0:
+            dg.fp8_gemm_nt((ta[start:start + r], tsa[start:start + r]), (tb[e], tsb[e]), ref[start:start + r])
+        start += r
+    skipped = torch.from_numpy(m_idx < 0).cuda()
+    assert torch.isnan(out[skipped].float()).all(), "rows of padding tiles must not be written"
+    assert torch.equal(out[~skipped].view(torch.int16), ref[~skipped].view(torch.int16))
+    # one slab straight against the oracle: the last tile of the longest run
+    e_big, n_big = max(blocks, key=lambda t: t[1] if t[0] >= 0 else -1)
+    first = 128 * sum(n for _, n in blocks[:blocks.index((e_big, n_big))])
+    lo = first + 128 * (n_big - 1)
+    exp = O.gemm_nt(a[lo:lo + 128], sa[lo:lo + 128], b[e_big], sb[e_big])
+    assert G.rel_fro(_bf(G.from_torch_bf16(out[lo:lo + 128])), _bf(exp)) <= BLOCK_FRO
+
+
 @pytest.fixture
 def few_cus(dg):
     """A budget of eight compute units (deep_gemm.set_num_sms): the persistent kernel runs one workgroup per
