@@ -383,45 +383,53 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     const int64_t q_rows_total = a.Qrows;
     const bool grouped = a.group == GROUP_CONTIG;
 
-    // Grouped layout with at most 256 row tiles: the row tiles are cut into groups that never span two experts
-    // (at most 12 tiles each), and the tiles of a group are walked q fastest, p slowest.  The 32 workgroups of an
-    // XCD then work on one or two weight strips of ONE expert at a time and on the few activation strips of that
-    // group, instead of on 16 activation strips that belong to a dozen experts.  Measured on config 3 (32 experts,
-    // Zipf load) against groups of 16 row tiles cut without regard to experts: the L2s miss 1.33 GB instead of
-    // 1.74 GB per up+gate launch (hit rate 64% against 53%) and 0.74 GB instead of 0.96 GB on the down GEMM; the
-    // launches get 3% and 2% shorter.  seg_tab[q] = first tile of q's group | tiles in it << 16.
-    __shared__ uint32_t seg_tab[256];
-    __shared__ int seg_wave_max[4];
-    const bool ordered = grouped && q_tiles <= 256;
+    // Grouped layout with at most 2048 row tiles: every expert's run of row tiles is cut into groups of at most 12
+    // tiles (no group spans two experts), and the tiles of a group are walked q fastest, p slowest.  The 32 workgroups
+    // of an XCD then work on one or two weight strips of ONE expert at a time and on the few activation strips of
+    // that group, instead of on 16 activation strips that belong to a dozen experts.  Measured on config 3 (32
+    // experts, Zipf load) against groups of 16 row tiles cut without regard to experts: the L2s miss 1.33 GB instead
+    // of 1.74 GB per up+gate launch (hit rate 64% against 53%) and 0.74 GB instead of 0.96 GB on the down GEMM; the
+    // launches get 3% and 2% shorter.  seg_tab[q] = first tile of q's group | tiles in it << 16; every workgroup
+    // builds the table for itself: the first tile of each run by a prefix maximum over the tiles, 256 at a time.
+    __shared__ uint32_t seg_tab[2048];
+    __shared__ int16_t seg_eid[2048 + 2];                  // expert of every row tile (one global load each), -1 = padding
+    __shared__ int seg_wave_max[2][4];
+    const bool ordered = grouped && q_tiles <= 2048 && a.E <= 32767;
     if (ordered) {
         constexpr int CAP = 12;
-        const int t = tid, qt = (int)q_tiles;
-        // expert of tile t and of its neighbours; every padding tile counts as expert -1, tiles past the end as -2
-        auto expert_of = [&](int i) -> int {
-            if (i < 0) return -3;
-            if (i >= qt) return -2;
-            const int e = a.m_indices[(int64_t)i * BQ];
-            return e < 0 ? -1 : e;
-        };
-        const int e_me = expert_of(t), e_prev = expert_of(t - 1), e_next = expert_of(t + 1);
-        int v = (t < qt && e_me != e_prev) ? t : 0;            // first tile of a run of one expert
-#pragma unroll
-        for (int dlt = 1; dlt < 64; dlt <<= 1) {
-            const int o = __shfl_up(v, dlt, 64);
-            if (lane >= dlt && o > v) v = o;
+        const int qt = (int)q_tiles;
+        for (int t = tid; t < qt; t += 256) {
+            const int e = a.m_indices[(int64_t)t * BQ];
+            seg_eid[t + 1] = (int16_t)(e < 0 ? -1 : e);
         }
-        if (lane == 63) seg_wave_max[wave] = v;
+        if (tid == 0) { seg_eid[0] = -2; seg_eid[qt + 1] = -2; }
         __syncthreads();
-        for (int w = 0; w < wave; ++w) v = seg_wave_max[w] > v ? seg_wave_max[w] : v;
-        const int run_start = v;
-        if (t < qt && e_me != e_next) seg_tab[run_start] = (uint32_t)(t - run_start + 1);
-        __syncthreads();
-        const int run_len = t < qt ? (int)seg_tab[run_start] : 0;
-        __syncthreads();
-        if (t < qt) {
-            const int gs = run_start + (t - run_start) / CAP * CAP;
-            const int left = run_start + run_len - gs;
-            seg_tab[t] = (uint32_t)gs | (uint32_t)(left < CAP ? left : CAP) << 16;
+        int carry = 0;                                     // first tile of the run the previous chunk ended in
+        for (int c0 = 0, par = 0; c0 < qt; c0 += 256, par ^= 1) {
+            const int t = c0 + tid;
+            const int e = t < qt ? seg_eid[t + 1] : -2;
+            int v = (t < qt && t > 0 && seg_eid[t] != e) ? t : 0;
+#pragma unroll
+            for (int dlt = 1; dlt < 64; dlt <<= 1) {
+                const int o = __shfl_up(v, dlt, 64);
+                if (lane >= dlt && o > v) v = o;
+            }
+            if (lane == 63) seg_wave_max[par][wave] = v;
+            __syncthreads();                               // the buffers alternate: one barrier per chunk
+            int all = carry;
+            for (int w = 0; w < 4; ++w) {
+                const int m = seg_wave_max[par][w];
+                if (w < wave && m > v) v = m;
+                if (m > all) all = m;
+            }
+            if (carry > v) v = carry;
+            carry = all;
+            if (t < qt) {
+                const int gs = v + (t - v) / CAP * CAP;    // v = first tile of this tile's run
+                int hi = t + 1;
+                while (hi < gs + CAP && seg_eid[hi + 1] == e) ++hi;     // stops at the end marker behind the last tile
+                seg_tab[t] = (uint32_t)gs | (uint32_t)(hi - gs) << 16;
+            }
         }
         __syncthreads();
     }
@@ -954,15 +962,14 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         const int64_t T128 = ((a.Prows + 255) / 256) * ((a.Qrows + 127) / 128);
         // the grid is padded to a multiple of 8 so that every XCD gets an equal run of tiles
         dim3 g128((unsigned)(((T128 + 7) / 8) * 8), grid.y);
-        // The persistent deep-pipeline kernel wins where the operand stream, not the matrix pipe, sets
-        // the pace.  Measured on MI355X against the two-workgroup kernel: +14..24% when all tiles
-        // fit one round of compute units (dense M <= 2048 at N = 4096), +15% / +7% on the up+gate /
-        // down GEMMs of 32 experts with a skewed 8192-row load, +10% on the dense 8192 x 4096 x 7168
-        // product (four rounds); beyond ten rounds of tiles its static tile assignment loses what the
-        // deeper pipeline gains.
+        // The persistent deep-pipeline kernel takes every shape it can tile (whole 256-column and 128-row tiles, at
+        // least three K blocks, dense or contiguous-grouped).  Measured on MI355X against the two-workgroup kernel:
+        // +14..24% when all tiles fit one round of compute units, +15% / +7% on the up+gate / down GEMMs of 32
+        // experts with a skewed 8192-row load, +7% / +17% on those of 128 experts with 131072 rows (47 and 68 rounds
+        // of tiles), +20..35% on dense products with 3 to 8 K blocks and 32 rounds, equal on 32768 x 8192 x 8192.
         const bool aligned = a.Prows % 256 == 0 && a.Qrows % 128 == 0 && a.red >= 384 && a.group != GROUP_MASKED;
         const int64_t cus = pf8_effective_cus();
-        const bool deep = aligned && (T128 <= cus || (a.red >= 2048 && T128 <= 10 * cus));
+        const bool deep = aligned;
         if (deep) {
             // persistent: one workgroup per compute unit (or per tile of an XCD's run, if fewer)
             const int64_t per_xcd = (T128 + 7) / 8;
