@@ -368,10 +368,13 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     const int wq = wave >> 1, wp = wave & 1;
     const int li = lane & 15, kg = lane >> 4;
 
-    const int64_t p_tiles = a.Prows / 256, q_tiles = a.Qrows / BQ;
+    // Prows may be 256 t + 128: the last column tile then covers the last 256 weight rows, i.e. it repeats the 128
+    // columns before it (those wavefronts store nothing) beside the 128 new ones.  Not with FUSE.
+    const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = a.Qrows / BQ;
+    const int64_t p_last0 = a.Prows - 256;                                   // first weight row of that tile
+    auto p_row0 = [&](int64_t pt) -> int64_t { return FUSE ? pt * 128 : (pt * 256 < p_last0 ? pt * 256 : p_last0); };
     const int64_t T = p_tiles * q_tiles;
     // FUSE: tile p takes weight rows [128 p, 128 p + 128) (gate) and inter + the same (up)
-    const int64_t p_rows_per_tile = FUSE ? 128 : 256;
     const int64_t up_off = FUSE ? a.inter * a.red : 128 * a.red;      // bytes from a tile's first half to its second
     const int64_t IB = FUSE ? a.inter / 128 : 0;
     // consecutive workgroups go round-robin to the 8 XCDs: every XCD owns a contiguous run of
@@ -460,9 +463,9 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     if (grouped) ce = __builtin_amdgcn_readfirstlane(a.m_indices[cq * BQ]);
     int c_rows = ce < 0 ? 0 : BQ;          // rows of the tile that are stored (none for a padding tile)
     if (ce < 0) ce = 0;
-    const uint8_t* c_ptile = a.p + ((int64_t)ce * a.Prows + cp * p_rows_per_tile) * a.red;
+    const uint8_t* c_ptile = a.p + ((int64_t)ce * a.Prows + p_row0(cp)) * a.red;
     const uint8_t* c_qtile = a.q + cq * BQ * a.red;
-    const ST* c_spb = sp_base + ((int64_t)ce * PB + (FUSE ? cp + wp * IB : cp * 2 + wp)) * KB;
+    const ST* c_spb = sp_base + ((int64_t)ce * PB + (FUSE ? cp + wp * IB : p_row0(cp) / 128 + wp)) * KB;
     const ST* c_sq0 = SQL == 0 ? sq_base + (cq * BQ + wq * 64) * KB : sq_base + cq * BQ + wq * 64;
     const uint8_t* n_ptile = c_ptile;
     const uint8_t* n_qtile = c_qtile;
@@ -541,9 +544,9 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                 if (n_valid) {
                     n_rows = ne < 0 ? 0 : BQ;
                     const int e = ne < 0 ? 0 : ne;
-                    n_ptile = a.p + ((int64_t)e * a.Prows + np * p_rows_per_tile) * a.red;
+                    n_ptile = a.p + ((int64_t)e * a.Prows + p_row0(np)) * a.red;
                     n_qtile = a.q + nq * BQ * a.red;
-                    n_spb = sp_base + ((int64_t)e * PB + (FUSE ? np + wp * IB : np * 2 + wp)) * KB;
+                    n_spb = sp_base + ((int64_t)e * PB + (FUSE ? np + wp * IB : p_row0(np) / 128 + wp)) * KB;
                     n_sq0 = SQL == 0 ? sq_base + (nq * BQ + wq * 64) * KB : sq_base + nq * BQ + wq * 64;
                 } else {
                     // past the last tile the copies and scale loads re-read this tile's first blocks:
@@ -690,7 +693,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
             uint8_t* ep = lds + last * STAGE + wave * (32 * EP_LD);
             uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
             const int er = lane >> 4, ec = lane & 15;
-            const int64_t col = cp * 256 + wp * 128 + ec * 8;
+            const int64_t col = p_row0(cp) + wp * 128 + ec * 8;
+            const bool store = c_rows && !(cp * 256 > p_last0 && wp == 0);      // the repeated half of a last half tile
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -709,7 +713,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                     const int rl = er + 4 * i;                        // row inside the 32-row slice
                     const int64_t row = cq * BQ + wq * 64 + half * 32 + rl;
                     const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
-                    if (c_rows) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
+                    if (store) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
                 }
             }
         }
@@ -962,12 +966,13 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         const int64_t T128 = ((a.Prows + 255) / 256) * ((a.Qrows + 127) / 128);
         // the grid is padded to a multiple of 8 so that every XCD gets an equal run of tiles
         dim3 g128((unsigned)(((T128 + 7) / 8) * 8), grid.y);
-        // The persistent deep-pipeline kernel takes every shape it can tile (whole 256-column and 128-row tiles, at
+        // The persistent deep-pipeline kernel takes every shape it can tile (128-row tiles, 256-column tiles of which the
+        // last may be half new, at
         // least three K blocks, dense or contiguous-grouped).  Measured on MI355X against the two-workgroup kernel:
         // +14..24% when all tiles fit one round of compute units, +15% / +7% on the up+gate / down GEMMs of 32
         // experts with a skewed 8192-row load, +7% / +17% on those of 128 experts with 131072 rows (47 and 68 rounds
         // of tiles), +20..35% on dense products with 3 to 8 K blocks and 32 rounds, equal on 32768 x 8192 x 8192.
-        const bool aligned = a.Prows % 256 == 0 && a.Qrows % 128 == 0 && a.red >= 384 && a.group != GROUP_MASKED;
+        const bool aligned = a.Prows % 128 == 0 && a.Prows >= 256 && a.Qrows % 128 == 0 && a.red >= 384 && a.group != GROUP_MASKED;
         const int64_t cus = pf8_effective_cus();
         const bool deep = aligned;
         if (deep) {

@@ -76,7 +76,7 @@ def _check(got_bits, a, sa, b, sb, what, lay=0):
     _elementwise_ok(_bf(got_bits), a, sa, b, sb, lay, what)
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 512, 1024), (200, 384, 256), (1, 128, 384), (130, 640, 128)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 512, 1024), (200, 384, 256), (1, 128, 384), (130, 640, 128), (256, 384, 512), (384, 640, 1024), (128, 1408, 384)])
 @pytest.mark.parametrize("lay", [0, 1])
 def test_fp8_gemm_nt_vs_oracle(dg, M, N, K, lay):
     xa = G.bf16_normal((M, K), seed=M + K)
