@@ -370,21 +370,20 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
 
     // Prows may be 256 t + 128: the last column tile then covers the last 256 weight rows, i.e. it repeats the 128
     // columns before it (those wavefronts store nothing) beside the 128 new ones.  Not with FUSE.
-    const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = a.Qrows / BQ;
+    const int64_t p_tiles = (a.Prows + 255) / 256;
+    int64_t q_tiles = a.Qrows / BQ;          // masked layout: row tiles per expert here, valid row tiles of all experts below
     const int64_t p_last0 = a.Prows - 256;                                   // first weight row of that tile
     auto p_row0 = [&](int64_t pt) -> int64_t { return FUSE ? pt * 128 : (pt * 256 < p_last0 ? pt * 256 : p_last0); };
-    const int64_t T = p_tiles * q_tiles;
     // FUSE: tile p takes weight rows [128 p, 128 p + 128) (gate) and inter + the same (up)
     const int64_t up_off = FUSE ? a.inter * a.red : 128 * a.red;      // bytes from a tile's first half to its second
     const int64_t IB = FUSE ? a.inter / 128 : 0;
     // consecutive workgroups go round-robin to the 8 XCDs: every XCD owns a contiguous run of
     // logical tiles (groups of q-tiles x all p-tiles, see below), walked W tiles at a time by its W workgroups
-    const int64_t per_xcd = (T + 7) / 8;
     const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, W = gridDim.x >> 3;
     const int64_t KB = a.red / 128;
     const int64_t PB = a.Prows / 128;
     const int64_t q_rows_total = a.Qrows;
-    const bool grouped = a.group == GROUP_CONTIG;
+    const bool grouped = a.group == GROUP_CONTIG, masked = a.group == GROUP_MASKED;
 
     // Grouped layout with at most 2048 row tiles: every expert's run of row tiles is cut into groups of at most 12
     // tiles (no group spans two experts), and the tiles of a group are walked q fastest, p slowest.  The 32 workgroups
@@ -437,6 +436,40 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         __syncthreads();
     }
 
+    // Masked layout (a [E, Mmax, K], masked_m[e] valid rows; at most 256 experts and 2048 row tiles): only the row tiles
+    // that hold valid rows are walked.  Every workgroup lists them for itself: seg_tab[slot] = expert | tile << 16,
+    // seg_valid[e] = valid rows; a row tile of expert e is row tile e * (Mmax / 128) + tile of the [E * Mmax, K] matrix.
+    __shared__ int seg_valid[256];
+    __shared__ int seg_total;
+    const int mt = (int)(a.Qrows / BQ);                    // row tiles per expert (masked)
+    if (masked) {
+        int valid = 0, cnt = 0;
+        if (tid < a.E) {
+            valid = a.masked_m[tid];
+            valid = valid < 0 ? 0 : (valid > (int)a.Qrows ? (int)a.Qrows : valid);
+            cnt = (valid + BQ - 1) / BQ;
+            seg_valid[tid] = valid;
+        }
+        int incl = cnt;                                    // inclusive prefix sum over the 256 threads
+#pragma unroll
+        for (int dlt = 1; dlt < 64; dlt <<= 1) {
+            const int o = __shfl_up(incl, dlt, 64);
+            if (lane >= dlt) incl += o;
+        }
+        if (lane == 63) seg_wave_max[0][wave] = incl;
+        __syncthreads();
+        int before = 0;
+        for (int w = 0; w < wave; ++w) before += seg_wave_max[0][w];
+        if (tid == 0) seg_total = seg_wave_max[0][0] + seg_wave_max[0][1] + seg_wave_max[0][2] + seg_wave_max[0][3];
+        const int first = before + incl - cnt;
+        for (int i = 0; i < cnt; ++i) seg_tab[first + i] = (uint32_t)tid | (uint32_t)i << 16;
+        __syncthreads();
+        q_tiles = seg_total;
+    }
+    const int64_t T = p_tiles * q_tiles;
+    const int64_t per_xcd = (T + 7) / 8;
+    int t_e = 0, t_rows = BQ;                              // masked: expert and valid rows of the tile tile_coords returned last
+
     auto tile_coords = [&](int64_t n, int64_t& q_tile, int64_t& p_tile) -> bool {
         constexpr int G = 16;
         const int64_t loc = slot + n * W, logical = xcd * per_xcd + loc;
@@ -453,6 +486,14 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         const int64_t gq = q_tiles - grp * G < G ? q_tiles - grp * G : G;
         q_tile = grp * G + rem % gq;
         p_tile = rem / gq;
+        if (masked) {
+            const uint32_t sg = (uint32_t)__builtin_amdgcn_readfirstlane((int)seg_tab[(int)q_tile]);
+            t_e = (int)(sg & 0xFFFFu);
+            const int lt = (int)(sg >> 16);
+            const int left = __builtin_amdgcn_readfirstlane(seg_valid[t_e]) - lt * BQ;
+            t_rows = left < BQ ? left : BQ;
+            q_tile = (int64_t)t_e * mt + lt;
+        }
         return true;
     };
 
@@ -461,7 +502,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     if (!tile_coords(0, cq, cp)) return;
     int ce = 0;
     if (grouped) ce = __builtin_amdgcn_readfirstlane(a.m_indices[cq * BQ]);
-    int c_rows = ce < 0 ? 0 : BQ;          // rows of the tile that are stored (none for a padding tile)
+    if (masked) ce = t_e;
+    int c_rows = ce < 0 ? 0 : (masked ? t_rows : BQ);   // rows of the tile that are stored (none for a padding tile)
     if (ce < 0) ce = 0;
     const uint8_t* c_ptile = a.p + ((int64_t)ce * a.Prows + p_row0(cp)) * a.red;
     const uint8_t* c_qtile = a.q + cq * BQ * a.red;
@@ -534,6 +576,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         const bool n_valid = tile_coords(n + 1, nq, np);
         int ne = 0;
         if (n_valid && grouped) asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ne) : "s"(a.m_indices + nq * BQ) : "memory");
+        const int ne_rows = t_rows;
+        if (masked) ne = t_e;
 #pragma unroll
         for (int i = 0; i < NPS; ++i)
 #pragma unroll
@@ -542,7 +586,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
         for (int64_t kb = 0; kb < KB; ++kb) {
             if (kb == 1) {
                 if (n_valid) {
-                    n_rows = ne < 0 ? 0 : BQ;
+                    n_rows = ne < 0 ? 0 : (masked ? ne_rows : BQ);
                     const int e = ne < 0 ? 0 : ne;
                     n_ptile = a.p + ((int64_t)e * a.Prows + p_row0(np)) * a.red;
                     n_qtile = a.q + nq * BQ * a.red;
@@ -694,7 +738,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
             uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
             const int er = lane >> 4, ec = lane & 15;
             const int64_t col = p_row0(cp) + wp * 128 + ec * 8;
-            const bool store = c_rows && !(cp * 256 > p_last0 && wp == 0);      // the repeated half of a last half tile
+            const bool store = !(cp * 256 > p_last0 && wp == 0);               // not the repeated half of a last half tile
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -713,7 +757,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                     const int rl = er + 4 * i;                        // row inside the 32-row slice
                     const int64_t row = cq * BQ + wq * 64 + half * 32 + rl;
                     const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
-                    if (store) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
+                    if (store && wq * 64 + half * 32 + rl < c_rows) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
                 }
             }
         }
@@ -972,12 +1016,14 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         // +14..24% when all tiles fit one round of compute units, +15% / +7% on the up+gate / down GEMMs of 32
         // experts with a skewed 8192-row load, +7% / +17% on those of 128 experts with 131072 rows (47 and 68 rounds
         // of tiles), +20..35% on dense products with 3 to 8 K blocks and 32 rounds, equal on 32768 x 8192 x 8192.
-        const bool aligned = a.Prows % 128 == 0 && a.Prows >= 256 && a.Qrows % 128 == 0 && a.red >= 384 && a.group != GROUP_MASKED;
+        const bool aligned = a.Prows % 128 == 0 && a.Prows >= 256 && a.Qrows % 128 == 0 && a.red >= 384 &&
+                             (a.group != GROUP_MASKED || (a.E <= 256 && (int64_t)a.E * (a.Qrows / 128) <= 2048));
         const int64_t cus = pf8_effective_cus();
         const bool deep = aligned;
         if (deep) {
-            // persistent: one workgroup per compute unit (or per tile of an XCD's run, if fewer)
-            const int64_t per_xcd = (T128 + 7) / 8;
+            // persistent: one workgroup per compute unit (or per tile of an XCD's run, if fewer); the masked layout is
+            // one launch over all experts (the kernel walks the row tiles that hold valid rows)
+            const int64_t per_xcd = (T128 * (a.group == GROUP_MASKED ? a.E : 1) + 7) / 8;
             int64_t w = cus / 8;
             if (w < 1) w = 1;
             if (w > per_xcd) w = per_xcd;
