@@ -210,14 +210,15 @@ def test_grouped_contiguous_equals_per_expert_loop(dg, rows, lay):
 # boundaries and hold at most twelve tiles; with more than 256 row tiles it falls back to fixed groups of sixteen.
 # Cases: runs longer than a group, padding tiles (m_indices = -1) between and inside experts' runs, a single expert,
 # and 300 row tiles.  Every 128-row tile must equal the dense GEMM of its rows with its expert's weight, bit for bit.
-@pytest.mark.parametrize("blocks", [
-    [(0, 13), (-1, 1), (1, 1), (2, 25), (-1, 2), (3, 2), (3, 1)],
-    [(2, 30)],
-    [(e % 5, 1 + (e * 7) % 4) for e in range(40)] + [(-1, 1)] + [(4, 199)],
+@pytest.mark.parametrize("K,blocks", [
+    (2048, [(0, 13), (-1, 1), (1, 1), (2, 25), (-1, 2), (3, 2), (3, 1)]),
+    (2048, [(2, 30)]),
+    (2048, [(e % 5, 1 + (e * 7) % 4) for e in range(40)] + [(-1, 1)] + [(4, 199)]),
+    (384, [(0, 1500), (-1, 1), (1, 3), (3, 600)]),          # more than 2048 row tiles: fixed groups of sixteen
 ])
 @pytest.mark.parametrize("cus", [0, 16])
-def test_grouped_contiguous_tile_groups_of_the_persistent_kernel(dg, blocks, cus):
-    E, N, K = 5, 512, 2048
+def test_grouped_contiguous_tile_groups_of_the_persistent_kernel(dg, K, blocks, cus):
+    E, N = 5, 512
     Mtot = 128 * sum(n for _, n in blocks)
     rng = np.random.default_rng(Mtot + cus)
     # one activation row block and its scales, repeated with a per-block sign and exponent change: cheap to build at
@@ -355,6 +356,35 @@ def test_grouped_masked(dg):
         assert np.array_equal(got[e, m:], init[e, m:]), f"expert {e}: rows beyond masked_m were written"
         if m:
             assert G.rel_fro(_bf(got[e, :m]), _bf(exp[e, :m])) <= BLOCK_FRO
+
+
+@pytest.mark.parametrize("E,Mmax", [(260, 128), (3, 200), (40, 384)])
+def test_grouped_masked_layouts_of_both_kernels(dg, E, Mmax):
+    """More than 256 experts and a capacity that is not a multiple of 128 take the two-workgroup kernel, 40 experts of
+    three row tiles the persistent one; every expert's valid rows must equal the dense GEMM of those rows, bit for bit."""
+    N, K = 256, 512
+    rng = np.random.default_rng(E + Mmax)
+    masked = rng.integers(0, Mmax + 1, size=E).astype(np.int32)
+    masked[0], masked[-1] = Mmax, 0
+    a0, sa0 = _quant_act(G.bf16_normal((Mmax, K), seed=7, outlier_frac=0.01, outlier_scale=20.0), 0)
+    b0, sb0 = _quant_w(G.bf16_normal((N, K), seed=8, std=0.02))
+    a = np.stack([np.roll(a0, e, axis=0) for e in range(E)])
+    sa = np.stack([np.roll(sa0, e, axis=0) for e in range(E)])
+    b = np.stack([np.roll(b0, 128 * (e % 2), axis=0) for e in range(E)])
+    sb = np.stack([np.roll(sb0, e % 2, axis=0) for e in range(E)])
+    ta, tsa, tb, tsb = G.to_torch_fp8(a), torch.from_numpy(sa).cuda(), G.to_torch_fp8(b), torch.from_numpy(sb).cuda()
+    out = torch.full((E, Mmax, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dg.m_grouped_fp8_gemm_nt_masked((ta, tsa), (tb, tsb), out, torch.from_numpy(masked).cuda(), int(masked.mean()))
+    ref = torch.empty((Mmax, N), dtype=torch.bfloat16, device="cuda")
+    for e in list(range(0, E, max(1, E // 12))) + [E - 1]:
+        m = int(masked[e])
+        assert torch.isnan(out[e, m:].float()).all(), f"expert {e}: rows beyond masked_m were written"
+        if m:
+            dg.fp8_gemm_nt((ta[e], tsa[e]), (tb[e], tsb[e]), ref)
+            assert torch.equal(out[e, :m].view(torch.int16), ref[:m].view(torch.int16)), f"expert {e}"
+    e = 0
+    exp = O.gemm_nt(a[e], sa[e], b[e], sb[e])
+    assert G.rel_fro(_bf(G.from_torch_bf16(out[e])), _bf(exp)) <= BLOCK_FRO
 
 
 # ---------------------------------------------------------------------------------------------
