@@ -32,6 +32,8 @@ FLAGS = [
     # packed fp32 arithmetic stays off on this target
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall",
+    # per-kernel register, LDS and scratch usage as compiler remarks: build() refuses a kernel that spills to scratch
+    "-Rpass-analysis=kernel-resource-usage",
 ]
 
 
@@ -50,14 +52,44 @@ def up_to_date() -> bool:
     return all(os.path.getmtime(d) <= t for d in deps)
 
 
+def kernels_with_scratch(remarks):
+    """(kernel, bytes per lane) for every kernel whose resource-usage remark reports scratch memory.  The hand-scheduled
+    kernels are written to fit the register file: a spill there is a performance bug, and scratch makes every launch
+    depend on a per-queue scratch allocation."""
+    found, name = [], None
+    for l in remarks:
+        if "Function Name:" in l:
+            name = l.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in l:
+            n = int(l.split("ScratchSize [bytes/lane]:")[1].split("[")[0].strip())
+            if n > 0 and name:
+                found.append((name, n))
+    return found
+
+
 def build(force: bool = False, verbose: bool = False) -> str:
     if not force and up_to_date():
         return LIB
     cmd = [hipcc()] + FLAGS + [os.path.join(CSRC, f) for f in SOURCES] + ["-o", LIB]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    lines = proc.stdout.splitlines()
+    # drop the feature warning of the host pass and the resource-usage remarks with the source lines they quote
+    kept, skip = [], 0
+    for l in lines:
+        if "kernel-resource-usage" in l:
+            skip = 2
+        elif skip and (l.lstrip().startswith("|") or l.lstrip().split(" |")[0].isdigit()):
+            skip -= 1
+        elif "packed-fp32-ops" not in l:
+            kept.append(l)
+            skip = 0
+    out = "\n".join(kept)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + out)
+    spilling = kernels_with_scratch(lines)
+    if spilling:
+        os.remove(LIB)
+        raise RuntimeError("kernels that spill registers to scratch memory (bytes per lane): " + ", ".join(f"{k}: {v}" for k, v in spilling))
     if verbose and out.strip():
         print(out)
     return LIB

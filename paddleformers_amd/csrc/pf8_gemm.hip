@@ -116,10 +116,6 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
     constexpr int BQ = 128, NPS = 8;
     constexpr int P_STAGE = 32768, Q_OFS = 65536;   // [P stage 0 | P stage 1 | Q]
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wq = wave >> 1, wp = wave & 1;
-    const int li = lane & 15, kg = lane >> 4;
-
     const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = (a.Qrows + BQ - 1) / BQ;
     const int64_t T = p_tiles * q_tiles;
     // consecutive workgroups go round-robin to the 8 XCDs: give every XCD a contiguous run of logical
@@ -127,6 +123,14 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
     // tile; under a compute-unit budget it is smaller and a workgroup walks its XCD's run in strides.
     const int64_t per_xcd = (T + 7) / 8;
     for (int64_t loc = blockIdx.x >> 3; loc < per_xcd; loc += gridDim.x >> 3) {
+    // the lane's coordinates are formed anew for every tile from a value the compiler cannot see through: hoisted
+    // out of the loop, everything a tile's set-up derives from them would stay live across the whole tile (39
+    // registers more than the file holds)
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wq = wave >> 1, wp = wave & 1;
+    const int li = lane & 15, kg = lane >> 4;
     const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + loc;
     if (logical >= T) break;
     constexpr int G = 16;
@@ -135,7 +139,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
     const int64_t q_tile = grp * G + rem % gq, p_tile = rem / gq;
     const int64_t p0 = p_tile * 256, q0 = q_tile * BQ;
 
-    const int64_t KB = a.red / 128;
+    int64_t KB = a.red / 128;
+    asm volatile("" : "+s"(KB));          // per tile as well: a flag derived from it was kept in a register across the loop
     const int64_t PB = (a.Prows + 127) / 128;
     const uint8_t* qbase = a.q;
     const float* sqb = a.sq;
@@ -354,7 +359,7 @@ __device__ __forceinline__ float e8m0_to_f32(uint32_t b) { return u2f(b ? b << 2
 // outputs is the 16 lanes of a DPP row, exactly the tile of the standalone SwiGLU quantizer, whose arithmetic is
 // restated operation for operation (bf16(silu(g) * u), bf16(. * p), amax, scale, quotient), so bytes and scales are
 // bit-identical to the un-fused pair of launches.
-template <int SQL, int SF = 0, int FUSE = 0>
+template <int SQL, int SF = 0, int FUSE = 0, int MASKED = 0>
 __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     using ST = typename std::conditional<SF == 1, uint8_t, float>::type;
     if (SF == 1 && a.pair_list && e8_paired_tiles_win(a.pair_list, a.Prows / 256, a.cus)) return;
@@ -383,7 +388,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     const int64_t KB = a.red / 128;
     const int64_t PB = a.Prows / 128;
     const int64_t q_rows_total = a.Qrows;
-    const bool grouped = a.group == GROUP_CONTIG, masked = a.group == GROUP_MASKED;
+    const bool grouped = a.group == GROUP_CONTIG;
+    constexpr bool masked = MASKED != 0;       // its own instantiation: the extra state costs the others registers
 
     // Grouped layout with at most 2048 row tiles: every expert's run of row tiles is cut into groups of at most 12
     // tiles (no group spans two experts), and the tiles of a group are walked q fastest, p slowest.  The 32 workgroups
@@ -738,7 +744,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
             uint8_t* outb = reinterpret_cast<uint8_t*>(a.out);
             const int er = lane >> 4, ec = lane & 15;
             const int64_t col = p_row0(cp) + wp * 128 + ec * 8;
-            const bool store = !(cp * 256 > p_last0 && wp == 0);               // not the repeated half of a last half tile
+            const bool store = c_rows && !(cp * 256 > p_last0 && wp == 0);     // not a padding tile, not the repeated half of a last half tile
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -757,7 +763,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                     const int rl = er + 4 * i;                        // row inside the 32-row slice
                     const int64_t row = cq * BQ + wq * 64 + half * 32 + rl;
                     const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
-                    if (store && wq * 64 + half * 32 + rl < c_rows) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
+                    if (store && (!masked || rl < c_rows - wq * 64 - half * 32)) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
                 }
             }
         }
@@ -1028,7 +1034,8 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
             if (w < 1) w = 1;
             if (w > per_xcd) w = per_xcd;
             dim3 gd((unsigned)(8 * w), 1);
-            if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0>), gd, dim3(256), 147456, st, a);
+            if (a.group == GROUP_MASKED) hipLaunchKernelGGL((k_gemm_fwd_deep<0, 0, 0, 1>), gd, dim3(256), 147456, st, a);
+            else if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0>), gd, dim3(256), 147456, st, a);
             else hipLaunchKernelGGL((k_gemm_fwd_deep<1>), gd, dim3(256), 147456, st, a);
         } else {
             // under a compute-unit budget: two workgroups per budgeted unit, each walking several tiles
@@ -1072,6 +1079,7 @@ static int ensure_lds_attr() {
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0, 0, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
