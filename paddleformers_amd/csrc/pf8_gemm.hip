@@ -1017,11 +1017,10 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         // the grid is padded to a multiple of 8 so that every XCD gets an equal run of tiles
         dim3 g128((unsigned)(((T128 + 7) / 8) * 8), grid.y);
         // The persistent deep-pipeline kernel takes every shape it can tile (128-row tiles, 256-column tiles of which the
-        // last may be half new, at
-        // least three K blocks, dense or contiguous-grouped).  Measured on MI355X against the two-workgroup kernel:
-        // +14..24% when all tiles fit one round of compute units, +15% / +7% on the up+gate / down GEMMs of 32
-        // experts with a skewed 8192-row load, +7% / +17% on those of 128 experts with 131072 rows (47 and 68 rounds
-        // of tiles), +20..35% on dense products with 3 to 8 K blocks and 32 rounds, equal on 32768 x 8192 x 8192.
+        // last may be half new, at least three K blocks; dense, contiguous-grouped or masked).  Measured on MI355X
+        // against the two-workgroup kernel: +14..24% when all tiles fit one round of compute units, +21% / +8% on the
+        // up+gate / down GEMMs of 32 experts with a skewed 8192-row load, +2% on those of 128 experts with 131072 rows,
+        // within 3% either way on dense products from 3 to 64 K blocks and up to 32 rounds of tiles.
         const bool aligned = a.Prows % 128 == 0 && a.Prows >= 256 && a.Qrows % 128 == 0 && a.red >= 384 &&
                              (a.group != GROUP_MASKED || (a.E <= 256 && (int64_t)a.E * (a.Qrows / 128) <= 2048));
         const int64_t cus = pf8_effective_cus();
