@@ -652,7 +652,22 @@ class FP8GroupGemmMlpFunctionNode:
                 self._group_items = deep_gemm.build_group_items(m_indices)
             items = self._group_items
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, F8.scales_to_ue8m0(a_scale, check=False)),
-                                                   (w_fp8, F8.scales_to_ue8m0(w_scale, check=False)), out, m_indices, items=items)
+                                                   (w_fp8, self._weight_scale_bytes(w_scale)), out, m_indices, items=items)
+
+    def _weight_scale_bytes(self, w_scale):
+        """UE8M0 bytes of a weight scale tensor, converted once per tensor contents: the four weight operands of the
+        node keep their scales from call to call when the per-step weight cache holds them (fp8_quant_weight), so the
+        conversion is remembered under the tensor's storage, view and version counter (an in-place requantization
+        bumps the version; a new cache is a new storage; the source tensor is kept alive with its entry)."""
+        key = (w_scale.untyped_storage().data_ptr(), w_scale.storage_offset(), tuple(w_scale.shape), tuple(w_scale.stride()),
+               w_scale._version)
+        memo = self.__dict__.setdefault("_ue8m0_memo", {})
+        hit = memo.get(key)
+        if hit is None:
+            if len(memo) >= 8:                 # four operands, two generations
+                memo.clear()
+            hit = memo[key] = (w_scale, F8.scales_to_ue8m0(w_scale, check=False))
+        return hit[1]
 
     def _stacked(self, expert_w, transpose, num_expert):
         q, s = fused_stack_quant(expert_w, transpose=transpose, using_pow2_scale=self.use_ue8m0)

@@ -288,6 +288,59 @@ def test_moe_node_ue8m0_needs_a_pow2_weight_cache():
     assert torch.equal(plain.view(torch.int16), cached.view(torch.int16))
 
 
+def test_moe_node_ue8m0_weight_scale_bytes_follow_the_weight_cache():
+    """The node remembers the UE8M0 bytes of the cached weight scales between calls; a new cache (new tensors) and a
+    cache rewritten in place (same tensors, new contents) must both be picked up."""
+    from paddleformers_amd import fp8_utils as U
+    from paddleformers_amd import functional as F8
+
+    E, H, I = 2, 512, 384
+    rows = [256, 384]
+    _, _, experts, x, probs = _make(E, H, I, rows, seed=37)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    tx = G.to_torch_bf16(x)
+    names = ("fp8_weight_stacked", "fp8_scale_stacked", "fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose", "fp8_scale_is_pow2")
+
+    def recache():
+        for e in experts:
+            for w in (e.w1, e.w2):
+                for name in names:
+                    if hasattr(w, name):
+                        delattr(w, name)
+        U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True, using_pow2_scale=True)
+
+    recache()
+    node = U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True)
+    first = node.forward(tx, tp, rows).clone()
+    again = node.forward(tx, tp, rows)
+    assert torch.equal(first.view(torch.int16), again.view(torch.int16))
+    assert len(node._ue8m0_memo) == 2                       # w1 and w2 scales, converted once
+    # new weights, new cache
+    with torch.no_grad():
+        for e in experts:
+            e.w1.mul_(4.0)
+            e.w2.mul_(0.5)
+    recache()
+    fresh = U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True).forward(tx, tp, rows)
+    same_node = node.forward(tx, tp, rows)
+    assert torch.equal(fresh.view(torch.int16), same_node.view(torch.int16))
+    assert not torch.equal(first.view(torch.int16), same_node.view(torch.int16))
+    # the cache rewritten in place
+    with torch.no_grad():
+        for e in experts:
+            e.w1.mul_(0.25)
+    w0 = experts[0].w1
+    q, s = F8.fused_stack_transpose_quant([e.w1 for e in experts], transpose=True, using_pow2_scale=True)
+    w0.fp8_weight_stacked_transpose.copy_(q)
+    w0.fp8_scale_stacked_transpose.copy_(s)
+    q, s = F8.fused_stack_transpose_quant([e.w1 for e in experts], transpose=False, using_pow2_scale=True)
+    w0.fp8_weight_stacked.copy_(q)
+    w0.fp8_scale_stacked.copy_(s)
+    fresh = U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True).forward(tx, tp, rows)
+    same_node = node.forward(tx, tp, rows)
+    assert torch.equal(fresh.view(torch.int16), same_node.view(torch.int16))
+
+
 @pytest.mark.parametrize("ue8m0", [False, True])
 def test_moe_node_backward_fused_gradient_quantization_is_bit_identical(ue8m0):
     # backward quantizes out_grad and do1 once (row-wise + transposed from one read) or twice (the
