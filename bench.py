@@ -693,6 +693,9 @@ def main():
             "traffic_source": None if traffic_rec is None else {k: traffic_rec[k] for k in ("commit", "command") if k in traffic_rec},
             "algorithmic_bytes": int(w1q[counts > 0].numel() + Mpad * H + Mpad * 2 * I * 2),
             "launch_ms": round(kms["gemm_up_gate"], 4),
+            # the launch sits below the ridge of the published roofline (465 flop per algorithmic byte against 625):
+            # the same launch against the 8 TB/s HBM peak, algorithmic bytes over launch time
+            "frac_hbm": round((w1q[counts > 0].numel() + Mpad * H + Mpad * 2 * I * 2) / (kms["gemm_up_gate"] * 1e-3) / 8e12, 4),
         },
     }
     if not args.no_quant:
