@@ -358,6 +358,81 @@ def test_grouped_masked(dg):
             assert G.rel_fro(_bf(got[e, :m]), _bf(exp[e, :m])) <= BLOCK_FRO
 
 
+def _random_fp8_problem(rows_total, K, E, N, seed):
+    """Random e4m3 codes (no NaN codes) and positive scales made on the GPU: for the capacity-edge cases below, which
+    compare two launches of verified kernels bit for bit and need no oracle data."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    def codes(shape):
+        c = torch.randint(0, 256, shape, dtype=torch.int16, device="cuda", generator=g)
+        c = torch.where((c & 0x7F) == 0x7F, c & 0xF0, c)          # 0x7F / 0xFF are NaN
+        return (c & 0x77 | (c & 0x80)).to(torch.uint8).view(torch.float8_e4m3fn)     # small magnitudes: sums stay finite
+    a = codes((rows_total, K))
+    sa = (torch.rand((K // 128, rows_total), device="cuda", generator=g) + 0.5).t()
+    b = codes((E, N, K))
+    sb = torch.rand((E, N // 128, K // 128), device="cuda", generator=g) + 0.5
+    return a, sa, b, sb
+
+
+@pytest.mark.parametrize("row_tiles", [2048, 2049])
+def test_grouped_contiguous_at_the_capacity_of_the_tile_group_table(dg, row_tiles):
+    """2048 row tiles is the most the persistent kernel orders by expert; one more and it walks fixed groups.  700
+    experts of one to five tiles each (some empty, padding tiles in between): every expert's rows must equal the dense
+    launch on them."""
+    E, N, K = 700, 256, 384
+    rng = np.random.default_rng(row_tiles)
+    blocks, left = [], row_tiles
+    for e in range(E):
+        if left == 0:
+            break
+        n = int(min(left, rng.integers(0, 6)))
+        if n:
+            blocks.append((e, n))
+            left -= n
+        if left and rng.random() < 0.05:
+            blocks.append((-1, 1))
+            left -= 1
+    if left:
+        blocks.append((E - 1, left))
+    Mtot = 128 * row_tiles
+    assert 128 * sum(n for _, n in blocks) == Mtot
+    a, sa, b, sb = _random_fp8_problem(Mtot, K, E, N, seed=row_tiles)
+    m_idx = torch.from_numpy(np.concatenate([np.full(128 * n, e, dtype=np.int32) for e, n in blocks])).cuda()
+    out = torch.full((Mtot, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dg.m_grouped_fp8_gemm_nt_contiguous((a, sa), (b, sb), out, m_idx)
+    ref = torch.full_like(out, float("nan"))
+    start = 0
+    for e, n in blocks:
+        r = 128 * n
+        if e >= 0:
+            dg.fp8_gemm_nt((a[start:start + r], sa[start:start + r]), (b[e], sb[e]), ref[start:start + r])
+        start += r
+    skipped = m_idx < 0
+    assert torch.isnan(out[skipped].float()).all()
+    assert torch.isfinite(ref[~skipped].float()).all()
+    assert torch.equal(out[~skipped].view(torch.int16), ref[~skipped].view(torch.int16))
+
+
+@pytest.mark.parametrize("E,Mmax", [(256, 1024), (256, 1152), (257, 128)])
+def test_grouped_masked_at_the_capacity_of_the_row_tile_list(dg, E, Mmax):
+    """256 experts x 8 row tiles fill the persistent kernel's list of valid row tiles; 9 tiles each, or 257 experts,
+    take the two-workgroup kernel."""
+    N, K = 256, 384
+    a, sa, b, sb = _random_fp8_problem(E * Mmax, K, E, N, seed=E + Mmax)
+    a, sa = a.view(E, Mmax, K), sa.contiguous().view(E, Mmax, K // 128)
+    rng = np.random.default_rng(E * Mmax)
+    masked = rng.integers(0, Mmax + 1, size=E).astype(np.int32)
+    masked[:3] = [Mmax, 0, 1]
+    out = torch.full((E, Mmax, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dg.m_grouped_fp8_gemm_nt_masked((a, sa), (b, sb), out, torch.from_numpy(masked).cuda(), int(masked.mean()))
+    ref = torch.empty((Mmax, N), dtype=torch.bfloat16, device="cuda")
+    for e in list(range(0, E, 17)) + [1, 2, E - 1]:
+        m = int(masked[e])
+        assert torch.isnan(out[e, m:].float()).all(), f"expert {e}: rows beyond masked_m were written"
+        if m:
+            dg.fp8_gemm_nt((a[e], sa[e]), (b[e], sb[e]), ref)
+            assert torch.equal(out[e, :m].view(torch.int16), ref[:m].view(torch.int16)), f"expert {e}"
+
+
 @pytest.mark.parametrize("E,Mmax", [(260, 128), (3, 200), (40, 384)])
 def test_grouped_masked_layouts_of_both_kernels(dg, E, Mmax):
     """More than 256 experts and a capacity that is not a multiple of 128 take the two-workgroup kernel, 40 experts of
