@@ -321,8 +321,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Deep-pipeline forward kernel for shapes without ragged tiles (Prows % 256 == 0, Qrows % 128 == 0,
-// at least three K blocks; dense and contiguous-grouped layouts).
+// Deep-pipeline forward kernel for shapes without ragged tiles: Qrows % 128 == 0, Prows % 128 == 0 and at least 256
+// (a last column tile may be half new), at least three K blocks; dense, contiguous-grouped and masked layouts.
 //   * One persistent workgroup per compute unit walks its XCD's run of 128x256 tiles; 144 KB of LDS
 //     is a three-stage ring of [P 32 KB | Q 16 KB] blocks that runs on ACROSS tile boundaries: the
 //     copies of the block two ahead are issued during the current block, one between every other
