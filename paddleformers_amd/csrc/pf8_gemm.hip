@@ -306,7 +306,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd128(const GemmArgs a) {
         if (rt >= row_hi || row >= q_rows_total) continue;
         uint8_t* dst = outb + (row * a.ldo + col) * 2;
         if (col + 8 <= a.Prows) {
-            *reinterpret_cast<uint4*>(dst) = v;
+            st16(dst, v);
         } else if (col + 4 <= a.Prows) {
             *reinterpret_cast<uint2*>(dst) = make_uint2(v.x, v.y);
         }
@@ -706,7 +706,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                         const int rl = er + 4 * i;
                         const int64_t row = cq * BQ + wq * 64 + half * 32 + rl;
                         const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
-                        if (c_rows) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
+                        if (c_rows) st16(outb + (row * a.ldo + col) * 2, v);
                     }
                 }
                 __syncthreads();      // the pair's gate and up rows are both staged
@@ -763,7 +763,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                     const int rl = er + 4 * i;                        // row inside the 32-row slice
                     const int64_t row = cq * BQ + wq * 64 + half * 32 + rl;
                     const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
-                    if (store && (!masked || rl < c_rows - wq * 64 - half * 32)) *reinterpret_cast<uint4*>(outb + (row * a.ldo + col) * 2) = v;
+                    if (store && (!masked || rl < c_rows - wq * 64 - half * 32)) st16(outb + (row * a.ldo + col) * 2, v);
                 }
             }
         }
@@ -991,7 +991,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
         for (int i = 0; i < 16; ++i) {
             int64_t row = q0 + wq * 64 + er + 4 * i;
             if (row > a.Qrows - 1) row = a.Qrows - 1;
-            old[i] = *reinterpret_cast<const f32x4*>(outb + (row * a.ldo + col_c) * 4);
+            { const uint4 ow = ld16(outb + (row * a.ldo + col_c) * 4); old[i] = (f32x4){u2f(ow.x), u2f(ow.y), u2f(ow.z), u2f(ow.w)}; }
         }
     } else {
 #pragma unroll
@@ -1002,7 +1002,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
         const int64_t row = q0 + wq * 64 + er + 4 * i;
         const f32x4 v = *reinterpret_cast<const f32x4*>(ep + (er + 4 * i) * EP_LD + ec * 16);
         const f32x4 o = (f32x4){old[i].x + v.x, old[i].y + v.y, old[i].z + v.z, old[i].w + v.w};
-        if (row < a.Qrows && col_ok) *reinterpret_cast<f32x4*>(outb + (row * a.ldo + col) * 4) = o;
+        if (row < a.Qrows && col_ok) st16(outb + (row * a.ldo + col) * 4, make_uint4(f2u(o.x), f2u(o.y), f2u(o.z), f2u(o.w)));
     }
 #undef PF8_DMA
 #undef PF8_LOAD_S

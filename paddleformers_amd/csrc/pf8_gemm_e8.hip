@@ -353,7 +353,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {
                 for (int it = 0; it < 4; ++it) {
                     const int rl = er + 4 * it;                        // staged row = li of the producer
                     const uint4 v = *reinterpret_cast<const uint4*>(ep + rl * EP_LD + ec * 16);
-                    *reinterpret_cast<uint4*>(row_out + vo + it * vo_step) = v;
+                    st16(row_out + vo + it * vo_step, v);
                 }
             });
         }

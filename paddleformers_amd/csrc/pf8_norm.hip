@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_fwd(const uint16_t* __restrict
 #pragma unroll
         for (int j = 0; j < MAXC; ++j) {
             const int64_t c = tid + 256 * j;
-            xp[j] = c < chunks ? xr[c] : make_uint4(0, 0, 0, 0);
+            xp[j] = c < chunks ? ld16(xr + c) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < MAXC; ++j) {
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_fwd(const uint16_t* __restrict
     } else {
         for (int64_t c = tid; c < chunks; c += 256) {
             float v[8];
-            unpack8(xr[c], v);
+            unpack8(ld16(xr + c), v);
 #pragma unroll
             for (int i = 0; i < 8; ++i) ss = __builtin_fmaf(v[i], v[i], ss);
         }
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_fwd(const uint16_t* __restrict
         o.y = pack_bf16(v[2] * iv * g[2], v[3] * iv * g[3]);
         o.z = pack_bf16(v[4] * iv * g[4], v[5] * iv * g[5]);
         o.w = pack_bf16(v[6] * iv * g[6], v[7] * iv * g[7]);
-        yr[c] = o;
+        st16(yr + c, o);
     };
     if (MAXC > 0) {
 #pragma unroll
@@ -105,8 +105,8 @@ __global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict
             xp[j] = make_uint4(0, 0, 0, 0);
             dp[j] = make_uint4(0, 0, 0, 0);
             if (c < chunks) {
-                xp[j] = xr[c];
-                dp[j] = dr[c];
+                xp[j] = ld16(xr + c);
+                dp[j] = ld16(dr + c);
             }
         }
 #pragma unroll
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_bwd(const uint16_t* __restrict
                 unpack8(wr[c], gv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) o[i] = dv[i] * gv[i] * iv - xv[i] * k;
-                oxr[c] = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+                st16(oxr + c, make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7])));
             }
         }
     }

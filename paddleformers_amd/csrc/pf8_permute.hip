@@ -81,7 +81,7 @@ __global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restri
         if (tid == 0) atomicOr(overflow, 2);
         for (int64_t r = base; r < limit; ++r) {
             uint4* dst = reinterpret_cast<uint4*>(out_x + r * row_bytes);
-            for (int64_t i = tid; i < row_bytes / 16; i += 1024) dst[i] = make_uint4(0, 0, 0, 0);
+            for (int64_t i = tid; i < row_bytes / 16; i += 1024) st16(dst + i, make_uint4(0, 0, 0, 0));
             if (out_xs)
                 for (int64_t i = tid; i < scale_cols; i += 1024) out_xs[r * scale_cols + i] = 0.0f;
             if (out_probs && tid == 0) out_probs[r] = 0.0f;
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void k_permute_zero_pad(PermuteArgs pa, int64_
     const int64_t r = pa.row_start[e] + pa.count[e] + blockIdx.x;
     if (r >= pa.row_start[e + 1]) return;
     uint4* dst = reinterpret_cast<uint4*>(out_x + r * row_bytes);
-    for (int64_t i = threadIdx.x; i < row_bytes / 16; i += 256) dst[i] = make_uint4(0, 0, 0, 0);
+    for (int64_t i = threadIdx.x; i < row_bytes / 16; i += 256) st16(dst + i, make_uint4(0, 0, 0, 0));
     if (out_xs)
         for (int64_t i = threadIdx.x; i < scale_cols; i += 256) out_xs[r * scale_cols + i] = 0.0f;
 }
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void k_permute_gather(const uint8_t* __restric
 #pragma unroll
     for (int i = 0; i < MAXV; ++i) {
         const int64_t c = tid + 256 * i;
-        if (c < chunks) v[i] = reinterpret_cast<const uint4*>(x + t * row_bytes)[c];
+        if (c < chunks) v[i] = ld16(reinterpret_cast<const uint4*>(x + t * row_bytes) + c);
     }
     for (int k = 0; k < topk; ++k) {
         const int e = routemap[t * topk + k];
@@ -127,9 +127,9 @@ __global__ __launch_bounds__(256) void k_permute_gather(const uint8_t* __restric
 #pragma unroll
         for (int i = 0; i < MAXV; ++i) {
             const int64_t c = tid + 256 * i;
-            if (c < chunks) dst[c] = v[i];
+            if (c < chunks) st16(dst + c, v[i]);
         }
-        for (int64_t c = tid + 256 * (int64_t)MAXV; c < chunks; c += 256) dst[c] = reinterpret_cast<const uint4*>(x + t * row_bytes)[c];
+        for (int64_t c = tid + 256 * (int64_t)MAXV; c < chunks; c += 256) st16(dst + c, *(reinterpret_cast<const uint4*>(x + t * row_bytes) + c));
         if (xs)
             for (int64_t c = tid; c < scale_cols; c += 256) out_xs[r * scale_cols + c] = xs[t * scale_cols + c];
         if (out_probs && tid == 0) out_probs[r] = probs ? probs[t * topk + k] : 0.0f;
