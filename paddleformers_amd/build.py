@@ -53,18 +53,41 @@ def up_to_date() -> bool:
 
 
 def kernels_with_scratch(remarks):
-    """(kernel, bytes per lane) for every kernel whose resource-usage remark reports scratch memory.  The hand-scheduled
-    kernels are written to fit the register file: a spill there is a performance bug, and scratch makes every launch
-    depend on a per-queue scratch allocation."""
-    found, name = [], None
+    """(kernels seen, [(kernel, bytes per lane)] of those that report scratch memory) from the compiler's
+    kernel-resource-usage remarks.  The hand-scheduled kernels are written to fit the register file: a spill there
+    is a performance bug, and scratch makes every launch depend on a per-queue scratch allocation."""
+    seen, found, name = [], [], None
     for l in remarks:
         if "Function Name:" in l:
             name = l.split("Function Name:")[1].split("[")[0].strip()
-        elif "ScratchSize [bytes/lane]:" in l:
+        elif "ScratchSize [bytes/lane]:" in l and name:
             n = int(l.split("ScratchSize [bytes/lane]:")[1].split("[")[0].strip())
-            if n > 0 and name:
+            seen.append(name)
+            if n > 0:
                 found.append((name, n))
-    return found
+            name = None
+    return seen, found
+
+
+# kernels whose register budget was fitted by hand: each must show up in the remarks, or the check has gone blind
+EXPECTED_KERNELS = ("k_gemm_fwd_deep", "k_gemm_fwd128", "k_gemm_wgrad", "k_gemm_e8", "k_quant_rowcol", "k_quant_1x128")
+
+
+def check_scratch(remarks) -> str:
+    """Raises when a kernel spills to scratch (PF8_ALLOW_SCRATCH=1 turns that into the returned warning text, for a
+    compiler release that spills a few bytes where this one does not) and when the remarks the check reads are not
+    there at all (a changed wording must not let it pass vacuously)."""
+    seen, spilling = kernels_with_scratch(remarks)
+    missing = [k for k in EXPECTED_KERNELS if not any(k in name for name in seen)]
+    if missing:
+        raise RuntimeError("resource remarks not found for: " + ", ".join(missing) +
+                           " (the -Rpass-analysis=kernel-resource-usage output has changed; the scratch check cannot run)")
+    if not spilling:
+        return ""
+    msg = "kernels that spill registers to scratch memory (bytes per lane): " + ", ".join(f"{k}: {v}" for k, v in spilling)
+    if os.environ.get("PF8_ALLOW_SCRATCH") == "1":
+        return "warning: " + msg
+    raise RuntimeError(msg + " (set PF8_ALLOW_SCRATCH=1 to build anyway)")
 
 
 def build(force: bool = False, verbose: bool = False) -> str:
@@ -86,10 +109,13 @@ def build(force: bool = False, verbose: bool = False) -> str:
     out = "\n".join(kept)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + out)
-    spilling = kernels_with_scratch(lines)
-    if spilling:
+    try:
+        warning = check_scratch(lines)
+    except RuntimeError:
         os.remove(LIB)
-        raise RuntimeError("kernels that spill registers to scratch memory (bytes per lane): " + ", ".join(f"{k}: {v}" for k, v in spilling))
+        raise
+    if warning:
+        print(warning, file=sys.stderr)
     if verbose and out.strip():
         print(out)
     return LIB

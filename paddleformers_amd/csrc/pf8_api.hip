@@ -3,6 +3,7 @@
 
 #include <atomic>
 #include <cstdio>
+#include <cstdlib>
 
 namespace {
 thread_local char g_err[512] = "";
@@ -42,6 +43,15 @@ int pf8_effective_cus() {
 bool pf8_cus_capped() {
     const int cap = g_num_cus.load();
     return cap > 0 && cap < device_cus();
+}
+
+void pf8_note_once(int id, const char* msg) {
+    static std::atomic<uint32_t> raised{0};
+    const uint32_t bit = 1u << (id & 31);
+    if (raised.fetch_or(bit) & bit) return;
+    const char* q = getenv("PF8_QUIET");
+    if (q && q[0] == '1') return;
+    fprintf(stderr, "pf8: %s\n", msg);
 }
 
 extern "C" int pf8_version(void) { return 100; }

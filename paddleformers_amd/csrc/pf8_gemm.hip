@@ -71,7 +71,9 @@ typedef const __attribute__((address_space(1))) void gbl_void;
 // global_load_lds as a pending FLAT access and then turns every later LDS wait into a full drain
 // (lgkmcnt(0)), which serialises the fragment reads of a K block with its first MFMA.  The copy
 // is tracked by vmcnt in hardware; the K loop waits for it explicitly before its barrier.
-// M0 is written here and used by nothing else in these kernels.
+// M0 is written here without being listed as clobbered: this compiler treats M0 as a reserved register (a clobber
+// entry for it is rejected with a warning and ignored), never allocates it, and sets it itself only directly in
+// front of an instruction that reads it, so no value of the compiler's lives in M0 across this statement.
 __device__ __forceinline__ void dma16_to_lds(const uint8_t* src, uint32_t lds_dst) {
     const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(m0v) : "memory");
@@ -359,6 +361,10 @@ __device__ __forceinline__ float e8m0_to_f32(uint32_t b) { return u2f(b ? b << 2
 // outputs is the 16 lanes of a DPP row, exactly the tile of the standalone SwiGLU quantizer, whose arithmetic is
 // restated operation for operation (bf16(silu(g) * u), bf16(. * p), amax, scale, quotient), so bytes and scales are
 // bit-identical to the un-fused pair of launches.
+// Capacities of the persistent kernel's LDS tables, shared by the kernel and by the host code that decides which
+// launches it may take: row tiles whose expert order is tabulated, experts of a masked launch, dynamic LDS of the ring.
+constexpr int kDeepSegTiles = 2048, kDeepMaskedExperts = 256, kDeepDynLds = 147456;
+
 template <int SQL, int SF = 0, int FUSE = 0, int MASKED = 0>
 __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     using ST = typename std::conditional<SF == 1, uint8_t, float>::type;
@@ -399,10 +405,14 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     // of 1.74 GB per up+gate launch (hit rate 64% against 53%) and 0.74 GB instead of 0.96 GB on the down GEMM; the
     // launches get 3% and 2% shorter.  seg_tab[q] = first tile of q's group | tiles in it << 16; every workgroup
     // builds the table for itself: the first tile of each run by a prefix maximum over the tiles, 256 at a time.
-    __shared__ uint32_t seg_tab[2048];
-    __shared__ int16_t seg_eid[2048 + 2];                  // expert of every row tile (one global load each), -1 = padding
+    __shared__ uint32_t seg_tab[kDeepSegTiles];
+    __shared__ int16_t seg_eid[MASKED ? 2 : kDeepSegTiles + 2];   // expert of every row tile (one global load each), -1 = padding
     __shared__ int seg_wave_max[2][4];
-    const bool ordered = grouped && q_tiles <= 2048 && a.E <= 32767;
+    __shared__ int seg_valid[MASKED ? kDeepMaskedExperts : 1];
+    __shared__ int seg_total;
+    static_assert(sizeof(seg_tab) + sizeof(seg_eid) + sizeof(seg_wave_max) + sizeof(seg_valid) + sizeof(int) + kDeepDynLds <= 163840,
+                  "static tables plus the dynamic ring exceed the 160 KB of LDS a workgroup can have");
+    const bool ordered = !MASKED && grouped && q_tiles <= kDeepSegTiles && a.E <= 32767;
     if (ordered) {
         constexpr int CAP = 12;
         const int qt = (int)q_tiles;
@@ -445,8 +455,6 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
     // Masked layout (a [E, Mmax, K], masked_m[e] valid rows; at most 256 experts and 2048 row tiles): only the row tiles
     // that hold valid rows are walked.  Every workgroup lists them for itself: seg_tab[slot] = expert | tile << 16,
     // seg_valid[e] = valid rows; a row tile of expert e is row tile e * (Mmax / 128) + tile of the [E * Mmax, K] matrix.
-    __shared__ int seg_valid[256];
-    __shared__ int seg_total;
     const int mt = (int)(a.Qrows / BQ);                    // row tiles per expert (masked)
     if (masked) {
         int valid = 0, cnt = 0;
@@ -1022,9 +1030,15 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
         // up+gate / down GEMMs of 32 experts with a skewed 8192-row load, +2% on those of 128 experts with 131072 rows,
         // within 3% either way on dense products from 3 to 64 K blocks and up to 32 rounds of tiles.
         const bool aligned = a.Prows % 128 == 0 && a.Prows >= 256 && a.Qrows % 128 == 0 && a.red >= 384 &&
-                             (a.group != GROUP_MASKED || (a.E <= 256 && (int64_t)a.E * (a.Qrows / 128) <= 2048));
+                             (a.group != GROUP_MASKED || (a.E <= kDeepMaskedExperts && (int64_t)a.E * (a.Qrows / 128) <= kDeepSegTiles));
         const int64_t cus = pf8_effective_cus();
         const bool deep = aligned;
+        if (a.group == GROUP_MASKED && !aligned && a.Prows % 128 == 0 && a.Prows >= 256 && a.Qrows % 128 == 0 && a.red >= 384)
+            pf8_note_once(PF8_NOTE_MASKED_TABLE, "masked grouped GEMM beyond 256 experts or 2048 row tiles: taking the two-workgroup kernel "
+                                                 "(one grid row per expert) instead of the persistent one");
+        if (deep && a.group == GROUP_CONTIG && a.Qrows / 128 > kDeepSegTiles)
+            pf8_note_once(PF8_NOTE_GROUPED_ORDER, "contiguous grouped GEMM with more than 2048 row tiles: tiles are walked in plain groups of 16 "
+                                                  "row tiles instead of expert by expert (more weight re-reads per XCD)");
         if (deep) {
             // persistent: one workgroup per compute unit (or per tile of an XCD's run, if fewer); the masked layout is
             // one launch over all experts (the kernel walks the row tiles that hold valid rows)
@@ -1033,9 +1047,9 @@ static int launch_gemm(const GemmArgs& a, int mode, dim3 grid, hipStream_t st, c
             if (w < 1) w = 1;
             if (w > per_xcd) w = per_xcd;
             dim3 gd((unsigned)(8 * w), 1);
-            if (a.group == GROUP_MASKED) hipLaunchKernelGGL((k_gemm_fwd_deep<0, 0, 0, 1>), gd, dim3(256), 147456, st, a);
-            else if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0>), gd, dim3(256), 147456, st, a);
-            else hipLaunchKernelGGL((k_gemm_fwd_deep<1>), gd, dim3(256), 147456, st, a);
+            if (a.group == GROUP_MASKED) hipLaunchKernelGGL((k_gemm_fwd_deep<0, 0, 0, 1>), gd, dim3(256), kDeepDynLds, st, a);
+            else if (a.sq_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0>), gd, dim3(256), kDeepDynLds, st, a);
+            else hipLaunchKernelGGL((k_gemm_fwd_deep<1>), gd, dim3(256), kDeepDynLds, st, a);
         } else {
             // under a compute-unit budget: two workgroups per budgeted unit, each walking several tiles
             if (pf8_cus_capped()) {
@@ -1075,12 +1089,12 @@ static int ensure_lds_attr() {
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_wgrad<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 69632);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd128<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 81920);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0, 0, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
-    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 147456);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0>), hipFuncAttributeMaxDynamicSharedMemorySize, kDeepDynLds);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1>), hipFuncAttributeMaxDynamicSharedMemorySize, kDeepDynLds);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, kDeepDynLds);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0, 0, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, kDeepDynLds);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<0, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, kDeepDynLds);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fwd_deep<1, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, kDeepDynLds);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm", hipGetErrorString(e));
     done.fetch_or(bit, std::memory_order_release);
     return PF8_OK;
@@ -1100,7 +1114,7 @@ int pf8_launch_deep_ue8m0(const uint8_t* p, const uint8_t* q, const uint8_t* sp8
     int64_t w = cus / 8;
     if (w < 1) w = 1;
     if (w > per_xcd) w = per_xcd;
-    hipLaunchKernelGGL((k_gemm_fwd_deep<1, 1>), dim3((unsigned)(8 * w)), dim3(256), 147456, stream, g);
+    hipLaunchKernelGGL((k_gemm_fwd_deep<1, 1>), dim3((unsigned)(8 * w)), dim3(256), kDeepDynLds, stream, g);
     return pf8_check_launch(where);
 }
 
@@ -1173,8 +1187,8 @@ extern "C" int pf8_grouped_gemm_swiglu_quant_nt_contiguous(const uint8_t* a, con
     if (w < 1) w = 1;
     if (w > per_xcd) w = per_xcd;
     dim3 gd((unsigned)(8 * w), 1);
-    if (sa_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0, 0, 1>), gd, dim3(256), 147456, (hipStream_t)stream, g);
-    else hipLaunchKernelGGL((k_gemm_fwd_deep<1, 0, 1>), gd, dim3(256), 147456, (hipStream_t)stream, g);
+    if (sa_layout == 0) hipLaunchKernelGGL((k_gemm_fwd_deep<0, 0, 1>), gd, dim3(256), kDeepDynLds, (hipStream_t)stream, g);
+    else hipLaunchKernelGGL((k_gemm_fwd_deep<1, 0, 1>), gd, dim3(256), kDeepDynLds, (hipStream_t)stream, g);
     return pf8_check_launch(__func__);
 }
 

@@ -15,6 +15,10 @@ int pf8_check_launch(const char* where);
 int pf8_effective_cus();
 // true when pf8_set_num_cus holds a budget below the current device's compute units
 bool pf8_cus_capped();
+// one line on stderr the first time note `id` (0..31) is raised in this process (PF8_QUIET=1 silences it): for launches
+// that leave a kernel's fast path because of a size limit, which would otherwise only show as a slower call
+void pf8_note_once(int id, const char* msg);
+enum { PF8_NOTE_GROUPED_ORDER = 0, PF8_NOTE_MASKED_TABLE = 1 };
 
 // Launches the 128x256 persistent forward kernel on a contiguous-grouped GEMM whose scales are UE8M0
 // bytes (implemented next to that kernel; used by the UE8M0 entry point when a skewed expert load

@@ -577,9 +577,35 @@ def fused_rms_norm_ext_grad(x: torch.Tensor, norm_weight: torch.Tensor, invvar: 
 # ---------------------------------------------------------------------------------------------
 
 
+_PERMUTE_FLAGS = {}      # device index -> int32[1], OR of the flags of every moe_permute since the last check
+
+
+def _permute_flag(dev: torch.device) -> torch.Tensor:
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    t = _PERMUTE_FLAGS.get(idx)
+    if t is None:
+        t = _PERMUTE_FLAGS[idx] = torch.zeros(1, dtype=torch.int32, device=torch.device("cuda", idx))
+    return t
+
+
+def moe_permute_check(device=None) -> None:
+    """Read and clear the flag word the `moe_permute` calls on `device` have OR-ed into since the last check
+    (one device-to-host copy, i.e. one synchronisation) and raise ValueError when any of them saw routing that
+    disagrees with its `tokens_per_expert`."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    t = _permute_flag(dev)
+    flags = int(t.item())
+    if flags:
+        t.zero_()
+    if flags & 1:
+        raise ValueError("expert_routemap_topk routes more tokens to an expert than tokens_per_expert allows")
+    if flags & 2:
+        raise ValueError("expert_routemap_topk routes fewer tokens to an expert than tokens_per_expert says")
+
+
 def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expert_routemap_topk: torch.Tensor,
                 expert_prob_topk: Optional[torch.Tensor], num_experts: int, tokens_per_expert: Sequence[int],
-                padding_alignment: int, do_gather: bool = True, validate: bool = True):
+                padding_alignment: int, do_gather: bool = True, validate: bool = False):
     """Gather the routed copies of every token into expert-sorted order, every expert's segment
     padded with zero rows to a multiple of `padding_alignment`.
 
@@ -588,9 +614,11 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
     expert_routemap_topk int32 [T, topk] (negative = unused slot); expert_prob_topk fp32 [T, topk].
     Returns (hidden_states_unzipped [Mpad, H], zipped_expertwise_rowmap int32 [T, num_experts],
     token_prob_unzipped fp32 [Mpad, 1], scale_unzipped fp32 [Mpad, H/128] or None).
-    Counts that do not match the routing raise ValueError (a token routed to an expert beyond its
-    `tokens_per_expert` count is dropped; rows of an overstated count are written as zeros); that check
-    reads a flag back from the device (one synchronisation), `validate=False` skips it.
+    Counts that do not match the routing (a token routed to an expert beyond its `tokens_per_expert` count is
+    dropped; rows of an overstated count are written as zeros) set a sticky flag word that lives on the device for
+    the life of the process: the call itself neither allocates nor reads it back, as the reference's operator has no
+    device-to-host round trip either.  `moe_permute_check()` reads and clears the flag wherever the caller
+    synchronises anyway; `validate=True` does so right after this call (one synchronisation) and raises ValueError.
     """
     if not do_gather:
         raise ValueError("do_gather=False is not supported")
@@ -624,16 +652,12 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
             raise ValueError("scale must be float32 [T, H/128]")
         xs = scale.contiguous()
         out_s = torch.empty((mpad, H // 128), dtype=torch.float32, device=dev)
-    overflow = torch.zeros(1, dtype=torch.int32, device=dev)
+    overflow = _permute_flag(dev)
     cnt = (C.c_int64 * num_experts)(*counts)
     _lib.call("pf8_moe_permute", _p(x), int(is_fp8), _p(xs), _p(rm), _p(pr), T, H, topk, num_experts, cnt, a, _p(out_x), _p(rowmap),
               _p(out_p), _p(out_s), _p(overflow), _stream())
     if validate:
-        flags = int(overflow.item())
-        if flags & 1:
-            raise ValueError("expert_routemap_topk routes more tokens to an expert than tokens_per_expert allows")
-        if flags & 2:
-            raise ValueError("expert_routemap_topk routes fewer tokens to an expert than tokens_per_expert says")
+        moe_permute_check(dev)
     return out_x, rowmap, out_p, out_s
 
 

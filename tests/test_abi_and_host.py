@@ -178,3 +178,32 @@ def test_ernie_and_inference_mirrors_host_logic_without_a_gpu():
         K8.act_quant(torch.zeros((4, 128), dtype=torch.bfloat16))
     with pytest.raises(AssertionError):
         K8.act_quant(torch.zeros((4, 100), dtype=torch.bfloat16))
+
+
+def _remark(name, scratch):
+    tag = "[-Rpass-analysis=kernel-resource-usage]"
+    return [f"x.hip:1:1: remark: Function Name: {name} {tag}", f"x.hip:1:1: remark:     VGPRs: 200 {tag}",
+            f"x.hip:1:1: remark:     ScratchSize [bytes/lane]: {scratch} {tag}", f"x.hip:1:1: remark:     VGPRs Spill: 0 {tag}"]
+
+
+def test_build_scratch_check_on_canned_remarks(monkeypatch):
+    """The build refuses a kernel that spills to scratch, can be told to warn instead, and fails when the remarks it
+    reads are missing rather than passing vacuously."""
+    from paddleformers_amd import build as B
+
+    clean = [l for k in B.EXPECTED_KERNELS for l in _remark(f"_ZN3pf8{len(k)}{k}ILi0EEEvNS_8GemmArgsE", 0)]
+    seen, spilling = B.kernels_with_scratch(clean)
+    assert len(seen) == len(B.EXPECTED_KERNELS) and spilling == []
+    assert B.check_scratch(clean) == ""
+    dirty = clean + _remark("_ZN3pf814k_rms_norm_fwdILi2EEEvPKt", 156)
+    monkeypatch.delenv("PF8_ALLOW_SCRATCH", raising=False)
+    with pytest.raises(RuntimeError, match="k_rms_norm_fwd.*156"):
+        B.check_scratch(dirty)
+    monkeypatch.setenv("PF8_ALLOW_SCRATCH", "1")
+    assert B.check_scratch(dirty).startswith("warning:") and "156" in B.check_scratch(dirty)
+    # remarks in a wording the parser does not know: nothing is seen, and that is an error of its own
+    reworded = [l.replace("ScratchSize [bytes/lane]:", "Scratch bytes per lane =") for l in dirty]
+    with pytest.raises(RuntimeError, match="resource remarks not found"):
+        B.check_scratch(reworded)
+    with pytest.raises(RuntimeError, match="resource remarks not found"):
+        B.check_scratch(["clang: warning: something else"])

@@ -102,7 +102,17 @@ def test_tokens_through_unzip_node_experts_zip_node_and_back(fp8_tokens):
     assert unzip.zipped_expertwise_rowmap is None               # the node drops its state after backward
     assert dx.shape == (T, H) and dprobs.shape == (T, topk)
 
+    # the two reordering passes that carry numbers, pinned to the bit against the oracle on the very rows they were
+    # handed (fp32 sum of a token's copies in slot order, bf16 out), independently of the FP8 noise of the MLP between them
+    ey, _ = O.moe_unpermute(G.from_torch_bf16(o3), rowmap.cpu().numpy(), rm, row_probs.cpu().numpy(), T, E)
+    assert (G.from_torch_bf16(y) == ey).all(), "ZipNode.forward differs from the oracle's moe_unpermute"
+    edx, edp = O.moe_unpermute(G.from_torch_bf16(dx_rows), rowmap.cpu().numpy(), rm, probs_grad_rows.cpu().numpy(), T, E)
+    assert (G.from_torch_bf16(dx) == edx).all(), "UnZipNode.backward differs from the oracle's moe_unpermute"
+    assert (dprobs.cpu().numpy() == edp).all(), "UnZipNode.backward: probability gradients differ from the oracle's"
+
     ref_y, ref_dx, ref_dp, ref_dw1, ref_dw2 = _fp32_layer(x, rm, probs, w1, w2, dy)
+    errs = {"y": G.rel_fro(y.float().cpu().numpy(), ref_y), "dx": G.rel_fro(dx.float().cpu().numpy(), ref_dx)}
+    print("layer errors vs fp32:", errs)
     tol = 0.09
     assert G.rel_fro(y.float().cpu().numpy(), ref_y) < tol
     assert G.rel_fro(dx.float().cpu().numpy(), ref_dx) < tol
@@ -134,3 +144,30 @@ def test_zip_node_backward_takes_fp8_gradients_with_scales():
         UnZipNode().forward(G.to_torch_bf16(x), trm, tpr, topk + 1, E, counts)
     with pytest.raises(RuntimeError):
         UnZipNode().backward(rows, T, None, trm, E)
+
+
+def test_reordering_nodes_issue_no_host_synchronisation():
+    """The reference's moe_permute / moe_unpermute calls return without a device-to-host round trip
+    (moe_utils.py:157-181, 205-212); torch's synchronisation debug mode turns any `.item()` / blocking copy into an
+    error, so the four node passes must get through it."""
+    from paddleformers_amd import functional as F8
+    from paddleformers_amd.moe_utils import UnZipNode, ZipNode
+
+    T, H, E, topk = 200, 384, 5, 2
+    rm, probs, counts, *_, x, dy = _layer(T, H, 128, E, topk, seed=31)
+    trm, tpr = torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda()
+    xt, dyt = G.to_torch_bf16(x), G.to_torch_bf16(dy)
+    unzip, zipn = UnZipNode(), ZipNode()
+    F8.moe_permute_check()                       # allocates the flag word of this device, outside the guarded region
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        rows, rowmap, up, _ = unzip.forward(xt, trm, tpr, topk, E, counts)
+        y = zipn.forward(rows, rowmap, trm, up, T, E)
+        drows = zipn.backward(dyt, trm, tpr, topk, E, counts)
+        dx, dp = unzip.backward(drows, T, up, trm, E)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    torch.cuda.synchronize()
+    F8.moe_permute_check()                       # consistent counts: nothing flagged
+    assert y.shape == (T, H) and dx.shape == (T, H) and dp.shape == (T, topk)

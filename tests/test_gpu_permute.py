@@ -96,16 +96,20 @@ def test_permute_rejects_inconsistent_counts_and_bad_arguments(F):
     short = list(counts)
     short[int(np.argmax(counts))] -= 1
     with pytest.raises(ValueError, match="tokens_per_expert"):
-        F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, short, 128)
+        F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, short, 128, validate=True)
     # a count that overstates what the routing sends: flagged, and with the check skipped the rows no token
     # lands on hold zeros (probability 0), like padding rows, not whatever the allocation held
     big = int(np.argmax(counts))
     over = list(counts)
     over[big] += 3
     with pytest.raises(ValueError, match="fewer tokens"):
-        F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, over, 128)
+        F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, over, 128, validate=True)
     torch.full((E * 256, H), float("nan"), dtype=torch.bfloat16, device="cuda")     # poison what the allocator hands out next
-    ox, orow, op, _ = F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, over, 128, validate=False)
+    ox, orow, op, _ = F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, over, 128)
+    # the default call reads nothing back: the flag stays on the device until somebody asks, and asking clears it
+    with pytest.raises(ValueError, match="fewer tokens"):
+        F.moe_permute_check()
+    F.moe_permute_check()
     start = sum((c + 127) // 128 * 128 for c in over[:big])
     assert not ox[start + counts[big]:start + over[big]].any() and not op[start + counts[big]:start + over[big]].any()
     gx, _, gp, _ = F.moe_permute(x, None, torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda(), E, counts, 128)

@@ -335,6 +335,10 @@ def test_quant_transpose_config4_full_size_property(F):
     eq, es = O.quant_1x128(bits[:2048], 0)
     _same(G.from_torch_fp8(q[:2048]), eq, "slab bytes vs oracle")
     _scales_same(s.t()[:2048].contiguous().cpu().numpy(), es, "slab scales vs oracle")
+    # the column-scaled copy straight against the oracle as well: 1024 columns of x = 1024 rows of the transposed output
+    eqt, est = O.quant_1x128(np.ascontiguousarray(bits[:, 1024:2048].T), 1)
+    _same(G.from_torch_fp8(qt[1024:2048]), eqt, "column-scaled slab bytes vs oracle")
+    _scales_same(st[:, 1024:2048].contiguous().cpu().numpy(), est, "column-scaled slab scales vs oracle")
 
 
 def test_padding_and_quant_input_unaligned_rows(F):
