@@ -201,6 +201,29 @@ int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_lay
                                    const float* sb, int E, int64_t Mtot, int64_t N, int64_t K,
                                    const int32_t* m_indices, uint16_t* out, pf8_stream_t stream);
 
+/* Fragment-major copy of a quantized weight, the operand form of the *_fm GEMMs below.  The reference keeps its FP8
+ * weights as plain [N, K] tensors that only deep_gemm reads (cache_fp8_weight / fp8_quant_weight,
+ * transformers/fp8_utils.py:97-137, 403-437); this library's GEMMs take the same bytes re-ordered into the order in which
+ * a wavefront's matrix instructions consume them: w e4m3 [E][N, K] row-major ->
+ *     wf[e][n / 64][k / 128][ps 0..3][h 0..1][lane 0..63][16 bytes],
+ * the 16 bytes being k = 128 (k / 128) + 32 (lane / 16) + 16 h .. + 15 of row n = 64 (n / 64) + 16 ps + lane % 16.
+ * A permutation of the same E * N * K bytes (no re-quantization; scales are shared with the plain form).
+ * N multiple of 64, K multiple of 128. */
+int pf8_weight_to_fragment_major(const uint8_t* w, int E, int64_t N, int64_t K, uint8_t* wf, pf8_stream_t stream);
+
+/* 1 when the *_fm GEMMs take this shape (M % 128 == 0, N % 256 == 0, K % 512 == 0), else 0.  No device access. */
+int pf8_gemm_fm_supported(int64_t M, int64_t N, int64_t K);
+
+/* deep_gemm.fp8_gemm_nt / m_grouped_fp8_gemm_nt_contiguous (transformers/fp8_utils.py:289-302, 949-954, 1002-1007) on a
+ * fragment-major weight b_fm (pf8_weight_to_fragment_major of the [N, K] / [E, N, K] operand); everything else as in
+ * pf8_gemm_nt / pf8_grouped_gemm_nt_contiguous, and the results are bit-identical to theirs.  Shapes outside
+ * pf8_gemm_fm_supported are rejected (the caller keeps the plain weight for those). */
+int pf8_gemm_nt_fm(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b_fm, const float* sb, int64_t M,
+                   int64_t N, int64_t K, uint16_t* out, int64_t ldo, pf8_stream_t stream);
+int pf8_grouped_gemm_nt_contiguous_fm(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b_fm,
+                                      const float* sb, int E, int64_t Mtot, int64_t N, int64_t K,
+                                      const int32_t* m_indices, uint16_t* out, pf8_stream_t stream);
+
 /* The up+gate grouped GEMM with the activation quantizer of the down projection in its epilogue: the two calls of
  * FP8GroupGemmMlpFunctionNode.forward -- deep_gemm.m_grouped_fp8_gemm_nt_contiguous (transformers/fp8_utils.py:949-954)
  * and fused_weighted_swiglu_act_quant(o1, probs, using_pow2_scaling) (:981-987; un-fused definition ernie

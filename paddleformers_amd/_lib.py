@@ -41,6 +41,10 @@ SIGNATURES = {
     "pf8_gemm_nt_1d1d_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp],
     "pf8_gemm_nt_1d1d_f32_pow2": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp],
     "pf8_grouped_gemm_nt_contiguous": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp],
+    "pf8_weight_to_fragment_major": [_vp, _i32, _i64, _i64, _vp, _vp],
+    "pf8_gemm_fm_supported": [_i64, _i64, _i64],
+    "pf8_gemm_nt_fm": [_vp, _vp, _i32, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
+    "pf8_grouped_gemm_nt_contiguous_fm": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp],
     "pf8_grouped_gemm_swiglu_quant_nt_contiguous": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i32, _vp],
     "pf8_gemm_nt_ue8m0": [_vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
     "pf8_grouped_gemm_nt_contiguous_ue8m0": [_vp, _vp, _i64, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp],

@@ -26,10 +26,48 @@ def get_num_sms() -> int:
     return int(_lib.lib().pf8_get_num_cus())
 
 
+class FragmentMajor:
+    """A quantized weight [N, K] or [E, N, K] whose bytes are stored in the order the matrix instructions consume
+    them (`pf8_weight_to_fragment_major`): pass it in place of the plain e4m3 tensor of a `(b, sb)` pair and
+    `fp8_gemm_nt` / `m_grouped_fp8_gemm_nt_contiguous` run the kernel that loads weight fragments straight into
+    registers.  Same bytes, same scales, bit-identical results; made once per cached weight by `to_fragment_major`.
+    No counterpart in the reference, whose FP8 weight cache is read by deep_gemm only."""
+
+    __slots__ = ("data", "shape")
+
+    def __init__(self, data: torch.Tensor, shape):
+        self.data, self.shape = data, tuple(shape)
+
+    def dim(self) -> int:
+        return len(self.shape)
+
+
+def fragment_major_supported(M: int, N: int, K: int) -> bool:
+    """Shapes the fragment-major kernels take (whole 128-row and 256-column tiles, K a multiple of 512)."""
+    return bool(_lib.lib().pf8_gemm_fm_supported(int(M), int(N), int(K)))
+
+
+def to_fragment_major(w: torch.Tensor) -> FragmentMajor:
+    """Fragment-major copy of an e4m3 weight [N, K] or [E, N, K] (N % 64 == 0, K % 128 == 0)."""
+    _dev(w, "w")
+    if w.dtype != FP8 or w.dim() not in (2, 3):
+        raise ValueError("w must be float8_e4m3fn [N, K] or [E, N, K]")
+    w = w if w.is_contiguous() else w.contiguous()
+    E = w.shape[0] if w.dim() == 3 else 1
+    N, K = w.shape[-2], w.shape[-1]
+    out = torch.empty_like(w)
+    _lib.call("pf8_weight_to_fragment_major", _p(w), E, N, K, _p(out), _stream())
+    return FragmentMajor(out, w.shape)
+
+
 def _check_pair(pair, what) -> Tuple[torch.Tensor, torch.Tensor]:
     if not (isinstance(pair, (tuple, list)) and len(pair) == 2):
         raise ValueError(f"{what} must be a (tensor, scale) pair")
     t, s = pair
+    if isinstance(t, FragmentMajor):
+        _dev(t.data, what)
+        _dev(s, what + " scale")
+        return t, s
     _dev(t, what)
     _dev(s, what + " scale")
     if t.dtype != FP8:
@@ -95,7 +133,17 @@ def fp8_gemm_nt(a, b, out: torch.Tensor, c: Optional[torch.Tensor] = None, recip
         raise ValueError(f"out must be [{M}, {N}]")
     if M == 0 or N == 0:
         return out
+    fm = isinstance(tb, FragmentMajor)
+    if fm and (recipe is not None or c is not None or _is_ue8m0(sa) or _is_ue8m0(sb) or not fragment_major_supported(M, N, K)
+               or out.dtype != torch.bfloat16 or out.stride(-1) != 1 or out.stride(0) % 8 != 0 or out.data_ptr() % 16 != 0):
+        raise ValueError("a fragment-major weight serves the default recipe with fp32 scales, M % 128 == 0, N % 256 == 0, K % 512 == 0")
     ta = ta if ta.is_contiguous() else ta.contiguous()
+    if fm:
+        sa, lay = _scale_layout_of(sa, M, K // 128, "a scale")
+        if tuple(sb.shape) != (N // 128, K // 128) or sb.dtype != torch.float32:
+            raise ValueError(f"b scale must be float32 [{N // 128}, {K // 128}]")
+        _lib.call("pf8_gemm_nt_fm", _p(ta), _p(sa), lay, _p(tb.data), _p(sb.contiguous()), M, N, K, _p(out), out.stride(0), _stream())
+        return out
     tb = tb if tb.is_contiguous() else tb.contiguous()
     if recipe is not None and tuple(recipe) == (1, 1, 128):
         if out.dtype != torch.float32 or not out.is_contiguous():
@@ -174,8 +222,17 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
     if Mtot == 0 or N == 0:
         return out
     ta = ta if ta.is_contiguous() else ta.contiguous()
-    tb = tb if tb.is_contiguous() else tb.contiguous()
     m_indices = m_indices if m_indices.is_contiguous() else m_indices.contiguous()
+    if isinstance(tb, FragmentMajor):
+        if _is_ue8m0(sa) or _is_ue8m0(sb) or not fragment_major_supported(Mtot, N, K):
+            raise ValueError("a fragment-major weight serves fp32 scales, Mtot % 128 == 0, N % 256 == 0, K % 512 == 0")
+        sa, lay = _scale_layout_of(sa, Mtot, K // 128, "a scale")
+        if tuple(sb.shape) != (E, N // 128, K // 128) or sb.dtype != torch.float32:
+            raise ValueError(f"b scale must be float32 [{E}, {N // 128}, {K // 128}]")
+        _lib.call("pf8_grouped_gemm_nt_contiguous_fm", _p(ta), _p(sa), lay, _p(tb.data), _p(sb.contiguous()), E, Mtot, N, K,
+                  _p(m_indices), _p(out), _stream())
+        return out
+    tb = tb if tb.is_contiguous() else tb.contiguous()
     if _is_ue8m0(sa) != _is_ue8m0(sb):
         raise ValueError("UE8M0 scales must be given for both operands or for neither")
     if _is_ue8m0(sa):
