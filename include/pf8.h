@@ -205,18 +205,21 @@ int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_lay
  * weights as plain [N, K] tensors that only deep_gemm reads (cache_fp8_weight / fp8_quant_weight,
  * transformers/fp8_utils.py:97-137, 403-437); this library's GEMMs take the same bytes re-ordered into the order in which
  * a wavefront's matrix instructions consume them: w e4m3 [E][N, K] row-major ->
- *     wf[e][n / 64][k / 128][ps 0..3][h 0..1][lane 0..63][16 bytes],
- * the 16 bytes being k = 128 (k / 128) + 32 (lane / 16) + 16 h .. + 15 of row n = 64 (n / 64) + 16 ps + lane % 16.
+ *     wf[e][n / 64][k / 128][pf 0..1][kh 0..1][h 0..1][lane 0..63][16 bytes],
+ * the 16 bytes being k = 128 (k / 128) + 64 kh + 32 (lane / 32) + 16 h .. + 15 of row n = 64 (n / 64) + 32 pf + lane % 32
+ * (the A-operand fragments of v_mfma_f32_32x32x64_f8f6f4, in the order a wavefront consumes them).
  * A permutation of the same E * N * K bytes (no re-quantization; scales are shared with the plain form).
  * N multiple of 64, K multiple of 128. */
 int pf8_weight_to_fragment_major(const uint8_t* w, int E, int64_t N, int64_t K, uint8_t* wf, pf8_stream_t stream);
 
-/* 1 when the *_fm GEMMs take this shape (M % 128 == 0, N % 256 == 0, K % 512 == 0), else 0.  No device access. */
+/* 1 when the *_fm GEMMs take this shape (M % 128 == 0, N % 256 == 0, K % 128 == 0, K >= 384), else 0.  No device access. */
 int pf8_gemm_fm_supported(int64_t M, int64_t N, int64_t K);
 
 /* deep_gemm.fp8_gemm_nt / m_grouped_fp8_gemm_nt_contiguous (transformers/fp8_utils.py:289-302, 949-954, 1002-1007) on a
  * fragment-major weight b_fm (pf8_weight_to_fragment_major of the [N, K] / [E, N, K] operand); everything else as in
- * pf8_gemm_nt / pf8_grouped_gemm_nt_contiguous, and the results are bit-identical to theirs.  Shapes outside
+ * pf8_gemm_nt / pf8_grouped_gemm_nt_contiguous (same scale factors, same order of the K blocks; a block's product is formed
+ * by two chained 32x32x64 matrix instructions instead of one 16x16x128, so results agree with theirs to the matrix pipe's
+ * precision, within the same bars against the reference formulation).  Shapes outside
  * pf8_gemm_fm_supported are rejected (the caller keeps the plain weight for those). */
 int pf8_gemm_nt_fm(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b_fm, const float* sb, int64_t M,
                    int64_t N, int64_t K, uint16_t* out, int64_t ldo, pf8_stream_t stream);

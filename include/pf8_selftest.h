@@ -25,6 +25,17 @@ int pf8_debug_div_encode(const float* x, const float* s, int64_t n, uint8_t* out
 /* Self-test hook: out[i] = silu(x[i]) with the device restatement of the oracle's expf. */
 int pf8_debug_silu(const float* x, int64_t n, float* out, pf8_stream_t stream);
 
+/* Measurement hook: pf8_grouped_gemm_nt_contiguous_fm (sa_layout 1) from an instantiation that reads the shader clock
+ * at four points of every K block.  cycles int64 [workgroups][8], workgroups >= the launch's grid (at most one per
+ * compute unit): per workgroup, wavefront 0's sums over all its K blocks of {MFMAs 0..23 with their copies and fragment
+ * reads, the counted wait for the next block's data, the barrier, MFMAs 24..31 with the next block's first reads},
+ * then {epilogue cycles, K blocks, tiles, unused}.  The output is the GEMM's; the launch is a few percent slower.
+ * ablate != 0 leaves instructions out (the output is then garbage) to price them: 2 = the weight-fragment loads, 4 = the
+ * activation and scale copies, 8 = the scale FMAs, 16 = the LDS fragment reads; sums of these where listed in the source. */
+int pf8_debug_grouped_gemm_fm_cycles(const uint8_t* a, const float* sa, const uint8_t* b_fm, const float* sb, int E,
+                                     int64_t Mtot, int64_t N, int64_t K, const int32_t* m_indices, uint16_t* out,
+                                     int64_t* cycles, int64_t workgroups, int ablate, pf8_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -54,6 +54,7 @@ SIGNATURES = {
     "pf8_grouped_gemm_nt_masked": [_vp, _vp, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _i32, _vp, _vp],
     "pf8_grouped_wgrad": [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _i32, _vp],
     "pf8_grouped_wgrad_pow2": [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _i32, _vp],
+    "pf8_debug_grouped_gemm_fm_cycles": [_vp, _vp, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _i32, _vp],
     "pf8_debug_copy": [_vp, _vp, _i64, _vp],
     "pf8_debug_encode": [_vp, _i64, _vp, _vp],
     "pf8_debug_div_encode": [_vp, _vp, _i64, _vp, _vp],

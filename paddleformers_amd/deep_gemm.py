@@ -30,7 +30,7 @@ class FragmentMajor:
     """A quantized weight [N, K] or [E, N, K] whose bytes are stored in the order the matrix instructions consume
     them (`pf8_weight_to_fragment_major`): pass it in place of the plain e4m3 tensor of a `(b, sb)` pair and
     `fp8_gemm_nt` / `m_grouped_fp8_gemm_nt_contiguous` run the kernel that loads weight fragments straight into
-    registers.  Same bytes, same scales, bit-identical results; made once per cached weight by `to_fragment_major`.
+    registers.  Same bytes, same scales, results equal to the plain kernels' to the matrix pipe's precision; made once per cached weight by `to_fragment_major`.
     No counterpart in the reference, whose FP8 weight cache is read by deep_gemm only."""
 
     __slots__ = ("data", "shape")
@@ -43,7 +43,7 @@ class FragmentMajor:
 
 
 def fragment_major_supported(M: int, N: int, K: int) -> bool:
-    """Shapes the fragment-major kernels take (whole 128-row and 256-column tiles, K a multiple of 512)."""
+    """Shapes the fragment-major kernels take (whole 128-row and 256-column tiles, at least three K blocks)."""
     return bool(_lib.lib().pf8_gemm_fm_supported(int(M), int(N), int(K)))
 
 
@@ -136,7 +136,7 @@ def fp8_gemm_nt(a, b, out: torch.Tensor, c: Optional[torch.Tensor] = None, recip
     fm = isinstance(tb, FragmentMajor)
     if fm and (recipe is not None or c is not None or _is_ue8m0(sa) or _is_ue8m0(sb) or not fragment_major_supported(M, N, K)
                or out.dtype != torch.bfloat16 or out.stride(-1) != 1 or out.stride(0) % 8 != 0 or out.data_ptr() % 16 != 0):
-        raise ValueError("a fragment-major weight serves the default recipe with fp32 scales, M % 128 == 0, N % 256 == 0, K % 512 == 0")
+        raise ValueError("a fragment-major weight serves the default recipe with fp32 scales, M % 128 == 0, N % 256 == 0, K % 128 == 0, K >= 384")
     ta = ta if ta.is_contiguous() else ta.contiguous()
     if fm:
         sa, lay = _scale_layout_of(sa, M, K // 128, "a scale")
@@ -225,7 +225,7 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
     m_indices = m_indices if m_indices.is_contiguous() else m_indices.contiguous()
     if isinstance(tb, FragmentMajor):
         if _is_ue8m0(sa) or _is_ue8m0(sb) or not fragment_major_supported(Mtot, N, K):
-            raise ValueError("a fragment-major weight serves fp32 scales, Mtot % 128 == 0, N % 256 == 0, K % 512 == 0")
+            raise ValueError("a fragment-major weight serves fp32 scales, Mtot % 128 == 0, N % 256 == 0, K % 128 == 0, K >= 384")
         sa, lay = _scale_layout_of(sa, Mtot, K // 128, "a scale")
         if tuple(sb.shape) != (E, N // 128, K // 128) or sb.dtype != torch.float32:
             raise ValueError(f"b scale must be float32 [{E}, {N // 128}, {K // 128}]")

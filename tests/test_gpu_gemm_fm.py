@@ -2,8 +2,9 @@
 `pf8_gemm_nt_fm`, `pf8_grouped_gemm_nt_contiguous_fm`) through the deep_gemm-named mirror, i.e. through the C ABI.
 
 The byte order is pinned by un-permuting on the host with the formula the header states; the GEMMs are compared with
-the CPU oracle at the bars of tests/test_gpu_gemm.py and, bit for bit, with the kernels that read the plain weight
-(same products, same scale factors, same order of the K blocks)."""
+the CPU oracle at the bars of tests/test_gpu_gemm.py and with the kernels that read the plain weight: same scale
+factors and order of the K blocks, but a K block's product comes from two chained 32x32x64 instructions instead of one
+16x16x128, so the two agree to the matrix pipe's own precision (a few 1e-6 of sum|a||b| per block), not to the bit."""
 import numpy as np
 import pytest
 
@@ -16,6 +17,7 @@ torch = pytest.importorskip("torch")
 
 REL_FRO = 1e-3
 BLOCK_FRO = 6e-4
+SAME_MATH_FRO = 2e-4   # against the plain-weight kernel: bf16 roundings that flip on a difference in the matrix pipe's last bits
 
 
 @pytest.fixture(scope="module")
@@ -29,8 +31,8 @@ def dg():
 def _fm_reference(w):
     """[E, N, K] bytes -> the fragment-major order, by the formula of include/pf8.h, in numpy."""
     E, N, K = w.shape
-    v = w.reshape(E, N // 64, 4, 16, K // 128, 4, 2, 16)        # e, n64, ps, li, kb, kg, h, byte
-    v = v.transpose(0, 1, 4, 2, 6, 5, 3, 7)                      # e, n64, kb, ps, h, kg, li, byte  (lane = 16 kg + li)
+    v = w.reshape(E, N // 64, 2, 32, K // 128, 2, 2, 2, 16)     # e, n64, pf, x, kb, kh, hh, h, byte
+    v = v.transpose(0, 1, 4, 2, 5, 7, 6, 3, 8)                   # e, n64, kb, pf, kh, h, hh, x, byte  (lane = 32 hh + x)
     return np.ascontiguousarray(v).reshape(E, N, K)
 
 
@@ -55,7 +57,7 @@ def _dense_case(M, N, K, seed):
     return a, sa, b, sb
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 256, 512), (384, 512, 1024), (256, 768, 2048), (1280, 256, 512)])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 384), (128, 256, 512), (384, 512, 1024), (256, 768, 2048), (1280, 256, 640), (256, 256, 1408)])
 @pytest.mark.parametrize("lay", [0, 1])
 def test_dense_fragment_major_against_oracle_and_plain_kernel(dg, M, N, K, lay):
     a, sa, b, sb = _dense_case(M, N, K, seed=M + N + K)
@@ -71,7 +73,7 @@ def test_dense_fragment_major_against_oracle_and_plain_kernel(dg, M, N, K, lay):
     assert G.rel_fro(O.bf16_bits_to_f32(got), O.bf16_bits_to_f32(blk)) <= BLOCK_FRO
     plain = torch.empty_like(out)
     dg.fp8_gemm_nt((ta, tsa), (tb, tsb), plain)
-    assert torch.equal(out.view(torch.int16), plain.view(torch.int16))
+    assert G.rel_fro(out.float().cpu().numpy(), plain.float().cpu().numpy()) <= SAME_MATH_FRO
 
 
 def test_dense_fragment_major_exact_integers(dg):
@@ -103,7 +105,9 @@ def _grouped_case(E, N, K, blocks, seed):
 
 @pytest.mark.parametrize("K,blocks", [
     (512, [(0, 1), (2, 3), (-1, 1), (1, 2)]),
+    (384, [(1, 2), (-1, 1), (0, 1), (3, 4)]),
     (1024, [(3, 13), (-1, 1), (1, 1), (2, 25), (-1, 2), (0, 2), (0, 1)]),
+    (896, [(e % 4, 1 + (e * 5) % 4) for e in range(12)]),
     (512, [(e % 4, 1 + (e * 7) % 3) for e in range(30)]),
 ])
 @pytest.mark.parametrize("lay", [0, 1])
@@ -126,7 +130,7 @@ def test_grouped_fragment_major_against_oracle_and_plain_kernel(dg, K, blocks, l
     # padding tiles are left untouched by both kernels
     valid = torch.from_numpy(m_idx >= 0).cuda()
     assert torch.isnan(out[~valid].float()).all()
-    assert torch.equal(out[valid].view(torch.int16), plain[valid].view(torch.int16))
+    assert G.rel_fro(out[valid].float().cpu().numpy(), plain[valid].float().cpu().numpy()) <= SAME_MATH_FRO
     exp = O.grouped_gemm_nt_contiguous(a, sa, b, sb, m_idx)
     got = G.from_torch_bf16(out)
     v = m_idx >= 0
@@ -138,11 +142,12 @@ def test_fragment_major_rejects_other_shapes_and_scales(dg):
     ta, tb = G.to_torch_fp8(a), G.to_torch_fp8(b)
     tsa, tsb = torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda()
     fm = dg.to_fragment_major(tb)
-    assert dg.fragment_major_supported(128, 256, 512) and not dg.fragment_major_supported(128, 384, 512)
-    assert not dg.fragment_major_supported(128, 256, 384) and not dg.fragment_major_supported(100, 256, 512)
-    with pytest.raises(ValueError):                             # K = 384 is not a multiple of 512
-        dg.fp8_gemm_nt((ta[:, :384].contiguous(), tsa[:, :3].contiguous()),
-                       (dg.to_fragment_major(tb[:, :384].contiguous()), tsb[:, :3].contiguous()),
+    assert dg.fragment_major_supported(128, 256, 512) and dg.fragment_major_supported(128, 256, 384)
+    assert not dg.fragment_major_supported(128, 384, 512) and not dg.fragment_major_supported(128, 256, 256)
+    assert not dg.fragment_major_supported(100, 256, 512)
+    with pytest.raises(ValueError):                             # K = 256: fewer than three K blocks
+        dg.fp8_gemm_nt((ta[:, :256].contiguous(), tsa[:, :2].contiguous()),
+                       (dg.to_fragment_major(tb[:, :256].contiguous()), tsb[:, :2].contiguous()),
                        torch.empty((128, 256), dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(ValueError):                             # UE8M0 scales go to the block-scaled kernel, which reads plain weights
         dg.fp8_gemm_nt((ta, tsa.to(torch.uint8)), (fm, tsb.to(torch.uint8)), torch.empty((128, 256), dtype=torch.bfloat16, device="cuda"))
