@@ -31,7 +31,9 @@ int pf8_debug_silu(const float* x, int64_t n, float* out, pf8_stream_t stream);
  * reads, the counted wait for the next block's data, the barrier, MFMAs 24..31 with the next block's first reads},
  * then {epilogue cycles, K blocks, tiles, unused}.  The output is the GEMM's; the launch is a few percent slower.
  * ablate != 0 leaves instructions out (the output is then garbage) to price them: 2 = the weight-fragment loads, 4 = the
- * activation and scale copies, 8 = the scale FMAs, 16 = the LDS fragment reads; sums of these where listed in the source. */
+ * activation and scale copies, 8 = the scale FMAs, 16 = the LDS fragment reads; built are 6 (no memory instructions), 8,
+ * 14 (only MFMAs and LDS reads left), 30 (only MFMAs, barriers and scalar code left) and 64 = every tile reads the
+ * operands of tile (0, 0), i.e. all operand traffic hits in the L2. */
 int pf8_debug_grouped_gemm_fm_cycles(const uint8_t* a, const float* sa, const uint8_t* b_fm, const float* sb, int E,
                                      int64_t Mtot, int64_t N, int64_t K, const int32_t* m_indices, uint16_t* out,
                                      int64_t* cycles, int64_t workgroups, int ablate, pf8_stream_t stream);

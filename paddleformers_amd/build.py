@@ -90,6 +90,29 @@ def check_scratch(remarks) -> str:
     raise RuntimeError(msg + " (set PF8_ALLOW_SCRATCH=1 to build anyway)")
 
 
+def check_fragment_ring(flags) -> None:
+    """pf8_gemm_fm.hip keeps its weight-fragment ring in AGPRs that only its inline assembly names; the compiler, which
+    sees them as free, must not have put anything of its own there.  It does so only through v_accvgpr_* copies, so the
+    device assembly of that file must hold none."""
+    import tempfile
+
+    src = os.path.join(CSRC, "pf8_gemm_fm.hip")
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "pf8_gemm_fm.s")
+        cmd = [hipcc()] + [f for f in flags if f not in ("-shared", "-fPIC") and not f.startswith("-Rpass")] + \
+              ["--offload-device-only", "-S", src, "-o", out]
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError("hipcc -S failed on pf8_gemm_fm.hip:\n" + proc.stdout)
+        text = open(out).read()
+    if "k_gemm_fm" not in text or "v_mfma_f32_32x32x64_f8f6f4" not in text:
+        raise RuntimeError("the device assembly of pf8_gemm_fm.hip does not look as expected; the AGPR check cannot run")
+    n = text.count("v_accvgpr")
+    if n:
+        raise RuntimeError(f"pf8_gemm_fm.hip: the compiler placed {n} accumulation-register copies of its own; they would "
+                           "overwrite the weight-fragment ring (lower the register pressure of k_gemm_fm)")
+
+
 def build(force: bool = False, verbose: bool = False) -> str:
     if not force and up_to_date():
         return LIB
@@ -111,6 +134,7 @@ def build(force: bool = False, verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed:\n" + out)
     try:
         warning = check_scratch(lines)
+        check_fragment_ring(FLAGS)
     except RuntimeError:
         os.remove(LIB)
         raise

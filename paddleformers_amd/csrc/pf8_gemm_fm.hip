@@ -89,11 +89,6 @@ __device__ __forceinline__ void fm_mfma_second(f32x16& d, const i32x8& q) {
     asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, a[%2:%3], %1, %0" : "+v"(d) : "v"(q), "n"(A), "n"(A + 7));
 }
 
-// timing experiments only: the copy without its M0 write (lands wherever M0 points)
-__device__ __forceinline__ void fm_dma16_keep_m0(uint32_t voff, const uint8_t* sbase) {
-    asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase) : "memory");
-}
-
 template <int SQL, int TRACE = 0>
 __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
     constexpr int BQ = 128;
@@ -203,7 +198,10 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
     if (!tile_coords(0, cq, cp)) return;
     auto expert_of = [&](int64_t qt) -> int {
         int e = 0;
-        if (grouped) asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(e) : "s"(a.m_indices + qt * BQ) : "memory");
+        // the tile index is the same in every lane, but comes out of a 64-bit division the compiler may carry out in vector
+        // registers: hand it to the scalar load as a scalar
+        const int qt_s = __builtin_amdgcn_readfirstlane((int)qt);
+        if (grouped) asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(e) : "s"(a.m_indices + (int64_t)qt_s * BQ) : "memory");
         return e;
     };
     const uint8_t *c_p, *c_q, *c_s, *n_p, *n_q, *n_s;
@@ -213,6 +211,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
         int e = expert_of(qt);
         store = e >= 0;
         if (e < 0) e = 0;                  // a padding tile is computed on expert 0's weights and not stored
+        if constexpr (TRACE & 64) { pt = 0; qt = 0; e = 0; }        // timing experiment: every tile reads the operands of tile (0, 0)
         pp = a.pf + (((int64_t)e * P64 + pt * 4 + wave) * KB) * 8192;
         qp = a.q + qt * BQ * a.red;
         if (wave < 2) sp_ = reinterpret_cast<const uint8_t*>(a.sq + (SQL == 1 ? qt * BQ : qt * BQ * KB));
@@ -232,8 +231,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
             if constexpr (!(TRACE & 2)) fm_pload<32 * TT + 4 * t, (t & 3) * 1024>(t < 4 ? p_voff0 : p_voff1, pp);
         } else {
             constexpr int c = I - 9;
-            if constexpr (TRACE & 32) fm_dma16_keep_m0(q_off, qp + c * q_cstep);
-            else if constexpr (!(TRACE & 4)) dma16_s(q_off, qp + c * q_cstep, lds_base + TT * STAGE + (4 * c + wave) * 1024);
+            if constexpr (!(TRACE & 4)) dma16_s(q_off, qp + c * q_cstep, lds_base + TT * STAGE + (4 * c + wave) * 1024);
         }
     };
     auto issue_all = [&](auto tc, const uint8_t* pp, const uint8_t* qp, const uint8_t* sp_) {
@@ -499,14 +497,11 @@ static int launch_fm(const char* where, const uint8_t* a, const float* sa, int s
         void (*k)(const FmArgs) = nullptr;
         switch (ablate) {
             case 0: k = k_gemm_fm<1, 1>; break;
-            case 2: k = k_gemm_fm<1, 1 | 2>; break;
-            case 4: k = k_gemm_fm<1, 1 | 4>; break;
             case 6: k = k_gemm_fm<1, 1 | 6>; break;
             case 8: k = k_gemm_fm<1, 1 | 8>; break;
-            case 16: k = k_gemm_fm<1, 1 | 16>; break;
             case 14: k = k_gemm_fm<1, 1 | 14>; break;
             case 30: k = k_gemm_fm<1, 1 | 30>; break;
-            case 32: k = k_gemm_fm<1, 1 | 32>; break;
+            case 64: k = k_gemm_fm<1, 1 | 64>; break;
             default: return pf8_fail(PF8_EINVAL, where, "unknown ablation");
         }
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, kFmDynLds);
