@@ -87,6 +87,18 @@ def _get_fp8_weight_and_scale(weight, stacked=False, transpose=False):
     return weight.fp8_weight, weight.fp8_scale
 
 
+def _cache_derived(holder, name, source, make):
+    """A tensor derived from the cached FP8 tensor `source` (its fragment-major copy, the UE8M0 bytes of its scales),
+    kept as attribute `name` of the weight object that holds the cache and rebuilt when the cache entry is another
+    tensor or has been written through torch since.  Writes through raw pointers (the C ABI, the Paddle binding)
+    bump no version counter and are not detected: whoever requantizes in place that way drops the attribute."""
+    slot = getattr(holder, name, None)
+    if slot is None or slot[0] is not source or slot[1] != source._version:
+        slot = (source, source._version, make())
+        setattr(holder, name, slot)
+    return slot[2]
+
+
 def fused_stack_quant(expert_weight_list, transpose=False, using_pow2_scale=False):
     """fp8_utils.py:91-102: use the per-step cache on expert 0's weight when present, else quantise.
     using_pow2_scale asks for power-of-two scales (the `use_ue8m0` mode): a cache written without
@@ -610,6 +622,9 @@ class FP8GroupGemmMlpFunctionNode:
         # has nothing to hide it behind), so what it buys is memory: with recompute_fwd_gate_up the bf16 o1 is never
         # written.  None = on exactly then; True / False force it.
         self.fuse_swiglu_epilogue = None
+        # the forward-type grouped GEMMs read a fragment-major copy of every cached FP8 weight whose shape the kernel
+        # takes (made on first use, kept next to the cache entry: one more FP8 copy of those weights); False = plain weights
+        self.use_fragment_major = True
         self._group_items = None
         self.m_indices = None
         self.input = None
@@ -640,51 +655,55 @@ class FP8GroupGemmMlpFunctionNode:
         counts = torch.tensor([int(t) for t in tokens_per_expert], dtype=torch.int64)
         return torch.repeat_interleave(torch.arange(len(tokens_per_expert), dtype=torch.int32), counts).to(dev)
 
-    def _grouped_gemm(self, a_fp8, a_scale, w_fp8, w_scale, out, m_indices):
-        """One forward-type grouped GEMM of the node; with use_ue8m0 the (power-of-two) scales go in as
-        exponent bytes and the work-item list of the node's own m_indices is built once and shared."""
+    def _grouped_gemm(self, a_fp8, a_scale, w_fp8, w_scale, out, m_indices, cache=None):
+        """One forward-type grouped GEMM of the node.  `cache` = (weight object holding the per-step FP8 cache, name of
+        the cached attribute `w_fp8` is a view of) or None when the weights were quantized on the fly.  fp32 scales:
+        the kernel that reads the fragment-major copy of the cached weight where the shape allows.  use_ue8m0: the
+        (power-of-two) scales go in as exponent bytes, the weights' converted once per cache contents, and the
+        work-item list of the node's own m_indices is built once and shared."""
         if not self.use_ue8m0:
-            deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, a_scale), (w_fp8, w_scale), out, m_indices)
+            w = w_fp8
+            if cache is not None and self.use_fragment_major and \
+                    deep_gemm.fragment_major_supported(a_fp8.shape[0], w_fp8.shape[1], w_fp8.shape[2]):
+                holder, name = cache
+                w = _cache_derived(holder, name + "_fragment_major", getattr(holder, name), lambda: deep_gemm.to_fragment_major(w_fp8))
+            deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, a_scale), (w, w_scale), out, m_indices)
             return
         items = None
         if m_indices is self.m_indices and a_fp8.shape[0] % 128 == 0:
             if self._group_items is None:
                 self._group_items = deep_gemm.build_group_items(m_indices)
             items = self._group_items
-        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, F8.scales_to_ue8m0(a_scale, check=False)),
-                                                   (w_fp8, self._weight_scale_bytes(w_scale)), out, m_indices, items=items)
-
-    def _weight_scale_bytes(self, w_scale):
-        """UE8M0 bytes of a weight scale tensor, converted once per tensor contents: the four weight operands of the
-        node keep their scales from call to call when the per-step weight cache holds them (fp8_quant_weight), so the
-        conversion is remembered under the tensor's storage, view and version counter (an in-place requantization
-        bumps the version; a new cache is a new storage; the source tensor is kept alive with its entry)."""
-        key = (w_scale.untyped_storage().data_ptr(), w_scale.storage_offset(), tuple(w_scale.shape), tuple(w_scale.stride()),
-               w_scale._version)
-        memo = self.__dict__.setdefault("_ue8m0_memo", {})
-        hit = memo.get(key)
-        if hit is None:
-            if len(memo) >= 8:                 # four operands, two generations
-                memo.clear()
-            hit = memo[key] = (w_scale, F8.scales_to_ue8m0(w_scale, check=False))
-        return hit[1]
+        if cache is not None:
+            holder, name = cache
+            scale_name = name.replace("fp8_weight", "fp8_scale")
+            w_bytes = _cache_derived(holder, scale_name + "_ue8m0", getattr(holder, scale_name),
+                                     lambda: F8.scales_to_ue8m0(w_scale, check=False))
+        else:
+            w_bytes = F8.scales_to_ue8m0(w_scale, check=False)
+        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, F8.scales_to_ue8m0(a_scale, check=False)), (w_fp8, w_bytes), out, m_indices,
+                                                   items=items)
 
     def _stacked(self, expert_w, transpose, num_expert):
+        """(e4m3 [E, N, K], scales [E, N/128, K/128], cache): the stacked quantized weights in the orientation asked for;
+        cache = (weight object, attribute name) when they are the per-step cache itself (then tensors derived from
+        them are kept next to it), None when they were quantized or transposed on the fly."""
         q, s = fused_stack_quant(expert_w, transpose=transpose, using_pow2_scale=self.use_ue8m0)
         q = q.reshape([num_expert, -1, q.shape[-1]])
         s = s.reshape([num_expert, -1, s.shape[-1]])
         w0 = expert_w[0]
         want, other = ("fp8_weight_stacked_transpose", "fp8_weight_stacked") if transpose else ("fp8_weight_stacked", "fp8_weight_stacked_transpose")
+        cache = (w0, want) if hasattr(w0, want) else None
         if hasattr(w0, other) and not hasattr(w0, want):
             q = q.contiguous().transpose(1, 2).contiguous()
             s = s.contiguous().transpose(1, 2).contiguous()
-        return q, s
+        return q, s, cache
 
     def fwd_gate_up(self, x, expert_w1, num_expert, tokens_per_expert, m_indices=None):
         """o1 [m_sum, 2I] = x [m_sum, H] . w1 (fp8_utils.py:913-959)."""
         if not self.is_split_group_gemm and self.m_indices is None:
             self.m_indices = self.gen_m_indices(tokens_per_expert)
-        w1_t_quant, w1_t_scale = self._stacked(expert_w1, True, num_expert)
+        w1_t_quant, w1_t_scale, w1_cache = self._stacked(expert_w1, True, num_expert)
         if x is None:
             x_fp8, x_scale = self.input_fp8, self.input_scale
             assert x_fp8 is not None and x_scale is not None
@@ -700,7 +719,7 @@ class FP8GroupGemmMlpFunctionNode:
             if self.is_split_group_gemm:
                 split_group_gemm(x_fp8, x_scale, w1_t_quant, w1_t_scale, tokens_per_expert, o1)
             else:
-                self._grouped_gemm(x_fp8, x_scale, w1_t_quant, w1_t_scale, o1, self.m_indices if m_indices is None else m_indices)
+                self._grouped_gemm(x_fp8, x_scale, w1_t_quant, w1_t_scale, o1, self.m_indices if m_indices is None else m_indices, w1_cache)
         if m_indices is None:
             self.input_fp8 = x_fp8
             self.input_scale = x_scale
@@ -711,7 +730,7 @@ class FP8GroupGemmMlpFunctionNode:
 
     def fwd_down(self, o1, unzipped_probs, expert_w2, num_expert, tokens_per_expert, m_indices=None, o3=None, clear_o1=False):
         """o3 [m_sum, H] = quant(swiglu(o1) * probs) . w2 (fp8_utils.py:965-1009)."""
-        w2_quant, w2_scale = self._stacked(expert_w2, True, num_expert)
+        w2_quant, w2_scale, w2_cache = self._stacked(expert_w2, True, num_expert)
         unzipped_probs = unzipped_probs.squeeze(-1)
         o2_fp8, o2_scale = F8.fused_weighted_swiglu_act_quant(o1, unzipped_probs, using_pow2_scaling=True)
         o3_shape = [o2_fp8.shape[0], w2_quant.shape[1]]
@@ -723,12 +742,12 @@ class FP8GroupGemmMlpFunctionNode:
             if self.is_split_group_gemm:
                 split_group_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, tokens_per_expert, o3)
             else:
-                self._grouped_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, o3, m_indices if self.fwd_subbatch else self.m_indices)
+                self._grouped_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, o3, m_indices if self.fwd_subbatch else self.m_indices, w2_cache)
         return o3
 
     def bwd_dowm_input(self, expert_w2, unzipped_grad, o1, tokens_per_expert, m_indices=None, unzipped_probs=None):
         """do2_s [m_sum, I] = do3 . w2^T, then the SwiGLU backward (fp8_utils.py:1011-1052)."""
-        bw_w2_quant, bw_w2_scale = self._stacked(expert_w2, False, len(expert_w2))
+        bw_w2_quant, bw_w2_scale, bw_w2_cache = self._stacked(expert_w2, False, len(expert_w2))
         if isinstance(unzipped_grad, tuple):
             unzipped_grad_fp8, unzipped_grad_scale = unzipped_grad
             unzipped_grad_scale = unzipped_grad_scale.t().contiguous().t()
@@ -743,14 +762,14 @@ class FP8GroupGemmMlpFunctionNode:
                 split_group_gemm(unzipped_grad_fp8, unzipped_grad_scale, bw_w2_quant, bw_w2_scale, tokens_per_expert, do2_s)
             else:
                 self._grouped_gemm(unzipped_grad_fp8, unzipped_grad_scale, bw_w2_quant, bw_w2_scale, do2_s,
-                                   m_indices if self.bwd_subbatch else self.m_indices)
+                                   m_indices if self.bwd_subbatch else self.m_indices, bw_w2_cache)
         do1, probs_grad, o2_s = F8.fused_swiglu_weighted_bwd(o1, do2_s, unzipped_probs)
         return do1, o2_s, probs_grad
 
     def bwd_gate_up_input(self, do1, expert_w1, tokens_per_expert, m_indices=None, dx=None):
         """dx [m_sum, H] = do1 . w1^T (fp8_utils.py:1058-1094).  do1: bf16, or the (fp8, scale) pair of
         its row-wise quantization (scale [m_sum, 2I/128] as a view of [2I/128, m_sum] memory)."""
-        bw_w1_quant, bw_w1_scale = self._stacked(expert_w1, False, len(expert_w1))
+        bw_w1_quant, bw_w1_scale, bw_w1_cache = self._stacked(expert_w1, False, len(expert_w1))
         if isinstance(do1, tuple):
             do1_fp8, do1_scale = do1
         else:
@@ -767,7 +786,7 @@ class FP8GroupGemmMlpFunctionNode:
             if self.is_split_group_gemm:
                 split_group_gemm(do1_fp8, do1_scale, bw_w1_quant, bw_w1_scale, tokens_per_expert, dx)
             else:
-                self._grouped_gemm(do1_fp8, do1_scale, bw_w1_quant, bw_w1_scale, dx, m_indices if self.bwd_subbatch else self.m_indices)
+                self._grouped_gemm(do1_fp8, do1_scale, bw_w1_quant, bw_w1_scale, dx, m_indices if self.bwd_subbatch else self.m_indices, bw_w1_cache)
         return dx
 
     def fused_transpose_split_quant(self, x, scale, tokens_per_expert, pow_2_scales):
@@ -890,7 +909,7 @@ class FP8GroupGemmMlpFunctionNode:
         that the fused kernel takes the shapes."""
         if self.m_indices is None:
             self.m_indices = self.gen_m_indices(tokens_per_expert)
-        w1_t_quant, w1_t_scale = self._stacked(expert_w1, True, num_expert)
+        w1_t_quant, w1_t_scale, w1_cache = self._stacked(expert_w1, True, num_expert)
         if x is None:
             x_fp8, x_scale = self.input_fp8, self.input_scale
             assert x_fp8 is not None and x_scale is not None
@@ -911,9 +930,9 @@ class FP8GroupGemmMlpFunctionNode:
             self.input_scale = x_scale
         if keep_o1:
             self.o1 = o1
-        w2_quant, w2_scale = self._stacked(expert_w2, True, num_expert)
+        w2_quant, w2_scale, w2_cache = self._stacked(expert_w2, True, num_expert)
         o3 = torch.empty([Mtot, w2_quant.shape[1]], dtype=expert_w1[0].dtype, device=x_fp8.device)
-        self._grouped_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, o3, m_indices if self.fwd_subbatch else self.m_indices)
+        self._grouped_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, o3, m_indices if self.fwd_subbatch else self.m_indices, w2_cache)
         return o3
 
     @torch.no_grad()

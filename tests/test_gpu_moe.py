@@ -314,7 +314,11 @@ def test_moe_node_ue8m0_weight_scale_bytes_follow_the_weight_cache():
     first = node.forward(tx, tp, rows).clone()
     again = node.forward(tx, tp, rows)
     assert torch.equal(first.view(torch.int16), again.view(torch.int16))
-    assert len(node._ue8m0_memo) == 2                       # w1 and w2 scales, converted once
+    # the bytes of the w1 and w2 scales are kept next to the cache they were made from, converted once
+    kept = experts[0].w1.fp8_scale_stacked_transpose_ue8m0
+    assert kept[0] is experts[0].w1.fp8_scale_stacked_transpose and experts[0].w2.fp8_scale_stacked_transpose_ue8m0[2].dtype == torch.uint8
+    node.forward(tx, tp, rows)
+    assert experts[0].w1.fp8_scale_stacked_transpose_ue8m0 is kept
     # new weights, new cache
     with torch.no_grad():
         for e in experts:
@@ -495,3 +499,52 @@ def test_moe_node_deferred_weight_gradients_run_at_flush_on_another_stream(stack
     for e, (ex, (r1, r2)) in enumerate(zip(experts, ref)):
         assert torch.equal(ex.w1.main_grad, r1) and torch.equal(ex.w2.main_grad, r2), f"expert {e}"
         assert bool(r1.any()) == (rows[e] > 0)
+
+
+def test_moe_node_reads_fragment_major_copies_of_the_cached_weights():
+    """With the per-step FP8 weight cache in place the node's forward-type grouped GEMMs read a fragment-major copy of
+    every cached weight whose shape the kernel takes, made once and kept next to the cache entry; the results are those of
+    the plain-weight kernels, and a replaced cache entry is picked up."""
+    from paddleformers_amd import fp8_utils as U
+
+    E, H, I = 3, 512, 384                    # 2I = 768 and H = 512 are multiples of 256; I = 384 is not (dgrad-down stays plain)
+    rows = [256, 0, 384]
+    _, _, experts, x, probs = _make(E, H, I, rows, seed=41)
+    dout = G.bf16_normal((sum(rows), H), seed=42, std=1e-3)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    tx, tdo = G.to_torch_bf16(x), G.to_torch_bf16(dout)
+    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True)
+
+    def run(fragment_major):
+        for e in experts:
+            e.w1.main_grad = None
+            e.w2.main_grad = None
+        node = U.FP8GroupGemmMlpFunctionNode(_Map(experts))
+        node.use_fragment_major = fragment_major
+        o3 = node.forward(tx, tp, rows).clone()
+        dx, pg = node.backward(tdo, tp, rows)
+        return o3, dx.clone(), pg.clone()
+
+    plain = run(False)
+    w0, v0 = experts[0].w1, experts[0].w2
+    assert not hasattr(w0, "fp8_weight_stacked_transpose_fragment_major")
+    fm = run(True)
+    for a, b in zip(plain, fm):
+        assert torch.equal(a.view(torch.int16) if a.dtype == torch.bfloat16 else a, b.view(torch.int16) if b.dtype == torch.bfloat16 else b)
+    kept = w0.fp8_weight_stacked_transpose_fragment_major
+    assert kept[0] is w0.fp8_weight_stacked_transpose and isinstance(kept[2], U.deep_gemm.FragmentMajor)
+    assert hasattr(v0, "fp8_weight_stacked_transpose_fragment_major") and hasattr(w0, "fp8_weight_stacked_fragment_major")
+    assert not hasattr(v0, "fp8_weight_stacked_fragment_major")          # [E, I, H] with I = 384: not a shape the kernel takes
+    run(True)
+    assert w0.fp8_weight_stacked_transpose_fragment_major is kept        # made once
+    # a new cache entry (next optimizer step) is another tensor: its copy replaces the old one
+    with torch.no_grad():
+        for e in experts:
+            e.w1.mul_(2.0)
+    for name in ("fp8_weight_stacked", "fp8_scale_stacked", "fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose"):
+        delattr(w0, name)
+    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True)
+    fresh_plain, fresh_fm = run(False), run(True)
+    assert torch.equal(fresh_plain[0].view(torch.int16), fresh_fm[0].view(torch.int16))
+    assert not torch.equal(fresh_fm[0].view(torch.int16), fm[0].view(torch.int16))
+    assert w0.fp8_weight_stacked_transpose_fragment_major is not kept
