@@ -51,7 +51,7 @@ def traffic_from_summary(kernel_name):
 
 
 # the kernel the up+gate grouped GEMM of the headline workload runs on (what rocprofv3 --kernel-trace names it)
-ROOFLINE_KERNEL = "pf8::k_gemm_fwd_deep<1, 0, 0, 0>"
+ROOFLINE_KERNEL = "pf8::k_gemm_fm<1, 0>"
 
 
 def zipf_counts(total, E, s, seed, n_empty=2, pad=128):
@@ -214,6 +214,10 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     b, sb = qweights(1, N, K)
     o = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
     out["dense_config2_8192x4096x7168"] = dict(tkern(lambda: deep_gemm.fp8_gemm_nt((a, sa.T), (b[0], sb[0]), o)), flop=2.0 * M * N * K)
+    # the same product from the fragment-major copy of the weight (what the layers keep next to their FP8 weight cache)
+    bfm = deep_gemm.to_fragment_major(b[0])
+    out["dense_config2_fragment_major"] = dict(tkern(lambda: deep_gemm.fp8_gemm_nt((a, sa.T), (bfm, sb[0]), o)), flop=2.0 * M * N * K)
+    del bfm
     # the same GEMM with power-of-two scales as exponent bytes: block-scaled MFMA kernel
     a, sa = qact(M, K, True)
     b, sb = qweights(1, N, K, True)
@@ -251,6 +255,11 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
         sa_l, s1_l = (e8(sa).T, e8(s1)) if pow2 else (sa.T, s1)
         out["grouped_config5_up_gate" + tag] = dict(tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa_l), (w1, s1_l), o1, mi)),
                                                     flop=2.0 * ROUTED * H * 2 * I, padded_rows=Mp)
+        if not pow2:
+            w1fm = deep_gemm.to_fragment_major(w1)
+            out["grouped_config5_up_gate_fragment_major"] = dict(
+                tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa_l), (w1fm, s1_l), o1, mi)), flop=2.0 * ROUTED * H * 2 * I, padded_rows=Mp)
+            del w1fm
         del a, w1, o1
         a2, sa2 = qact(Mp, I, pow2)
         w2, s2 = qweights(E, H, I, pow2)
@@ -258,6 +267,11 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
         sa2_l, s2_l = (e8(sa2).T, e8(s2)) if pow2 else (sa2.T, s2)
         out["grouped_config5_down" + tag] = dict(tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a2, sa2_l), (w2, s2_l), o3, mi)),
                                                  flop=2.0 * ROUTED * I * H, padded_rows=Mp)
+        if not pow2:
+            w2fm = deep_gemm.to_fragment_major(w2)
+            out["grouped_config5_down_fragment_major"] = dict(
+                tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a2, sa2_l), (w2fm, s2_l), o3, mi)), flop=2.0 * ROUTED * I * H, padded_rows=Mp)
+            del w2fm
         del a2, w2, o3
     torch.cuda.empty_cache()
     # config 5 weight gradient dW1[e] [H, 2I] += x_e^T . do1_e, all experts in one launch
@@ -501,6 +515,69 @@ def cpu_baseline(H, I, rows=12288):
             "sample": f"{rows} token rows of one expert through quant/up+gate GEMM/SwiGLU+requant/down GEMM ({flops / 1e9:.1f} GFLOP, {dt:.1f} s)"}
 
 
+def bench_gemm_analysis(iters=40):
+    """Where the time of the config 3 up+gate launch goes (fragment-major kernel): wall time of the launch with classes
+    of instructions left out (pf8_debug_grouped_gemm_fm_cycles: the traced instantiation and its ablations), the
+    shader-clock sections of one K block from the same runs, and the launch under compute-unit budgets (what one
+    compute unit delivers when fewer of them run).  Prints nothing; returns a dict."""
+    import ctypes as C
+
+    import numpy as np
+    import torch
+
+    from paddleformers_amd import _lib, deep_gemm
+    from paddleformers_amd import functional as F8
+
+    vp = C.c_void_p
+    st = vp(torch.cuda.current_stream().cuda_stream)
+    E, H, I, ROUTED = 32, 7168, 2048, 8192
+    counts, padded = zipf_counts(ROUTED, E, 1.1, seed=3)
+    Mp = int(padded.sum())
+    mi = torch.from_numpy(np.repeat(np.arange(E, dtype=np.int32), padded)).cuda()
+    x = torch.randn((Mp, H), device="cuda").to(torch.bfloat16)
+    a, sa = F8.fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True)
+    w = torch.empty((E, 2 * I, H), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, 2 * I // 128, H // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        w[e], ws[e] = F8.fp8_quant_blockwise((torch.randn((2 * I, H), device="cuda") * 0.02).to(torch.bfloat16), quant_method="128x128")
+    wfm = deep_gemm.to_fragment_major(w)
+    o = torch.empty((Mp, 2 * I), dtype=torch.bfloat16, device="cuda")
+    cyc = torch.zeros((256, 8), dtype=torch.int64, device="cuda")
+    flop = 2.0 * ROUTED * H * 2 * I
+    out = {"workload": "config 3 up+gate grouped GEMM (32 experts, 8192 routed rows, 9984 padded)", "ablations": {}, "cu_budget": {}}
+
+    def t(fn):
+        r = time_kernel(fn, [()], iters, 10)
+        return r["ms"]
+
+    names = {0: "traced, nothing left out", 64: "every tile reads tile (0,0)'s operands (all L2 hits)", 6: "no global memory instructions",
+             8: "no scale FMAs", 14: "MFMAs and LDS fragment reads only", 30: "MFMAs, barriers and scalar code only"}
+    for ab, nm in names.items():
+        fn = lambda: _lib.call("pf8_debug_grouped_gemm_fm_cycles", vp(a.data_ptr()), vp(sa.data_ptr()), vp(wfm.data.data_ptr()), vp(ws.data_ptr()),
+                               E, Mp, 2 * I, H, vp(mi.data_ptr()), vp(o.data_ptr()), vp(cyc.data_ptr()), 256, ab, st)
+        ms = t(fn)
+        c = cyc.cpu().numpy().astype(np.float64)
+        c = c[c[:, 5] > 0]
+        per = c[:, :4].sum(0) / c[:, 5].sum()
+        out["ablations"][str(ab)] = {"what": nm, "launch_ms": round(ms, 4),
+                                     "cycles_per_block": {"mfma_0_11": round(per[0]), "wait_next_block": round(per[1]), "barrier": round(per[2]),
+                                                          "mfma_12_15": round(per[3]), "total": round(per.sum())},
+                                     "epilogue_cycles_per_tile": round(c[:, 4].sum() / c[:, 6].sum()),
+                                     "shader_clock_GHz": round(float(c[:, :5].sum(1).max()) / (ms * 1e6), 3)}
+    out["untraced_launch_ms"] = round(t(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa.T), (wfm, ws), o, mi)), 4)
+    for cus in (256, 192, 128, 64, 32):
+        deep_gemm.set_num_sms(cus)
+        try:
+            ms_fm = t(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa.T), (wfm, ws), o, mi))
+            ms_pl = t(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa.T), (w, ws), o, mi))
+        finally:
+            deep_gemm.set_num_sms(0)
+        out["cu_budget"][str(cus)] = {"fragment_major_ms": round(ms_fm, 4), "plain_ms": round(ms_pl, 4),
+                                      "fragment_major_TFLOPs_per_cu": round(flop / ms_fm / 1e9 / cus, 2),
+                                      "plain_TFLOPs_per_cu": round(flop / ms_pl / 1e9 / cus, 2)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -515,6 +592,8 @@ def main():
     ap.add_argument("--copy-yardstick", action="store_true",
                     help="also launch one plain 1 GiB copy (pf8::k_debug_copy) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings of the GEMM can be scaled by a kernel of known traffic")
+    ap.add_argument("--gemm-analysis", action="store_true",
+                    help="run only the analysis of the config 3 up+gate launch (ablations, block cycles, compute-unit budgets) and print it")
     ap.add_argument("--moe-node", choices=["fp32", "ue8m0"],
                     help="run only the config 5 MoE node leg (forward + backward, --steps/--warmup iterations) with fp32 or "
                          "UE8M0 scales and print its time: the run to profile for the node's per-kernel breakdown")
@@ -537,6 +616,9 @@ def main():
 
     if args.quant_only:
         print(json.dumps({"quant": bench_quantizers(args.leg_iters, min(10, args.leg_iters)) if args.leg_iters else bench_quantizers()}))
+        return
+    if args.gemm_analysis:
+        print(json.dumps({"gemm_analysis": bench_gemm_analysis(args.leg_iters or 40)}))
         return
     if args.gemm_legs_only:
         it = args.leg_iters or 50
@@ -576,58 +658,69 @@ def main():
         w2q[e], w2s[e] = q.view(H, I), s.view(H // 128, I // 128)
     torch.cuda.synchronize()
 
+    # the fragment-major copies of the cached FP8 weights (same bytes re-ordered, made once per weight cache like the
+    # cache itself, outside the forward): what the MoE node's forward GEMMs read
+    w1fm, w2fm = deep_gemm.to_fragment_major(w1q), deep_gemm.to_fragment_major(w2q)
+    torch.cuda.synchronize()
+
     o1 = torch.empty((Mpad, 2 * I), dtype=torch.bfloat16, device="cuda")
     o3 = torch.empty((Mpad, H), dtype=torch.bfloat16, device="cuda")
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
 
-    def step(evs=None):
+    def step(evs=None, w1=w1fm, w2=w2fm):
         if evs: evs[0].record()
         xq, xs = F8.fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True)
         if evs: evs[1].record()
-        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((xq, xs.T), (w1q, w1s), o1, m_idx)
+        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((xq, xs.T), (w1, w1s), o1, m_idx)
         if evs: evs[2].record()
         # power-of-two scales for the requantised activation, as the reference's fused node asks (transformers/fp8_utils.py:984-986)
         o2q, o2s = F8.fused_weighted_swiglu_act_quant(o1, None, using_pow2_scaling=True)
         if evs: evs[3].record()
-        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2q, w2s), o3, m_idx)
+        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2, w2s), o3, m_idx)
         if evs: evs[4].record()
+
+    def step_plain_weights():
+        """The same four launches on the plain [E, N, K] weights (the persistent kernel that stages both operands in LDS)."""
+        step(None, w1q, w2q)
 
     def step_one_launch():
         """The same forward with SwiGLU and the requantization in the up+gate GEMM's epilogue (one launch, bit-identical
         o2; the bf16 o1 is never written: what the node does when recompute_fwd_gate_up makes o1 disposable)."""
         xq, xs = F8.fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True)
         o2q, o2s = deep_gemm.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((xq, xs.T), (w1q, w1s), m_idx, None, using_pow2_scaling=True)
-        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2q, w2s), o3, m_idx)
+        deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2fm, w2s), o3, m_idx)
 
-    # First the comparison leg: the same forward with the SwiGLU quantizer in the GEMM's epilogue, timed like the
-    # headline (W warm-up steps, K timed steps).  It runs first on purpose: after idle or memory-bound work (the setup
-    # above) this GPU needs some 15 ms of matrix load before its clocks settle, and a 25-step window that starts cold
-    # reads 5-14% slow (measured: 0.64-0.69 ms against 0.60 ms for the same step); whatever leg runs first pays that.
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) * 1e3 / n
+
+    # Protocol ("warm-abba"): after idle or memory-bound work (the setup above) this GPU needs some 15 ms of matrix load
+    # before its clocks settle, and a window that starts cold reads 5-14% slow, so whatever runs first pays that.  Order:
+    #   1. the plain-weight step, W + K steps (a comparison leg; it also brings the GPU to its clocks),
+    #   2. the headline step: W untimed warm-up steps, then EXACTLY K timed steps between two synchronisations -> `value`;
+    #      no event is recorded inside them (recording one idles the stream for about 6 us, five per step would charge
+    #      the step 4-5% for its own instrumentation),
+    #   3. the plain-weight step and the fused-epilogue step again, K steps each, equally warm -> the comparison figures,
+    #   4. the headline step with an event between the kernels, K steps -> per-kernel times, and the wall time of that
+    #      loop as the figure an events-inside protocol reads for the same step.
     for _ in range(args.warmup):
-        step_one_launch()
-    torch.cuda.synchronize()
-    t2 = time.perf_counter()
-    for k in range(args.steps):
-        step_one_launch()
-    torch.cuda.synchronize()
-    ms_one_launch = (time.perf_counter() - t2) * 1e3 / args.steps
-    # W warm-up steps, then EXACTLY K timed steps between two synchronisations: `value`.  No event is
-    # recorded inside them: recording one idles the stream for about 6 us on this machine, and five per
-    # step would charge the step 4-5% for its own instrumentation.
+        step_plain_weights()
+    ms_plain_first = timed(step_plain_weights, args.steps)
     for _ in range(args.warmup):
         step()
+    ms_per_step = timed(step, args.steps)
+    ms_plain = timed(step_plain_weights, args.steps)
+    ms_one_launch = timed(step_one_launch, args.steps)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    # the same K steps once more with an event between the kernels: the per-kernel times and the
-    # duration of the roofline kernel (each carries the cost of one event record, reported below)
+    t_ev = time.perf_counter()
     for k in range(args.steps):
         step(ev[k])
     torch.cuda.synchronize()
+    ms_with_events = (time.perf_counter() - t_ev) * 1e3 / args.steps
     eo = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
     for e in eo:
         e.record()
@@ -656,6 +749,7 @@ def main():
     value = flops / (ms_per_step * 1e-3) / 1e12
     ach = flops_up / (kms["gemm_up_gate"] * 1e-3) / 1e12
     traffic, traffic_rec = traffic_from_summary(ROOFLINE_KERNEL)
+    alg_bytes = int((counts > 0).sum()) * 2 * I * H + ROUTED * H + ROUTED * 2 * I * 2
 
     res = {
         "metric": "FP8 MoE grouped-GEMM TFLOP/s + block-quant GB/s on 1 MI355X (% of peak)",
@@ -664,6 +758,9 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        # steps of this workload that ran before the timed ones: the comparison leg's W + K and the headline's own W
+        "effective_warmup_steps": 2 * args.warmup + args.steps,
+        "protocol": "warm-abba: plain-weight leg (W+K) -> headline (W untimed, K timed, no events inside) -> comparison legs (K each) -> K steps with events",
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -682,6 +779,12 @@ def main():
         "kernel_ms_min": {k: round(v, 4) for k, v in kmin.items()},
         "event_record_ms": round(event_overhead_ms, 4),
         "swiglu_in_gemm_epilogue_ms_per_step": round(ms_one_launch, 4),
+        # the same step on the plain [E, N, K] weights (both operands staged in LDS): first = run cold as leg 1, then warm
+        "plain_weight_ms_per_step": round(ms_plain, 4),
+        "plain_weight_ms_per_step_first_leg": round(ms_plain_first, 4),
+        # the headline step as a protocol with five events recorded inside every step reads it (wall time of leg 4)
+        "ms_per_step_events_inside": round(ms_with_events, 4),
+        "value_events_inside": round(flops / (ms_with_events * 1e-3) / 1e12, 2),
         "roofline": {
             "kernel": ROOFLINE_KERNEL + " (up+gate grouped GEMM)",
             "bound": "mfma",
@@ -691,15 +794,16 @@ def main():
             "frac": round(ach / FP8_PEAK_TFLOPS, 4),
             "traffic": traffic,
             "traffic_source": None if traffic_rec is None else {k: traffic_rec[k] for k in ("commit", "command") if k in traffic_rec},
-            "algorithmic_bytes": int(w1q[counts > 0].numel() + Mpad * H + Mpad * 2 * I * 2),
+            # weights of the experts that receive rows + the routed activation rows in + their bf16 outputs (padding rows are not counted)
+            "algorithmic_bytes": int(alg_bytes),
             "launch_ms": round(kms["gemm_up_gate"], 4),
             # the launch sits below the ridge of the published roofline (465 flop per algorithmic byte against 625):
             # the same launch against the 8 TB/s HBM peak, algorithmic bytes over launch time
-            "frac_hbm": round((w1q[counts > 0].numel() + Mpad * H + Mpad * 2 * I * 2) / (kms["gemm_up_gate"] * 1e-3) / 8e12, 4),
+            "frac_hbm": round(alg_bytes / (kms["gemm_up_gate"] * 1e-3) / 8e12, 4),
         },
     }
     if not args.no_quant:
-        del x, w1q, w1s, w2q, w2s, o1, o3
+        del x, w1q, w1s, w2q, w2s, w1fm, w2fm, o1, o3
         torch.cuda.empty_cache()
         res["quant"] = bench_quantizers()
         res["other_gemm"] = bench_other_gemms()
