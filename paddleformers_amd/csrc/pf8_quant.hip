@@ -375,9 +375,18 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
     __shared__ uint32_t lds_rm[128];           // row maxima
     __shared__ float4 lds_sc[256];             // (s, 1/s, -, slow) for rows 0..127, columns 128..255
     const int tid = threadIdx.x, g = tid >> 4, l = tid & 15, wave = tid >> 6, lane = tid & 63;
-    const int64_t tc = blockIdx.x, tr = blockIdx.y;
-    const int64_t row0 = tr * 128, col0 = tc * 128;
     const int64_t KB = K / 128, MB = M / 128;
+    // Consecutive workgroups go round-robin to the 8 XCDs: every XCD gets a contiguous run of tiles, walked in bands of four
+    // row tiles x all column tiles, row tile fastest.  The four workgroups that run side by side on an XCD then write four
+    // adjacent 128-byte pieces of every transposed row and four consecutive row bands of the row-scaled copy, which its L2
+    // hands to memory as longer runs than the 128-byte pieces of a plain grid (adjacent column tiles on eight different
+    // XCDs): 103 -> 95 us on [16384, 7168].
+    const int64_t nt = KB * MB, per_xcd = (nt + 7) / 8;
+    const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if ((int64_t)(blockIdx.x >> 3) >= per_xcd || logical >= nt) return;
+    const int64_t band = logical / (4 * KB), in_band = logical % (4 * KB), band_h = MB - band * 4 < 4 ? MB - band * 4 : 4;
+    const int64_t tr = band * 4 + in_band % band_h, tc = in_band / band_h;
+    const int64_t row0 = tr * 128, col0 = tc * 128;
     const bool want_rows = q != nullptr;
 
     uint4 w[8];
@@ -735,10 +744,10 @@ extern "C" int pf8_quant_transpose(const uint16_t* x, int64_t M, int64_t K, uint
     PF8_REQUIRE((q != nullptr) == (s != nullptr), "q and s come as a pair");
     PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q) && PF8_ALIGNED16(q_t) && PF8_ALIGNED16(s_t), "pointers must be 16-byte aligned");
     PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
-    PF8_REQUIRE(M / 128 <= 65535, "M too large");
+    PF8_REQUIRE((K / 128) * (M / 128) <= 0x7FFFFFF0ll, "too many tiles");
     TileSrc src = {x, nullptr, nullptr, K, M, 0};
     SplitArgs sp = {};
-    dim3 grid((unsigned)(K / 128), (unsigned)(M / 128)), block(256);
+    dim3 grid((unsigned)(((K / 128) * (M / 128) + 7) / 8 * 8)), block(256);
     if (scale_layout == 0)
         hipLaunchKernelGGL((k_quant_rowcol<false, 0>), grid, block, 0, (hipStream_t)stream, src, M, K, q, s, q_t, s_t, sp, pow2 ? 3 : 0);
     else
@@ -764,7 +773,7 @@ static int transpose_split_quant(const char* where, const void* x, const float* 
         sp.tile_start[e] = (int32_t)(total / 128);
         total += rows_per_expert[e];
     }
-    PF8_REQUIRE_AT(total / 128 <= 65535, "too many rows");
+    PF8_REQUIRE_AT(total / 128 <= 65535 && (K / 128) * (total / 128) <= 0x7FFFFFF0ll, "too many rows");
     sp.tile_start[E] = (int32_t)(total / 128);
     sp.E = E;
     if (total == 0) return PF8_OK;
@@ -779,7 +788,7 @@ static int transpose_split_quant(const char* where, const void* x, const float* 
     src.ld = K;
     src.rows = total;
     src.xs_layout = xs_layout;
-    dim3 grid((unsigned)(K / 128), (unsigned)(total / 128)), block(256);
+    dim3 grid((unsigned)(((K / 128) * (total / 128) + 7) / 8 * 8)), block(256);
     hipLaunchKernelGGL((k_quant_rowcol<true, 1>), grid, block, 0, (hipStream_t)stream, src, total, K, q, s, q_t, s_t, sp, pow2_bits);
     return pf8_check_launch(where);
 }
