@@ -327,7 +327,37 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     out["moe_permute_config5"] = dict(ms, bytes=Tt * Ht * 2 + ux.numel() * 2)
     ms = time_kernel(lambda: F8.moe_unpermute(ux, rowmap, rm_t, up, Tt, Et), [()], 20, 3)
     out["moe_unpermute_config5"] = dict(ms, bytes=Tt * tk * Ht * 2 + Tt * Ht * 2)
-    del xt, ux, rowmap, up
+    del ux, rowmap, up
+    # FP8 dispatch at config 5: the unzip as a copy of e4m3 tokens and scales, and as a row map only; then the two
+    # readers of the unzipped tokens (up+gate grouped GEMM, transposed quantizer of the weight gradient) on the copied rows
+    # and through the map
+    xq, xs = F8.fp8_quant_blockwise(xt, quant_method="1x128")
+    del xt
+    ms = time_kernel(lambda: F8.moe_permute(xq, xs, rm_t, pr_t, Et, cnts, 128), [()], 20, 3)
+    cq, _, _, cs = F8.moe_permute(xq, xs, rm_t, pr_t, Et, cnts, 128)
+    Mp5 = cq.shape[0]
+    out["unzip_fp8_config5_copy"] = dict(ms, bytes=(Tt + Mp5) * (Ht + (Ht // 128) * 4))
+    ms = time_kernel(lambda: F8.moe_permute(xq, xs, rm_t, pr_t, Et, cnts, 128, do_gather=False), [()], 20, 3)
+    gq = F8.moe_permute(xq, xs, rm_t, pr_t, Et, cnts, 128, do_gather=False)[0]
+    out["unzip_fp8_config5_map_only"] = dict(ms, bytes=Tt * tk * 8 + Tt * Et * 4 + Mp5 * 8)
+    N5 = 2 * 1408
+    wq5, ws5 = qweights(Et, N5, Ht)
+    wfm5 = deep_gemm.to_fragment_major(wq5)
+    del wq5
+    pad5 = [(c + 127) // 128 * 128 for c in cnts]
+    midx5 = torch.repeat_interleave(torch.arange(Et, dtype=torch.int32), torch.tensor(pad5)).cuda()
+    o15 = torch.empty((Mp5, N5), dtype=torch.bfloat16, device="cuda")
+    flop5 = 2.0 * Tt * tk * Ht * N5
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((cq, cs), (wfm5, ws5), o15, midx5), [()], iters, warmup)
+    out["grouped_config5_up_gate_fragment_major_copied_rows"] = dict(ms, flop=flop5)
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((gq, None), (wfm5, ws5), o15, midx5), [()], iters, warmup)
+    out["grouped_config5_up_gate_fragment_major_through_row_map"] = dict(ms, flop=flop5)
+    tsq_bytes = Mp5 * Ht * 2 + Mp5 * (Ht // 128) * 4 + (Mp5 // 128) * Ht * 4
+    ms = time_kernel(lambda: F8.fused_transpose_split_quant(cq, cs, pad5, True), [()], 20, 3)
+    out["transpose_split_quant_fp8_config5_copied_rows"] = dict(ms, bytes=tsq_bytes)
+    ms = time_kernel(lambda: F8.fused_transpose_split_quant(gq, None, pad5, True), [()], 20, 3)
+    out["transpose_split_quant_fp8_config5_through_row_map"] = dict(ms, bytes=tsq_bytes)
+    del xq, xs, cq, cs, gq, wfm5, ws5, o15, midx5
     torch.cuda.empty_cache()
     # the RMSNorm the dense FP8 MLP recomputes: forward and backward on [16384, 7168] bf16
     Mn, Hn = 16384, 7168
@@ -436,6 +466,9 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     node_flop = 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H)
     out["moe_node_config5_fwd_bwd"] = dict(bench_moe_node(False, 20, 3), flop=node_flop)
     out["moe_node_config5_fwd_bwd_ue8m0"] = dict(bench_moe_node(True, 20, 3), flop=node_flop)
+    # the layer around the node (unzip -> node -> zip and back) with FP8 dispatch, the unzip as a copy and as a row map only
+    out["moe_layer_config5_fp8_dispatch_fwd_bwd_unzip_copies"] = dict(bench_moe_layer(False, 10, 2), flop=node_flop)
+    out["moe_layer_config5_fp8_dispatch_fwd_bwd_unzip_maps"] = dict(bench_moe_layer(True, 10, 2), flop=node_flop)
     torch.cuda.empty_cache()
     return _finish(out)
 
@@ -482,6 +515,50 @@ def bench_moe_node(ue8m0, iters, warmup):
 
     ms = time_kernel(fwd_bwd, [()], iters, warmup)
     del node, exps, g1, g2, xin, dout
+    torch.cuda.empty_cache()
+    return ms
+
+
+def bench_moe_layer(fuse_unzip, iters, warmup):
+    """ms per forward + backward of FusionMlpNode (unzip -> FP8 expert MLP -> zip and back) at config 5 with FP8 dispatch:
+    16384 e4m3 tokens x top-8 over 128 experts (uniform routing), H=4096, I=1408, one grouped launch per GEMM, cached
+    stacked FP8 weights.  fuse_unzip: the unzip copies no token row (the readers go through the row map)."""
+    import types
+
+    import numpy as np
+    import torch
+
+    from paddleformers_amd import fp8_utils as U8
+    from paddleformers_amd import functional as F8
+    from paddleformers_amd.moe_layer import FusionMlpNode
+
+    E, H, I, T, topk = 128, 4096, 1408, 16384, 8
+    rng = np.random.default_rng(5)
+    rm = torch.from_numpy(np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)).cuda()
+    counts = [int((rm == e).sum().item()) for e in range(E)]
+    probs = torch.rand((T, topk), device="cuda")
+    g1 = torch.zeros((E, H, 2 * I), dtype=torch.float32, device="cuda")
+    g2 = torch.zeros((E, I, H), dtype=torch.float32, device="cuda")
+    exps = []
+    for e in range(E):
+        ex = types.SimpleNamespace(w1=(torch.randn((H, 2 * I), device="cuda") * 0.02).to(torch.bfloat16),
+                                   w2=(torch.randn((I, H), device="cuda") * 0.02).to(torch.bfloat16))
+        ex.w1.main_grad, ex.w2.main_grad = g1[e], g2[e]
+        exps.append(ex)
+    U8.fp8_quant_weight([ex.w1 for ex in exps], [ex.w2 for ex in exps], batch_mode=True)
+    cmap = types.SimpleNamespace(experts=exps, token_dispatcher=types.SimpleNamespace(_comm_manager=types.SimpleNamespace(tokens_per_expert=counts)),
+                                 config=types.SimpleNamespace(seq_length=4096, num_experts_per_tok=topk, adaptive_remained_O1_recompute_ratio=1.0))
+    tokens = F8.fp8_quant_blockwise(torch.randn((T, H), device="cuda").to(torch.bfloat16), quant_method="1x128")
+    dy = (torch.randn((T, H), device="cuda") * 1e-3).to(torch.bfloat16)
+
+    def fwd_bwd():
+        layer = FusionMlpNode(cmap, topk, is_split_group_gemm=False)
+        layer.fuse_unzip = fuse_unzip
+        layer.forward(tokens, rm, probs)
+        layer.backward(dy)
+
+    ms = time_kernel(fwd_bwd, [()], iters, warmup)
+    del exps, g1, g2, tokens, dy
     torch.cuda.empty_cache()
     return ms
 

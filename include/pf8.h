@@ -102,6 +102,14 @@ int pf8_transpose_split_quant(const void* x, const float* xs, int x_is_fp8, int 
                               const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q_t, float* s_t,
                               int pow2, pf8_stream_t stream);
 
+/* pf8_transpose_split_quant of an e4m3 input with UnZipNode.forward's row copy folded into the read: row r of the
+ * expert-sorted input is row src_row[r] of tokens [T, K] with that row's scales (xs_layout 0 = [T, K/128], 1 = [K/128, T]);
+ * src_row[r] < 0 is a row of zeros.  src_row int32 [sum rows_per_expert], entries below T.  Outputs bit-identical to
+ * pf8_transpose_split_quant on the rows pf8_moe_permute copies out. */
+int pf8_transpose_split_quant_gather(const uint8_t* tokens, const float* token_scales, int xs_layout, int64_t T,
+                                     const int32_t* src_row, const int64_t* rows_per_expert, int E, int64_t K,
+                                     uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream);
+
 /* The two quantizations the MoE node's backward applies to the SAME bf16 gradient, from one read:
  * fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True, using_pow2_scale=pow2_rows)
  * for the dgrad GEMM and fused_transpose_split_quant(x, None, tokens_per_expert, pow2_t) for the wgrad
@@ -147,6 +155,16 @@ int pf8_moe_permute(const void* x, int x_is_fp8, const float* xs, const int32_t*
                     const int64_t* tokens_per_expert, int padding_alignment, void* out_x,
                     int32_t* rowmap, float* out_probs, float* out_xs, int32_t* overflow,
                     pf8_stream_t stream);
+
+/* The same reordering as pf8_moe_permute with no row copied: src_row int32 [Mpad] receives, for every row of the
+ * expert-sorted padded layout, the index of the token that pf8_moe_permute would have copied there (-1 for a padding row
+ * and for the rows left over when an expert receives fewer tokens than its count says); rowmap, out_probs and *overflow
+ * are what pf8_moe_permute writes.  The consumers that take (tokens, src_row) in place of the copied rows
+ * (pf8_grouped_gemm_nt_contiguous_fm_gather, pf8_transpose_split_quant_gather) read a -1 row as zeros, which is what
+ * the copy holds there; UnZipNode.forward's token copy (moe_utils.py:141-186) then never exists in memory. */
+int pf8_moe_permute_map(const int32_t* routemap, const float* probs, int64_t T, int topk, int E,
+                        const int64_t* tokens_per_expert, int padding_alignment, int32_t* rowmap,
+                        int32_t* src_row, float* out_probs, int32_t* overflow, pf8_stream_t stream);
 
 /* paddle.nn.functional.moe_unpermute(hidden_states_unzipped, zipped_expertwise_rowmap,
  * expert_routemap_topk, token_prob_unzipped, total_zipped_tokens, num_experts) as ZipNode.forward /
@@ -226,6 +244,16 @@ int pf8_gemm_nt_fm(const uint8_t* a, const float* sa, int sa_layout, const uint8
 int pf8_grouped_gemm_nt_contiguous_fm(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b_fm,
                                       const float* sb, int E, int64_t Mtot, int64_t N, int64_t K,
                                       const int32_t* m_indices, uint16_t* out, pf8_stream_t stream);
+
+/* pf8_grouped_gemm_nt_contiguous_fm with UnZipNode.forward's row copy (moe_utils.py:141-186) folded into the read of the
+ * activation operand: row r of the expert-sorted operand is row src_row[r] of tokens [T, K] (e4m3) with the scales of that
+ * row of token_scales [T, K/128] (fp32, row-major); src_row[r] < 0 (see pf8_moe_permute_map) is a row of zeros.  out is
+ * bit-identical to pf8_grouped_gemm_nt_contiguous_fm on the rows pf8_moe_permute copies out.  src_row: int32 [Mtot],
+ * 16-byte aligned, every entry below T; tokens below 2 GiB. */
+int pf8_grouped_gemm_nt_contiguous_fm_gather(const uint8_t* tokens, const float* token_scales, int64_t T,
+                                             const int32_t* src_row, const uint8_t* b_fm, const float* sb, int E,
+                                             int64_t Mtot, int64_t N, int64_t K, const int32_t* m_indices,
+                                             uint16_t* out, pf8_stream_t stream);
 
 /* The up+gate grouped GEMM with the activation quantizer of the down projection in its epilogue: the two calls of
  * FP8GroupGemmMlpFunctionNode.forward -- deep_gemm.m_grouped_fp8_gemm_nt_contiguous (transformers/fp8_utils.py:949-954)

@@ -81,7 +81,8 @@ __global__ __launch_bounds__(1024) void k_permute_rowmap(const int32_t* __restri
         if (tid == 0) atomicOr(overflow, 2);
         for (int64_t r = base; r < limit; ++r) {
             uint4* dst = reinterpret_cast<uint4*>(out_x + r * row_bytes);
-            for (int64_t i = tid; i < row_bytes / 16; i += 1024) st16(dst + i, make_uint4(0, 0, 0, 0));
+            if (out_x)
+                for (int64_t i = tid; i < row_bytes / 16; i += 1024) st16(dst + i, make_uint4(0, 0, 0, 0));
             if (out_xs)
                 for (int64_t i = tid; i < scale_cols; i += 1024) out_xs[r * scale_cols + i] = 0.0f;
             if (out_probs && tid == 0) out_probs[r] = 0.0f;
@@ -134,6 +135,27 @@ __global__ __launch_bounds__(256) void k_permute_gather(const uint8_t* __restric
             for (int64_t c = tid; c < scale_cols; c += 256) out_xs[r * scale_cols + c] = xs[t * scale_cols + c];
         if (out_probs && tid == 0) out_probs[r] = probs ? probs[t * topk + k] : 0.0f;
     }
+}
+
+// The map-only form of the gather: one thread per routing slot writes the slot's token index (and probability) at the
+// slot's row; rows no slot claims keep the -1 the fill kernel wrote.
+__global__ __launch_bounds__(256) void k_fill_i32(int32_t* __restrict__ p, int64_t n, int32_t v) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+__global__ __launch_bounds__(256) void k_permute_source_rows(const int32_t* __restrict__ routemap, const float* __restrict__ probs,
+                                                             const int32_t* __restrict__ rowmap, int64_t T, int topk, int E,
+                                                             int32_t* __restrict__ src_row, float* __restrict__ out_probs) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= T * topk) return;
+    const int64_t t = i / topk;
+    const int e = routemap[i];
+    if (e < 0 || e >= E) return;
+    const int64_t r = rowmap[t * E + e];
+    if (r < 0) return;
+    src_row[r] = (int32_t)t;
+    if (out_probs) out_probs[r] = probs ? probs[i] : 0.0f;
 }
 
 // One workgroup per token: fp32 sum of its routed copies in slot order, bf16 out; probabilities back
@@ -233,6 +255,45 @@ extern "C" int pf8_moe_permute(const void* x, int x_is_fp8, const float* xs, con
         rc = pf8_check_launch(__func__);
     }
     return rc;
+}
+
+extern "C" int pf8_moe_permute_map(const int32_t* routemap, const float* probs, int64_t T, int topk, int E, const int64_t* tokens_per_expert,
+                                   int padding_alignment, int32_t* rowmap, int32_t* src_row, float* out_probs, int32_t* overflow,
+                                   pf8_stream_t stream) {
+    PF8_REQUIRE(T >= 0 && topk > 0 && E > 0, "bad shape");
+    PF8_REQUIRE(E <= 256, "at most 256 experts");
+    PF8_REQUIRE(padding_alignment > 0, "padding_alignment must be positive");
+    PF8_REQUIRE(tokens_per_expert, "tokens_per_expert is a host array of E counts");
+    PermuteArgs pa = {};
+    pa.E = E;
+    int64_t total = 0;
+    for (int e = 0; e < E; ++e) {
+        PF8_REQUIRE(tokens_per_expert[e] >= 0 && tokens_per_expert[e] <= 0x7FFFFFFF, "bad tokens_per_expert");
+        pa.row_start[e] = total;
+        pa.count[e] = (int32_t)tokens_per_expert[e];
+        total += (tokens_per_expert[e] + padding_alignment - 1) / padding_alignment * padding_alignment;
+    }
+    pa.row_start[E] = total;
+    PF8_REQUIRE(total <= 0x7FFFFFFF && T <= 0x7FFFFFFF && T * topk <= 0x7FFFFFFFll * 256, "too many rows");
+    if (total == 0 && T == 0) return PF8_OK;
+    PF8_REQUIRE(rowmap && overflow && (total == 0 || src_row), "null pointer");
+    PF8_REQUIRE(T == 0 || routemap, "null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (total > 0) {
+        hipLaunchKernelGGL(k_fill_i32, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, src_row, total, -1);
+        int rc = pf8_check_launch(__func__);
+        if (rc) return rc;
+    }
+    const bool rm16 = (reinterpret_cast<uintptr_t>(routemap) & 15u) == 0;
+    // no token rows to clear: the rows of an expert whose count overstates its routed tokens keep source -1 (read as zeros)
+    if (topk == 8 && rm16) hipLaunchKernelGGL(k_permute_rowmap<8>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow, (uint8_t*)nullptr, (int64_t)0, (float*)nullptr, (int64_t)0);
+    else if (topk == 4 && rm16) hipLaunchKernelGGL(k_permute_rowmap<4>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow, (uint8_t*)nullptr, (int64_t)0, (float*)nullptr, (int64_t)0);
+    else hipLaunchKernelGGL(k_permute_rowmap<0>, dim3(E), dim3(1024), 0, st, routemap, T, topk, pa, rowmap, out_probs, overflow, (uint8_t*)nullptr, (int64_t)0, (float*)nullptr, (int64_t)0);
+    int rc = pf8_check_launch(__func__);
+    if (rc || T == 0) return rc;
+    hipLaunchKernelGGL(k_permute_source_rows, dim3((unsigned)((T * topk + 255) / 256)), dim3(256), 0, st, routemap, probs, rowmap, T, topk, E,
+                       src_row, out_probs);
+    return pf8_check_launch(__func__);
 }
 
 extern "C" int pf8_moe_unpermute(const uint16_t* unzipped, const int32_t* rowmap, const int32_t* routemap, const float* probs_unzipped,

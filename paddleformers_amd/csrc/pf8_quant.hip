@@ -227,6 +227,7 @@ struct TileSrc {
     int64_t ld;            // row stride in elements
     int64_t rows;          // total rows (for xs_layout 1)
     int xs_layout;
+    const int32_t* src_row;   // e4m3 source only: row r of the tile grid is row src_row[r] of xq / xs (negative = a row of zeros); null = r
 };
 
 // load this thread's 8x8 patch as fp32 values; amax bit patterns per row chunk go to rmax[i]
@@ -287,7 +288,7 @@ __global__ __launch_bounds__(256) void k_quant_128x128(const uint16_t* __restric
     const int64_t tc = blockIdx.x, tr = blockIdx.y, e = blockIdx.z;
     TileSrc src;
     src.x = STACK ? ptrs.w[e] : w;
-    src.xq = nullptr; src.xs = nullptr; src.ld = C; src.rows = R; src.xs_layout = 0;
+    src.xq = nullptr; src.xs = nullptr; src.ld = C; src.rows = R; src.xs_layout = 0; src.src_row = nullptr;
     const int64_t row0 = tr * 128, col0 = tc * 128;
     float v[8][8];
     load_patch(src, row0, col0, g, l, v);
@@ -343,7 +344,13 @@ __device__ __forceinline__ void load_patch_packed(const TileSrc& src, int64_t ro
         const int64_t KB = src.ld / 128;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const int64_t r = row0 + 8 * g + i;
+            int64_t r = row0 + 8 * g + i;
+            if (src.src_row) r = src.src_row[r];
+            if (r < 0) {                // a zero byte times a zero scale, as the copied padding row holds them
+                q[i] = make_uint2(0, 0);
+                sc[i] = 0.0f;
+                continue;
+            }
             q[i] = ld8(src.xq + r * src.ld + col0 + 8 * l);
             sc[i] = src.xs_layout == 0 ? src.xs[r * KB + col0 / 128] : src.xs[(col0 / 128) * src.rows + r];
         }
@@ -745,7 +752,7 @@ extern "C" int pf8_quant_transpose(const uint16_t* x, int64_t M, int64_t K, uint
     PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q) && PF8_ALIGNED16(q_t) && PF8_ALIGNED16(s_t), "pointers must be 16-byte aligned");
     PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
     PF8_REQUIRE((K / 128) * (M / 128) <= 0x7FFFFFF0ll, "too many tiles");
-    TileSrc src = {x, nullptr, nullptr, K, M, 0};
+    TileSrc src = {x, nullptr, nullptr, K, M, 0, nullptr};
     SplitArgs sp = {};
     dim3 grid((unsigned)(((K / 128) * (M / 128) + 7) / 8 * 8)), block(256);
     if (scale_layout == 0)
@@ -758,7 +765,7 @@ extern "C" int pf8_quant_transpose(const uint16_t* x, int64_t M, int64_t K, uint
 // shared by pf8_transpose_split_quant and pf8_quant_and_transpose_split: q/s null = no row-scaled copy
 static int transpose_split_quant(const char* where, const void* x, const float* xs, int x_is_fp8, int xs_layout,
                                  const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
-                                 int pow2_bits, pf8_stream_t stream) {
+                                 int pow2_bits, pf8_stream_t stream, const int32_t* src_row = nullptr, int64_t src_rows = 0) {
 #define PF8_REQUIRE_AT(cond, msg) do { if (!(cond)) return pf8_fail(PF8_EINVAL, where, msg); } while (0)
     PF8_REQUIRE_AT(xs_layout == 0 || xs_layout == 1, "xs_layout must be 0 or 1");
     PF8_REQUIRE_AT(E >= 0 && K >= 0, "negative shape");
@@ -786,8 +793,9 @@ static int transpose_split_quant(const char* where, const void* x, const float* 
     src.xq = x_is_fp8 ? (const uint8_t*)x : nullptr;
     src.xs = xs;
     src.ld = K;
-    src.rows = total;
+    src.rows = src_row ? src_rows : total;
     src.xs_layout = xs_layout;
+    src.src_row = src_row;
     dim3 grid((unsigned)(((K / 128) * (total / 128) + 7) / 8 * 8)), block(256);
     hipLaunchKernelGGL((k_quant_rowcol<true, 1>), grid, block, 0, (hipStream_t)stream, src, total, K, q, s, q_t, s_t, sp, pow2_bits);
     return pf8_check_launch(where);
@@ -796,6 +804,15 @@ static int transpose_split_quant(const char* where, const void* x, const float* 
 extern "C" int pf8_transpose_split_quant(const void* x, const float* xs, int x_is_fp8, int xs_layout, const int64_t* rows_per_expert,
                                          int E, int64_t K, uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream) {
     return transpose_split_quant(__func__, x, xs, x_is_fp8, xs_layout, rows_per_expert, E, K, nullptr, nullptr, q_t, s_t, pow2 ? 1 : 0, stream);
+}
+
+extern "C" int pf8_transpose_split_quant_gather(const uint8_t* tokens, const float* token_scales, int xs_layout, int64_t T,
+                                                const int32_t* src_row, const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q_t,
+                                                float* s_t, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(T > 0, "the token matrix is empty");
+    PF8_REQUIRE(src_row, "null pointer");
+    return transpose_split_quant(__func__, tokens, token_scales, 1, xs_layout, rows_per_expert, E, K, nullptr, nullptr, q_t, s_t, pow2 ? 1 : 0,
+                                 stream, src_row, T);
 }
 
 extern "C" int pf8_quant_and_transpose_split(const uint16_t* x, const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q, float* s,

@@ -13,7 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from .functional import FP8, _dev, _p, _scale_layout_of, _stream
+from .functional import FP8, GatheredRows, _dev, _p, _scale_layout_of, _stream
 
 
 def set_num_sms(num: int) -> None:
@@ -60,10 +60,16 @@ def to_fragment_major(w: torch.Tensor) -> FragmentMajor:
     return FragmentMajor(out, w.shape)
 
 
-def _check_pair(pair, what) -> Tuple[torch.Tensor, torch.Tensor]:
+def _check_pair(pair, what, gathered_ok=False) -> Tuple[torch.Tensor, torch.Tensor]:
     if not (isinstance(pair, (tuple, list)) and len(pair) == 2):
         raise ValueError(f"{what} must be a (tensor, scale) pair")
     t, s = pair
+    if isinstance(t, GatheredRows):
+        if not gathered_ok:
+            raise ValueError(f"{what}: gathered rows are read by m_grouped_fp8_gemm_nt_contiguous only (materialize() them)")
+        if s is not None:
+            raise ValueError(f"{what}: gathered rows carry their own scales (pass None)")
+        return t, None
     if isinstance(t, FragmentMajor):
         _dev(t.data, what)
         _dev(s, what + " scale")
@@ -202,9 +208,11 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
 
     transformers/fp8_utils.py:949-954: a [Mtot, K] + sa [Mtot, K/128] (any strides), b [E, N, K] +
     sb [E, N/128, K/128], m_indices int32 [Mtot]; every expert segment is a multiple of 128 rows.
+    a may be `(GatheredRows, None)` with a fragment-major b: the rows are then read from the tokens through the source
+    map, with the result the copied rows would give, to the bit.
     `items` (optional, UE8M0 scales only): the list build_group_items made for this m_indices.
     """
-    (ta, sa), (tb, sb) = _check_pair(a, "a"), _check_pair(b, "b")
+    (ta, sa), (tb, sb) = _check_pair(a, "a", gathered_ok=True), _check_pair(b, "b")
     _dev(out, "out")
     _dev(m_indices, "m_indices")
     Mtot, K = ta.shape
@@ -221,8 +229,19 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
         raise ValueError("m_indices must be int32 with one entry per row")
     if Mtot == 0 or N == 0:
         return out
-    ta = ta if ta.is_contiguous() else ta.contiguous()
+    ta = ta.contiguous()
     m_indices = m_indices if m_indices.is_contiguous() else m_indices.contiguous()
+    if isinstance(ta, GatheredRows):
+        if not isinstance(tb, FragmentMajor) or _is_ue8m0(sb) or not fragment_major_supported(Mtot, N, K):
+            raise ValueError("gathered rows go with a fragment-major weight and fp32 scales (materialize() them for the other kernels)")
+        if tuple(sb.shape) != (E, N // 128, K // 128) or sb.dtype != torch.float32:
+            raise ValueError(f"b scale must be float32 [{E}, {N // 128}, {K // 128}]")
+        T = ta.tokens.shape[0]
+        if T == 0 or T * K >= 2 ** 31 or ta.src_row.data_ptr() % 16:
+            raise ValueError("gathered rows: the token matrix must be non-empty and below 2 GiB, the source map 16-byte aligned")
+        _lib.call("pf8_grouped_gemm_nt_contiguous_fm_gather", _p(ta.tokens), _p(ta.scale), T, _p(ta.src_row), _p(tb.data), _p(sb.contiguous()),
+                  E, Mtot, N, K, _p(m_indices), _p(out), _stream())
+        return out
     if isinstance(tb, FragmentMajor):
         if _is_ue8m0(sa) or _is_ue8m0(sb) or not fragment_major_supported(Mtot, N, K):
             raise ValueError("a fragment-major weight serves fp32 scales, Mtot % 128 == 0, N % 256 == 0, K % 128 == 0, K >= 384")

@@ -684,6 +684,14 @@ class FP8GroupGemmMlpFunctionNode:
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a_fp8, F8.scales_to_ue8m0(a_scale, check=False)), (w_fp8, w_bytes), out, m_indices,
                                                    items=items)
 
+    def _reads_gathered(self, g, w_fp8, cache):
+        """Whether the up+gate grouped GEMM can read these gathered rows through their source map (the fragment-major
+        kernel, fp32 scales, one grouped launch); otherwise the rows are copied out first."""
+        T, K = g.tokens.shape
+        return (not self.use_ue8m0 and not self.is_split_group_gemm and cache is not None and self.use_fragment_major
+                and 0 < T and T * K < 2 ** 31 and g.src_row.data_ptr() % 16 == 0
+                and deep_gemm.fragment_major_supported(g.shape[0], w_fp8.shape[1], w_fp8.shape[2]))
+
     def _stacked(self, expert_w, transpose, num_expert):
         """(e4m3 [E, N, K], scales [E, N/128, K/128], cache): the stacked quantized weights in the orientation asked for;
         cache = (weight object, attribute name) when they are the per-step cache itself (then tensors derived from
@@ -704,9 +712,17 @@ class FP8GroupGemmMlpFunctionNode:
         if not self.is_split_group_gemm and self.m_indices is None:
             self.m_indices = self.gen_m_indices(tokens_per_expert)
         w1_t_quant, w1_t_scale, w1_cache = self._stacked(expert_w1, True, num_expert)
+        if isinstance(x, tuple) and isinstance(x[0], F8.GatheredRows):
+            x = x[0]
+        if x is None and isinstance(self.input_fp8, F8.GatheredRows):
+            x = self.input_fp8
+        if isinstance(x, F8.GatheredRows) and not self._reads_gathered(x, w1_t_quant, w1_cache):
+            x = x.materialize()
         if x is None:
             x_fp8, x_scale = self.input_fp8, self.input_scale
-            assert x_fp8 is not None and x_scale is not None
+            assert x_fp8 is not None and (x_scale is not None or isinstance(x_fp8, F8.GatheredRows))
+        elif isinstance(x, F8.GatheredRows):
+            x_fp8, x_scale = x.contiguous(), None           # rows that were never copied: read through their source map
         elif isinstance(x, tuple):
             x_fp8, x_scale = x
             x_scale = x_scale.t().contiguous().t()
@@ -871,8 +887,8 @@ class FP8GroupGemmMlpFunctionNode:
 
     @torch.no_grad()
     def forward(self, hs_out, unzipped_probs, tokens_per_expert, m_indices=None):
-        """fp8_utils.py:1191-1232.  hs_out: bf16 [m_sum, H], a (fp8, scale) pair, or None to reuse
-        the cached quantised input.  Zero rows -> zeros."""
+        """fp8_utils.py:1191-1232.  hs_out: bf16 [m_sum, H], a (fp8, scale) pair, the `GatheredRows` of
+        moe_permute(..., do_gather=False), or None to reuse the cached quantised input.  Zero rows -> zeros."""
         if self.fwd_subbatch:
             assert m_indices is not None
         dtype = torch.bfloat16
@@ -891,7 +907,8 @@ class FP8GroupGemmMlpFunctionNode:
         num_expert = len(expert_w1)
         in_scale = hs_out[1] if isinstance(hs_out, tuple) else (self.input_scale if hs_out is None else None)
         fuse = self.recompute_fwd_gate_up if self.fuse_swiglu_epilogue is None else self.fuse_swiglu_epilogue
-        if (fuse and not self.is_split_group_gemm and not self.use_ue8m0
+        gathered = isinstance(self.input_fp8 if hs_out is None else hs_out, F8.GatheredRows)     # read through the row map instead
+        if (fuse and not gathered and not self.is_split_group_gemm and not self.use_ue8m0
                 and (in_scale is None or in_scale.dtype == torch.float32)
                 and deep_gemm.swiglu_quant_fusable(shape[0], expert_w1[0].shape[1], shape[1])):
             return self._forward_fused(hs_out, unzipped_probs, expert_w1, expert_w2, num_expert, tokens_per_expert, m_indices)
@@ -910,6 +927,10 @@ class FP8GroupGemmMlpFunctionNode:
         if self.m_indices is None:
             self.m_indices = self.gen_m_indices(tokens_per_expert)
         w1_t_quant, w1_t_scale, w1_cache = self._stacked(expert_w1, True, num_expert)
+        if x is None and isinstance(self.input_fp8, F8.GatheredRows):
+            x = self.input_fp8
+        if isinstance(x, F8.GatheredRows):
+            x = x.materialize()                 # the kernel with the SwiGLU epilogue reads plain rows
         if x is None:
             x_fp8, x_scale = self.input_fp8, self.input_scale
             assert x_fp8 is not None and x_scale is not None
@@ -941,7 +962,8 @@ class FP8GroupGemmMlpFunctionNode:
         """fp8_utils.py:1234-1321.  Returns (dx, probs_grad); weight gradients are accumulated
         into each expert weight's main_grad (or grad)."""
         if self.bwd_subbatch:
-            assert m_indices is not None and input_fp8_slice is not None and input_scale_slice is not None and tokens_per_expert is not None
+            assert m_indices is not None and input_fp8_slice is not None and tokens_per_expert is not None
+            assert input_scale_slice is not None or isinstance(input_fp8_slice, F8.GatheredRows)
         dtype = torch.bfloat16
         g0 = extract_first_if_tuple(out_grad)
         if g0.shape[0] == 0:

@@ -37,6 +37,55 @@ def _as2d(x: torch.Tensor) -> torch.Tensor:
     return x.reshape(-1, x.shape[-1])
 
 
+class GatheredRows:
+    """The expert-sorted, padded rows `moe_permute` would write, not copied: row r is row src_row[r] of `tokens`
+    (float8_e4m3fn [T, H]) with that row of `scale` (fp32 [T, H/128]); src_row[r] < 0 is a row of zeros.
+    What `moe_permute(..., do_gather=False)` returns in place of the copied rows; `m_grouped_fp8_gemm_nt_contiguous` (on a
+    fragment-major weight) and `fused_transpose_split_quant` take it where they take the copied rows and read the tokens
+    through the map, with bit-identical results.  A slice `g[a:b]` is the same tokens behind a slice of the map."""
+
+    __slots__ = ("tokens", "scale", "src_row")
+
+    def __init__(self, tokens: torch.Tensor, scale: torch.Tensor, src_row: torch.Tensor):
+        if tokens.dtype != FP8 or tokens.dim() != 2 or not tokens.is_contiguous():
+            raise ValueError("tokens must be a contiguous float8_e4m3fn [T, H] tensor")
+        if scale.dtype != torch.float32 or tuple(scale.shape) != (tokens.shape[0], tokens.shape[1] // 128) or not scale.is_contiguous():
+            raise ValueError("scale must be a contiguous float32 [T, H/128] tensor")
+        if src_row.dtype != torch.int32 or src_row.dim() != 1:
+            raise ValueError("src_row must be int32 [rows]")
+        self.tokens, self.scale, self.src_row = tokens, scale, src_row
+
+    @property
+    def shape(self):
+        return torch.Size((self.src_row.shape[0], self.tokens.shape[1]))
+
+    @property
+    def device(self):
+        return self.tokens.device
+
+    @property
+    def dtype(self):
+        return self.tokens.dtype
+
+    def dim(self) -> int:
+        return 2
+
+    def __getitem__(self, sl):
+        if not isinstance(sl, slice) or sl.step not in (None, 1):
+            raise TypeError("only contiguous row slices of gathered rows can be taken")
+        return GatheredRows(self.tokens, self.scale, self.src_row[sl])
+
+    def contiguous(self):
+        return self if self.src_row.is_contiguous() else GatheredRows(self.tokens, self.scale, self.src_row.contiguous())
+
+    def materialize(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(rows e4m3 [rows, H], scales fp32 [rows, H/128]): the copy, for a consumer that cannot read through the map."""
+        live = self.src_row >= 0
+        idx = self.src_row.clamp(min=0).long()
+        rows = self.tokens.view(torch.uint8)[idx] * live[:, None].to(torch.uint8)
+        return rows.view(FP8), self.scale[idx] * live[:, None].to(torch.float32)
+
+
 def _scale_layout_of(s: torch.Tensor, rows: int, blocks: int, what: str) -> Tuple[torch.Tensor, int]:
     """A logical [rows, blocks] scale tensor -> (tensor, layout flag) without copying when its
     memory is either row-major (0) or blocks-major, i.e. a transposed view of [blocks, rows] (1)."""
@@ -240,12 +289,17 @@ def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], 
     Returns lists with one q_t [K, M_e] and one s_t [M_e/128, K] per expert (empty tensors for
     experts without rows).
     """
+    gathered = x if isinstance(x, GatheredRows) else None
+    if gathered is not None:
+        if scale is not None:
+            raise ValueError("gathered rows carry their own scales")
+        x = gathered.tokens
     _dev(x, "x")
     if x.dim() != 2:
         raise ValueError("x must be 2-D")
     if not x.is_contiguous():
         x = x.contiguous()
-    Mtot, K = x.shape
+    Mtot, K = x.shape if gathered is None else gathered.shape
     rows = [int(t) for t in tokens_per_expert]
     if sum(rows) != Mtot:
         raise ValueError(f"tokens_per_expert sums to {sum(rows)} but x has {Mtot} rows")
@@ -253,6 +307,8 @@ def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], 
         raise ValueError("every tokens_per_expert entry must be a non-negative multiple of 128")
     if K % 128 != 0:
         raise ValueError(f"last dimension must be divisible by 128, got {K}")
+    if gathered is not None:
+        return _transpose_split_quant_gathered(gathered, rows, pow_2_scales)
     is_fp8 = x.dtype == FP8
     xs_layout = 0
     if is_fp8:
@@ -282,6 +338,31 @@ def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], 
         qp = C.c_void_p(q_t.data_ptr() + off * K)
         sp = C.c_void_p(s_t.data_ptr() + (off // 128) * K * 4)
         _lib.call("pf8_transpose_split_quant", xp, xs_ptr, int(is_fp8), lay, arr, len(chunk), K, qp, sp, int(bool(pow_2_scales)), _stream())
+    qs, ss, off = [], [], 0
+    for r in rows:
+        qs.append(q_t[off * K:(off + r) * K].view(K, r))
+        ss.append(s_t[(off // 128) * K:((off + r) // 128) * K].view(r // 128, K))
+        off += r
+    return qs, ss
+
+
+def _transpose_split_quant_gathered(g: GatheredRows, rows: List[int], pow_2_scales: bool):
+    """fused_transpose_split_quant of rows that are read through their source map (rows already checked)."""
+    Mtot, K = g.shape
+    T = g.tokens.shape[0]
+    if T == 0 and Mtot:
+        raise ValueError("gathered rows need a non-empty token matrix")
+    src = g.src_row if g.src_row.is_contiguous() else g.src_row.contiguous()
+    q_t = torch.empty((K * Mtot,), dtype=FP8, device=g.device)
+    s_t = torch.empty(((Mtot // 128) * K,), dtype=torch.float32, device=g.device)
+    for e0 in range(0, len(rows), 256):
+        chunk = rows[e0:e0 + 256]
+        off = sum(rows[:e0])
+        if sum(chunk) == 0:
+            continue
+        arr = (C.c_int64 * len(chunk))(*chunk)
+        _lib.call("pf8_transpose_split_quant_gather", _p(g.tokens), _p(g.scale), 0, T, C.c_void_p(src.data_ptr() + off * 4), arr, len(chunk), K,
+                  C.c_void_p(q_t.data_ptr() + off * K), C.c_void_p(s_t.data_ptr() + (off // 128) * K * 4), int(bool(pow_2_scales)), _stream())
     qs, ss, off = [], [], 0
     for r in rows:
         qs.append(q_t[off * K:(off + r) * K].view(K, r))
@@ -614,14 +695,14 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
     expert_routemap_topk int32 [T, topk] (negative = unused slot); expert_prob_topk fp32 [T, topk].
     Returns (hidden_states_unzipped [Mpad, H], zipped_expertwise_rowmap int32 [T, num_experts],
     token_prob_unzipped fp32 [Mpad, 1], scale_unzipped fp32 [Mpad, H/128] or None).
+    do_gather=False (float8 hidden_states only) copies no row: the first result is a `GatheredRows` (the tokens, their
+    scales and the source token of every output row), the last is None.
     Counts that do not match the routing (a token routed to an expert beyond its `tokens_per_expert` count is
     dropped; rows of an overstated count are written as zeros) set a sticky flag word that lives on the device for
     the life of the process: the call itself neither allocates nor reads it back, as the reference's operator has no
     device-to-host round trip either.  `moe_permute_check()` reads and clears the flag wherever the caller
     synchronises anyway; `validate=True` does so right after this call (one synchronisation) and raises ValueError.
     """
-    if not do_gather:
-        raise ValueError("do_gather=False is not supported")
     _dev(hidden_states, "hidden_states")
     _dev(expert_routemap_topk, "expert_routemap_topk")
     if hidden_states.dim() != 2 or expert_routemap_topk.dim() != 2 or expert_routemap_topk.shape[0] != hidden_states.shape[0]:
@@ -642,7 +723,6 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
     rm = expert_routemap_topk.to(torch.int32).contiguous()
     pr = None if expert_prob_topk is None else expert_prob_topk.to(torch.float32).contiguous()
     dev = x.device
-    out_x = torch.empty((mpad, H), dtype=hidden_states.dtype, device=dev)
     rowmap = torch.empty((T, num_experts), dtype=torch.int32, device=dev)
     out_p = torch.empty((mpad, 1), dtype=torch.float32, device=dev)
     out_s = None
@@ -651,9 +731,20 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
         if tuple(scale.shape) != (T, H // 128) or scale.dtype != torch.float32:
             raise ValueError("scale must be float32 [T, H/128]")
         xs = scale.contiguous()
-        out_s = torch.empty((mpad, H // 128), dtype=torch.float32, device=dev)
     overflow = _permute_flag(dev)
     cnt = (C.c_int64 * num_experts)(*counts)
+    if not do_gather:
+        if not is_fp8:
+            raise ValueError("do_gather=False serves float8 hidden_states (the consumers of gathered rows read e4m3 tokens)")
+        src_row = torch.empty((mpad,), dtype=torch.int32, device=dev)
+        _lib.call("pf8_moe_permute_map", _p(rm), _p(pr), T, topk, num_experts, cnt, a, _p(rowmap), _p(src_row), _p(out_p), _p(overflow),
+                  _stream())
+        if validate:
+            moe_permute_check(dev)
+        return GatheredRows(x, xs, src_row), rowmap, out_p, None
+    out_x = torch.empty((mpad, H), dtype=hidden_states.dtype, device=dev)
+    if is_fp8:
+        out_s = torch.empty((mpad, H // 128), dtype=torch.float32, device=dev)
     _lib.call("pf8_moe_permute", _p(x), int(is_fp8), _p(xs), _p(rm), _p(pr), T, H, topk, num_experts, cnt, a, _p(out_x), _p(rowmap),
               _p(out_p), _p(out_s), _p(overflow), _stream())
     if validate:

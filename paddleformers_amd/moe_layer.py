@@ -25,6 +25,7 @@ from typing import Optional, Tuple, Union
 
 import torch
 
+from . import functional as F8
 from .fp8_utils import FP8GroupGemmMlpFunctionNode, extract_first_if_tuple
 from .moe_utils import UnZipNode, ZipNode
 
@@ -67,6 +68,10 @@ class FusionMlpNode:
         self.output_subbatch_rows = output_subbatch_rows     # granularity of the reference's fp32 zip; unused here (see module text)
         self.unzipped_probs = None
         self.m_indices = None
+        # with FP8 dispatch and one grouped launch per GEMM (is_split_group_gemm=False) the unzip copies no token row: the
+        # up+gate GEMM and the transposed quantizer of the weight gradient read the dispatched tokens through the row map
+        # (same results to the bit; the expert-sorted copy of the tokens and of their scales never exists).  False = copy.
+        self.fuse_unzip = True
 
     def set_recompute_fwd_gate_up(self, recompute_fwd_gate_up):
         self.experts_group_gemm_node.recompute_fwd_gate_up = recompute_fwd_gate_up
@@ -88,7 +93,7 @@ class FusionMlpNode:
     def prepare_env_subbatch(self, unzipped_tokens=None, unzipped_tokens_scale=None, is_fwd=True):
         node = self.experts_group_gemm_node
         if is_fwd:
-            assert unzipped_tokens is not None and unzipped_tokens_scale is not None
+            assert unzipped_tokens is not None and (unzipped_tokens_scale is not None or isinstance(unzipped_tokens, F8.GatheredRows))
             node.input_fp8 = unzipped_tokens
             node.input_scale = unzipped_tokens_scale
             self.m_indices = node.gen_m_indices(self.padding_token_per_experts)
@@ -113,7 +118,8 @@ class FusionMlpNode:
         # (what a one-shot backward uses) from the counts it is handed: the full list, as the reference passes; the
         # expert-by-expert loop (is_split_group_gemm) needs the slice's own counts
         counts = _split_list_prefix(padding_token_per_experts, start_idx, end_idx) if node.is_split_group_gemm else padding_token_per_experts
-        output[sl] = node.forward((unzipped_tokens[sl], unzipped_tokens_scale[sl]), unzipped_probs[sl], counts, m_indices=self.m_indices[sl])
+        rows = unzipped_tokens[sl] if isinstance(unzipped_tokens, F8.GatheredRows) else (unzipped_tokens[sl], unzipped_tokens_scale[sl])
+        output[sl] = node.forward(rows, unzipped_probs[sl], counts, m_indices=self.m_indices[sl])
         return output
 
     def gemm_backward_subbatch(self, unzipped_grad, output, padding_token_per_experts, start_idx, end_idx, reset_status=False):
@@ -127,7 +133,8 @@ class FusionMlpNode:
             else unzipped_grad[sl].contiguous()
         dx, probs_grad = node.backward(
             grad, self.unzipped_probs[sl].contiguous(), _split_list_prefix(padding_token_per_experts, start_idx, end_idx),
-            input_fp8_slice=node.input_fp8[sl].contiguous(), input_scale_slice=node.input_scale[sl].contiguous(),
+            input_fp8_slice=node.input_fp8[sl].contiguous(),
+            input_scale_slice=None if node.input_scale is None else node.input_scale[sl].contiguous(),
             m_indices=self.m_indices[sl].contiguous(), reset_status=reset_status)
         output[sl] = dx
         return probs_grad
@@ -145,11 +152,13 @@ class FusionMlpNode:
         self.padding_token_per_experts = padding_token_per_experts
         self.dispatched_indices = dispatched_indices.to(torch.int32)
         total_zipped_tokens = extract_first_if_tuple(hs_2d_dispatched).shape[0]
+        node = self.experts_group_gemm_node
+        map_only = (self.fuse_unzip and isinstance(hs_2d_dispatched, tuple) and not node.is_split_group_gemm and not node.use_ue8m0
+                    and total_zipped_tokens > 0)
         unzipped_tokens, zipped_expertwise_rowmap, unzipped_probs, unzipped_tokens_scale = self.unzip_node.forward(
             hs_2d_dispatched, self.dispatched_indices, dispatched_probs, topk=self.router_topk, num_experts=num_experts,
-            tokens_per_expert=self.tokens_per_expert)
+            tokens_per_expert=self.tokens_per_expert, do_gather=not map_only)
         self.unzipped_probs = unzipped_probs          # [rows, 1] already
-        node = self.experts_group_gemm_node
         total_unzipped_tokens = unzipped_tokens.shape[0]
         # adaptive recompute of the up+gate output: on when this rank received more rows than the balanced share times a ratio
         if self.recompute_fwd_gate_up == -1:
@@ -167,7 +176,8 @@ class FusionMlpNode:
                 self.gemm_forward_subbatch(unzipped_tokens, unzipped_tokens_scale, unzipped_probs, expert_out,
                                            padding_token_per_experts, start, start + subbatch_rows)
         elif fp8_tokens:
-            expert_out = node.forward((unzipped_tokens, unzipped_tokens_scale), unzipped_probs, padding_token_per_experts)
+            rows = unzipped_tokens if map_only else (unzipped_tokens, unzipped_tokens_scale)
+            expert_out = node.forward(rows, unzipped_probs, padding_token_per_experts)
         else:
             expert_out = node.forward(unzipped_tokens, unzipped_probs, padding_token_per_experts)
         return self.zip_node.forward(expert_out.reshape(-1, expert_out.shape[-1]), zipped_expertwise_rowmap, self.dispatched_indices,

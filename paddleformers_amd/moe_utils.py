@@ -20,11 +20,11 @@ PADDING_ALIGNMENT = 128     # row granularity of the contiguous grouped GEMM (mo
 _Tokens = Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]
 
 
-def _permute(tokens: _Tokens, routemap, probs, num_experts, tokens_per_expert):
+def _permute(tokens: _Tokens, routemap, probs, num_experts, tokens_per_expert, do_gather=True):
     """moe_permute on bf16 tokens or on an (e4m3 tokens, 1x128 scales) pair, as both nodes call it."""
     x, scale = tokens if isinstance(tokens, tuple) else (tokens, None)
     return F8.moe_permute(x, scale, routemap, probs, num_experts=num_experts, tokens_per_expert=tokens_per_expert,
-                          padding_alignment=PADDING_ALIGNMENT)
+                          padding_alignment=PADDING_ALIGNMENT, do_gather=do_gather)
 
 
 class UnZipNode:
@@ -41,10 +41,13 @@ class UnZipNode:
 
     @torch.no_grad()
     def forward(self, hs_2d_dispatched: _Tokens, dispatched_indices: torch.Tensor, dispatched_probs: Optional[torch.Tensor],
-                topk: int, num_experts: int, tokens_per_expert: Sequence[int]):
+                topk: int, num_experts: int, tokens_per_expert: Sequence[int], do_gather: bool = True):
+        """do_gather=False (e4m3 tokens only): no row is copied; the first result is the `GatheredRows` the expert MLP
+        node reads the tokens through, the last is None."""
         if dispatched_indices.shape[1] != topk:
             raise ValueError(f"dispatched_indices holds {dispatched_indices.shape[1]} slots per token, topk is {topk}")
-        rows, rowmap, probs, scale = _permute(hs_2d_dispatched, dispatched_indices, dispatched_probs, num_experts, tokens_per_expert)
+        rows, rowmap, probs, scale = _permute(hs_2d_dispatched, dispatched_indices, dispatched_probs, num_experts, tokens_per_expert,
+                                              do_gather=do_gather)
         self.unzipped_probs, self.zipped_expertwise_rowmap = probs, rowmap
         return rows, rowmap, probs, scale
 
