@@ -87,26 +87,31 @@ PF8O_API uint16_t pf8o_f32_to_bf16(float f) {
     return (uint16_t)(b >> 16);
 }
 
-/* expf with a fixed, portable operation sequence so that the device code can restate it bit for
- * bit: clamp, Cody-Waite reduction with two fused steps, degree-5 polynomial (Cephes expf
- * coefficients) evaluated by Horner with fused multiply-adds, exact power-of-two scaling.
- * The reference only says `F.silu(x) * y` (transformers/fp8_utils.py:26-29); which expf Paddle's
- * CUDA swiglu uses is not visible, so this definition is the build's own (parity unpinned). */
+/* expf with a fixed, portable operation sequence that the device code restates bit for bit, chosen short (the fused
+ * SwiGLU quantizer is bound by its arithmetic): t = x * log2(e) clamped to [-125, 126]; n = round-to-nearest-even of t by
+ * adding and subtracting 1.5 * 2^23; f = t - n (exact, |f| <= 0.5); 2^f by a degree-4 polynomial (minimax for the relative
+ * error, 2^-18.4, constant term 1) in Horner form with fused multiply-adds; the scaling by 2^n adds n to the exponent
+ * field, n taken from the low bits of the rounded sum.  Relative error below 2^-17 over the clamp range (the product
+ * x * log2(e) is rounded once); outside it the value is the clamp's.
+ * The reference only says `F.silu(x) * y` (transformers/fp8_utils.py:26-29); which expf Paddle's CUDA swiglu uses is not
+ * visible, so this definition is the build's own (parity unpinned); its results are rounded to bf16 (relative 2^-8). */
 PF8O_API float pf8o_expf(float x) {
-    x = fminf(fmaxf(x, -87.0f), 88.5f);
-    float n = rintf(x * 1.44269504088896341f);
-    float r = fmaf(n, -0.693359375f, x);
-    r = fmaf(n, 2.12194440e-4f, r);
-    float p = 1.9875691500e-4f;
-    p = fmaf(p, r, 1.3981999507e-3f);
-    p = fmaf(p, r, 8.3334519073e-3f);
-    p = fmaf(p, r, 4.1665795894e-2f);
-    p = fmaf(p, r, 1.6666665459e-1f);
-    p = fmaf(p, r, 5.0000001201e-1f);
-    float r2 = r * r;
-    float y = fmaf(p, r2, r);
-    y = y + 1.0f;
-    return ldexpf(y, (int)n);
+    float t = x * 1.44269504088896341f;
+    t = fminf(fmaxf(t, -125.0f), 126.0f);
+    float s = t + 12582912.0f;
+    float n = s - 12582912.0f;
+    float f = t - n;
+    float p = 9.584701620042324e-3f;
+    p = fmaf(p, f, 5.590607970952988e-2f);
+    p = fmaf(p, f, 2.4024060368537903e-1f);
+    p = fmaf(p, f, 6.931242942810059e-1f);
+    p = fmaf(p, f, 1.0f);
+    uint32_t pb, sb;
+    memcpy(&pb, &p, 4);
+    memcpy(&sb, &s, 4);
+    pb += sb << 23;
+    memcpy(&p, &pb, 4);
+    return p;
 }
 
 /* silu(g) = g / (1 + exp(-g)) in fp32.  transformers/fp8_utils.py:26-29, nn/mlp.py:21-23. */

@@ -105,7 +105,13 @@ __device__ __forceinline__ TileScale make_scale_from(float s) {
     return t;
 }
 // s = amax/448 (IEEE divide), amax == 0 -> 1; pow2: decode scale rounded up to a power of two.
+// For a bf16-valued amax m 2^E with a normal quotient the rounded-up power of two needs no division: 448 = 1.75 2^8, so
+// it is 2^(E-8) when m <= 1.75 and 2^(E-7) above (the next bf16 mantissa after 1.75 is 2^-7 away, far from where the fp32
+// rounding of the quotient could reach a power of two), i.e. the exponent field of amax + 0x1FFFFF less 8.  Any other
+// amax (not a bf16 value, or so small that the quotient is subnormal) takes the division.
 __device__ __forceinline__ float scale_of(uint32_t amax_bits, bool pow2) {
+    if (pow2 && __builtin_expect(amax_bits >= 0x04800000u && (amax_bits & 0xFFFFu) == 0u, 1))
+        return u2f(((amax_bits + 0x001FFFFFu) & 0x7F800000u) - 0x04000000u);
     float s = u2f(amax_bits) / 448.0f;
     if (pow2) s = u2f((f2u(s) + 0x007FFFFFu) & 0x7F800000u);
     return amax_bits == 0u ? 1.0f : s;
@@ -197,41 +203,48 @@ __device__ __forceinline__ void e4m3x4_to_f32(uint32_t w, float* f) {
     f[0] = lo[0]; f[1] = lo[1]; f[2] = hi[0]; f[3] = hi[1];
 }
 
-// expf restated operation for operation from the CPU checker: clamp, Cody-Waite reduction with two
-// fused steps, degree-5 Horner polynomial with fused multiply-adds, exact power-of-two scaling.
-__device__ __forceinline__ float expf_fixed(float x) {
-    x = __builtin_fminf(__builtin_fmaxf(x, -87.0f), 88.5f);
-    float n = __builtin_rintf(x * 1.44269504088896341f);
-    float r = __builtin_fmaf(n, -0.693359375f, x);
-    r = __builtin_fmaf(n, 2.12194440e-4f, r);
-    float p = 1.9875691500e-4f;
-    p = __builtin_fmaf(p, r, 1.3981999507e-3f);
-    p = __builtin_fmaf(p, r, 8.3334519073e-3f);
-    p = __builtin_fmaf(p, r, 4.1665795894e-2f);
-    p = __builtin_fmaf(p, r, 1.6666665459e-1f);
-    p = __builtin_fmaf(p, r, 5.0000001201e-1f);
-    float r2 = r * r;
-    float y = __builtin_fmaf(p, r2, r);
-    y = y + 1.0f;
-    return __builtin_ldexpf(y, (int)n);
+// expf restated operation for operation from the CPU checker: t = x log2(e) clamped to [-125, 126], n = t rounded by adding
+// and subtracting 1.5 * 2^23, 2^(t - n) by a degree-4 Horner polynomial with fused multiply-adds, n added to the exponent
+// field straight from the low bits of the rounded sum.  Ten instructions; relative error below 2^-17.
+// The polynomial's coefficients as values the compiler has to keep in registers: handed to expf_fixed / silu_exact by a
+// kernel that evaluates many of them, they turn the Horner steps into three-operand multiply-adds with no constant to
+// re-materialise in between.
+struct ExpPoly { float c4, c3, c2, c1; };
+__device__ __forceinline__ ExpPoly exp_poly() {
+    return ExpPoly{9.584701620042324e-3f, 5.590607970952988e-2f, 2.4024060368537903e-1f, 6.931242942810059e-1f};
 }
+__device__ __forceinline__ ExpPoly exp_poly_in_registers() {
+    ExpPoly k = exp_poly();
+    asm volatile("" : "+v"(k.c4), "+v"(k.c3), "+v"(k.c2), "+v"(k.c1));
+    return k;
+}
+__device__ __forceinline__ float expf_fixed(float x, const ExpPoly& k) {
+    // the clamp as one median-of-three (a NaN comes out as the lower bound, as fminf(fmaxf()) leaves it)
+    const float t = __builtin_amdgcn_fmed3f(x * 1.44269504088896341f, -125.0f, 126.0f);
+    const float s = t + 12582912.0f;
+    const float n = s - 12582912.0f;
+    const float f = t - n;
+    float p = __builtin_fmaf(k.c4, f, k.c3);
+    p = __builtin_fmaf(p, f, k.c2);
+    p = __builtin_fmaf(p, f, k.c1);
+    p = __builtin_fmaf(p, f, 1.0f);
+    return u2f(f2u(p) + (f2u(s) << 23));
+}
+__device__ __forceinline__ float expf_fixed(float x) { return expf_fixed(x, exp_poly()); }
 
-// silu(g) = g / (1 + exp(-g)) with the correctly rounded quotient, without the IEEE division sequence.
-// Numerator and denominator are both scaled by 1/8 (exact: g is a bf16 value, the denominator is at least
-// 1), which keeps the denominator below 2^125 where v_rcp_f32 still returns a normal number (the
-// exponential clamps at exp(88.5) = 2.7e38).  Then y = rcp refined by one Newton step, q0 = g' y,
-// r = fma(-q0, den', g'), q = fma(r, y, q0), and the sign of g is copied over (g = -0).  g is always a bf16
-// value in this library: the GPU test suite compares this routine with the CPU checker's division on every
-// one of the 65,536 bf16 inputs, bit for bit.
-__device__ __forceinline__ float silu_exact(float g) {
-    const float den = __builtin_fmaf(expf_fixed(-g), 0.125f, 0.125f);     // (1 + exp(-g)) / 8, same rounding
-    const float g8 = g * 0.125f;
-    float y = __builtin_amdgcn_rcpf(den);
-    y = __builtin_fmaf(__builtin_fmaf(-den, y, 1.0f), y, y);
-    const float q0 = g8 * y;
-    const float r = __builtin_fmaf(-q0, den, g8);
+// silu(g) = g / (1 + exp(-g)) with the correctly rounded quotient, without the IEEE division sequence: y = v_rcp_f32 of
+// the denominator (within one unit in the last place), q0 = g y, r = fma(-q0, den, g), q = fma(r, y, q0), and the sign of g
+// copied over (g = -0).  The denominator lies in [1, 2^126], so the reciprocal is a normal number.  g is always a bf16
+// value in this library and the denominator a function of g: the GPU test suite compares this routine with the CPU
+// checker's division on every one of the 65,536 bf16 inputs, bit for bit.
+__device__ __forceinline__ float silu_exact(float g, const ExpPoly& k) {
+    const float den = 1.0f + expf_fixed(-g, k);
+    const float y = __builtin_amdgcn_rcpf(den);
+    const float q0 = g * y;
+    const float r = __builtin_fmaf(-q0, den, g);
     return __builtin_copysignf(__builtin_fmaf(r, y, q0), g);
 }
+__device__ __forceinline__ float silu_exact(float g) { return silu_exact(g, exp_poly()); }
 
 // Contiguous-grouped GEMM with UE8M0 scales: which of the two kernels takes an expert load, from the
 // work-item list's header {paired 256-row items, 128-row blocks}.  Rounds of tiles per compute unit,

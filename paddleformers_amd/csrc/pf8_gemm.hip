@@ -631,6 +631,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
             const int er = lane >> 4, ec = lane & 15;
             const int64_t col = (wp ? a.inter : 0) + cp * 128 + ec * 8;          // column of o1
             const bool has_p = a.probs != nullptr;
+            const ExpPoly poly = exp_poly_in_registers();
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -661,18 +662,18 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                     const uint4 wg = *reinterpret_cast<const uint4*>(ep_g + rl * EP_LD + ec * 16);
                     const uint4 wu = *reinterpret_cast<const uint4*>(ep_u + rl * EP_LD + ec * 16);
                     const float pr = has_p ? a.probs[row] : 1.0f;
-                    float gv[8], uv[8], v[8];
-                    unpack8(wg, gv);
-                    unpack8(wu, uv);
-                    uint32_t am = 0;
+                    // as in k_swiglu_quant: products rounded to bf16 in pairs, amax on the packed magnitudes
+                    const uint32_t gw[4] = {wg.x, wg.y, wg.z, wg.w}, uw[4] = {wu.x, wu.y, wu.z, wu.w};
+                    uint32_t pk[4];
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        float y = round_bf16(silu_exact(gv[i]) * uv[i]);
-                        if (has_p) y = round_bf16(y * pr);
-                        v[i] = y;
-                        am = umax(am, f2u(y) & 0x7FFFFFFFu);
+                    for (int i = 0; i < 4; ++i) {
+                        uint32_t w = pack_bf16(silu_exact(bf16_lo(gw[i]), poly) * bf16_lo(uw[i]), silu_exact(bf16_hi(gw[i]), poly) * bf16_hi(uw[i]));
+                        pk[i] = pack_bf16(bf16_lo(w) * pr, bf16_hi(w) * pr);         // pr = 1 without probabilities: the product is exact
                     }
-                    const TileScale t = make_scale(row16_max(am), a.pow2_out != 0);
+                    const uint32_t m = pkmax_u16(pkmax_u16(pk[0] & 0x7FFF7FFFu, pk[1] & 0x7FFF7FFFu), pkmax_u16(pk[2] & 0x7FFF7FFFu, pk[3] & 0x7FFF7FFFu));
+                    const TileScale t = make_scale(row16_max(umax(m << 16, m & 0xFFFF0000u)), a.pow2_out != 0);
+                    float v[8];
+                    unpack8(make_uint4(pk[0], pk[1], pk[2], pk[3]), v);
                     const uint2 o = quant8(v, t);
                     if (c_rows) {
                         st8(a.q2 + row * a.inter + cp * 128 + ec * 8, o);
