@@ -17,6 +17,11 @@
  *   - scale_layout: 0 = row-major [rows, K/128] (output_scale_transpose=False),
  *                   1 = [K/128, rows]          (output_scale_transpose=True, the layout the GEMMs
  *                       consume as `.T`, transformers/fp8_utils.py:278,941).
+ *                   2 = [K/128, rows] UE8M0 exponent bytes (uint8 behind the float* argument, scale =
+ *                       2^(byte - 127); needs pow2): what the *_ue8m0 GEMMs read as `sa`, the scale format of
+ *                       use_ue8m0 (transformers/configuration_utils.py:454-459).  Taken by pf8_quant_1x128 and
+ *                       pf8_swiglu_weighted_quant; pf8_quant_and_transpose_split writes its row scales this
+ *                       way with pow2_rows = 2, pf8_transpose_split_quant reads such scales with xs_layout = 2.
  *   - pow2: 0 = s = amax/448 (cli/train/deepseek_v3_pretrain/kernel.py:44);
  *           1 = s rounded up to a power of two (utils/upcast_downcast_triton.py:71-85).
  *     An all-zero tile gets s = 1 and zero bytes.

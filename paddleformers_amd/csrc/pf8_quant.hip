@@ -56,7 +56,8 @@ __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict_
         const int kb = kb0 + 4 * l + g;
         if (kb < KB) {
             if (LAYOUT == 0) s[r * KB + kb] = sc;
-            else s[(int64_t)kb * M + r] = sc;
+            else if (LAYOUT == 1) s[(int64_t)kb * M + r] = sc;
+            else reinterpret_cast<uint8_t*>(s)[(int64_t)kb * M + r] = (uint8_t)(f2u(sc) >> 23);     // UE8M0: the exponent field of a power of two
         }
     }
     // cross-lane reads see only active lanes: every broadcast happens while the wavefront is whole
@@ -134,7 +135,8 @@ __global__ __launch_bounds__(256) void k_swiglu_quant(const uint16_t* __restrict
             st8(qr + kb * 16 + l, o);
             if (l == 0) {
                 if (LAYOUT == 0) s[r * IB + kb] = t.s;
-                else s[(int64_t)kb * M + r] = t.s;
+                else if (LAYOUT == 1) s[(int64_t)kb * M + r] = t.s;
+                else reinterpret_cast<uint8_t*>(s)[(int64_t)kb * M + r] = (uint8_t)(f2u(t.s) >> 23);
             }
         }
     }
@@ -348,7 +350,8 @@ __device__ __forceinline__ void load_patch_packed(const TileSrc& src, int64_t ro
                 continue;
             }
             q[i] = ld8(src.xq + r * src.ld + col0 + 8 * l);
-            sc[i] = src.xs_layout == 0 ? src.xs[r * KB + col0 / 128] : src.xs[(col0 / 128) * src.rows + r];
+            if (src.xs_layout == 2) sc[i] = u2f((uint32_t)reinterpret_cast<const uint8_t*>(src.xs)[(col0 / 128) * src.rows + r] << 23);
+            else sc[i] = src.xs_layout == 0 ? src.xs[r * KB + col0 / 128] : src.xs[(col0 / 128) * src.rows + r];
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -449,6 +452,7 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
             st8(q + r * K + col0 + 8 * l, quant8(v, t));
             if (l == i) {
                 if (LAYOUT == 0) s[r * KB + tc] = t.s;
+                else if (pow2 & 4) reinterpret_cast<uint8_t*>(s)[tc * M + r] = (uint8_t)(f2u(t.s) >> 23);      // UE8M0 bytes [K/128, M]
                 else s[tc * M + r] = t.s;
             }
         }
@@ -651,8 +655,9 @@ extern "C" int pf8_quant_1x128(const uint16_t* x, int64_t M, int64_t K, int64_t 
     if (M == 0 || K == 0) return PF8_OK;
     PF8_REQUIRE(x && q && s, "null pointer");
     PF8_REQUIRE(ldx >= K && ldx % 8 == 0, "ldx must be >= K and a multiple of 8");
-    PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q) && (reinterpret_cast<uintptr_t>(s) & 3u) == 0, "pointers must be 16-byte aligned");
-    PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
+    PF8_REQUIRE(PF8_ALIGNED16(x) && PF8_ALIGNED16(q) && (scale_layout == 2 || (reinterpret_cast<uintptr_t>(s) & 3u) == 0), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(scale_layout >= 0 && scale_layout <= 2, "scale_layout must be 0, 1 or 2");
+    PF8_REQUIRE(scale_layout != 2 || pow2, "UE8M0 scale bytes (scale_layout 2) need power-of-two scales");
     PF8_REQUIRE(K / 128 <= 0x7FFFFF, "shape too large");
     hipStream_t st = (hipStream_t)stream;
     const int KB = (int)(K / 128);
@@ -663,7 +668,8 @@ extern "C" int pf8_quant_1x128(const uint16_t* x, int64_t M, int64_t K, int64_t 
         const int64_t m = M - m0 < slab ? M - m0 : slab;
         dim3 grid((unsigned)((KB + 4 * U - 1) / (4 * U)), (unsigned)((m + 3) / 4)), block(256);
         if (scale_layout == 0) hipLaunchKernelGGL((k_quant_1x128<0, U>), grid, block, 0, st, x, M, m0, KB, ldx, q, s, pow2);
-        else hipLaunchKernelGGL((k_quant_1x128<1, U>), grid, block, 0, st, x, M, m0, KB, ldx, q, s, pow2);
+        else if (scale_layout == 1) hipLaunchKernelGGL((k_quant_1x128<1, U>), grid, block, 0, st, x, M, m0, KB, ldx, q, s, pow2);
+        else hipLaunchKernelGGL((k_quant_1x128<2, U>), grid, block, 0, st, x, M, m0, KB, ldx, q, s, pow2);
         int rc = pf8_check_launch(__func__);
         if (rc) return rc;
     }
@@ -763,7 +769,7 @@ static int transpose_split_quant(const char* where, const void* x, const float* 
                                  const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q, float* s, uint8_t* q_t, float* s_t,
                                  int pow2_bits, pf8_stream_t stream, const int32_t* src_row = nullptr, int64_t src_rows = 0) {
 #define PF8_REQUIRE_AT(cond, msg) do { if (!(cond)) return pf8_fail(PF8_EINVAL, where, msg); } while (0)
-    PF8_REQUIRE_AT(xs_layout == 0 || xs_layout == 1, "xs_layout must be 0 or 1");
+    PF8_REQUIRE_AT(xs_layout >= 0 && xs_layout <= 2, "xs_layout must be 0, 1 or 2");
     PF8_REQUIRE_AT(E >= 0 && K >= 0, "negative shape");
     PF8_REQUIRE_AT(K % 128 == 0, "K must be a multiple of 128");
     PF8_REQUIRE_AT(E <= 256, "at most 256 experts per call");
@@ -814,7 +820,9 @@ extern "C" int pf8_transpose_split_quant_gather(const uint8_t* tokens, const flo
 extern "C" int pf8_quant_and_transpose_split(const uint16_t* x, const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q, float* s,
                                              int pow2_rows, uint8_t* q_t, float* s_t, int pow2_t, pf8_stream_t stream) {
     PF8_REQUIRE(q && s, "null pointer");
-    return transpose_split_quant(__func__, x, nullptr, 0, 0, rows_per_expert, E, K, q, s, q_t, s_t, (pow2_t ? 1 : 0) | (pow2_rows ? 2 : 0), stream);
+    // pow2_rows == 2: the row scales (powers of two) are written as UE8M0 bytes [K/128, Mtot] into s
+    return transpose_split_quant(__func__, x, nullptr, 0, 0, rows_per_expert, E, K, q, s, q_t, s_t,
+                                 (pow2_t ? 1 : 0) | (pow2_rows ? 2 : 0) | (pow2_rows == 2 ? 4 : 0), stream);
 }
 
 extern "C" int pf8_swiglu_weighted_quant(const uint16_t* o1, const float* probs, int64_t M, int64_t I, uint8_t* q, float* s,
@@ -824,7 +832,8 @@ extern "C" int pf8_swiglu_weighted_quant(const uint16_t* o1, const float* probs,
     if (M == 0 || I == 0) return PF8_OK;
     PF8_REQUIRE(o1 && q && s, "null pointer");
     PF8_REQUIRE(PF8_ALIGNED16(o1) && PF8_ALIGNED16(q) && PF8_ALIGNED16(o2), "pointers must be 16-byte aligned");
-    PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
+    PF8_REQUIRE(scale_layout >= 0 && scale_layout <= 2, "scale_layout must be 0, 1 or 2");
+    PF8_REQUIRE(scale_layout != 2 || pow2, "UE8M0 scale bytes (scale_layout 2) need power-of-two scales");
     PF8_REQUIRE(I / 128 <= 0x7FFFFF, "shape too large");
     const int IB = (int)(I / 128);
     const int64_t slab = (int64_t)65535 * 4;
@@ -835,10 +844,14 @@ extern "C" int pf8_swiglu_weighted_quant(const uint16_t* o1, const float* probs,
             hipLaunchKernelGGL((k_swiglu_quant<0, true>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
         else if (scale_layout == 0)
             hipLaunchKernelGGL((k_swiglu_quant<0, false>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
-        else if (probs)
+        else if (scale_layout == 1 && probs)
             hipLaunchKernelGGL((k_swiglu_quant<1, true>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
-        else
+        else if (scale_layout == 1)
             hipLaunchKernelGGL((k_swiglu_quant<1, false>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
+        else if (probs)
+            hipLaunchKernelGGL((k_swiglu_quant<2, true>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
+        else
+            hipLaunchKernelGGL((k_swiglu_quant<2, false>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
         int rc = pf8_check_launch(__func__);
         if (rc) return rc;
     }

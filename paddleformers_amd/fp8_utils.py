@@ -635,6 +635,13 @@ class FP8GroupGemmMlpFunctionNode:
         self.fwd_subbatch = None
         self.bwd_subbatch = None
 
+    @property
+    def _scale_bytes(self):
+        """use_ue8m0 with one grouped launch per GEMM: the activation quantizers write their (power-of-two) scales as the
+        UE8M0 bytes the block-scaled GEMM reads, so no conversion pass runs between them (the expert-by-expert loop of
+        is_split_group_gemm takes fp32 scales)."""
+        return bool(self.use_ue8m0 and not self.is_split_group_gemm)
+
     def reset_statue(self):
         self.m_indices = None
         self._group_items = None
@@ -728,7 +735,7 @@ class FP8GroupGemmMlpFunctionNode:
             x_scale = x_scale.t().contiguous().t()
         else:
             x_fp8, x_scale = F8.fp8_quant_blockwise(x, output_scale_transpose=True, quant_method="1x128", input_transpose=False,
-                                                    using_pow2_scale=self.use_ue8m0)
+                                                    using_pow2_scale=self.use_ue8m0, ue8m0_scale=self._scale_bytes)
             x_scale = x_scale.T
         o1 = torch.empty([x_fp8.shape[0], w1_t_quant.shape[1]], dtype=expert_w1[0].dtype, device=x_fp8.device)
         if numpy.prod(x_fp8.shape) != 0:
@@ -748,7 +755,7 @@ class FP8GroupGemmMlpFunctionNode:
         """o3 [m_sum, H] = quant(swiglu(o1) * probs) . w2 (fp8_utils.py:965-1009)."""
         w2_quant, w2_scale, w2_cache = self._stacked(expert_w2, True, num_expert)
         unzipped_probs = unzipped_probs.squeeze(-1)
-        o2_fp8, o2_scale = F8.fused_weighted_swiglu_act_quant(o1, unzipped_probs, using_pow2_scaling=True)
+        o2_fp8, o2_scale = F8.fused_weighted_swiglu_act_quant(o1, unzipped_probs, using_pow2_scaling=True, ue8m0_scale=self._scale_bytes)
         o3_shape = [o2_fp8.shape[0], w2_quant.shape[1]]
         if o3 is not None:
             assert list(o3.shape) == o3_shape, "{} vs {}".format(list(o3.shape), o3_shape)
@@ -770,7 +777,7 @@ class FP8GroupGemmMlpFunctionNode:
         else:
             unzipped_grad_fp8, unzipped_grad_scale = F8.fp8_quant_blockwise(unzipped_grad, output_scale_transpose=True,
                                                                             quant_method="1x128", input_transpose=False,
-                                                                            using_pow2_scale=self.use_ue8m0)
+                                                                            using_pow2_scale=self.use_ue8m0, ue8m0_scale=self._scale_bytes)
             unzipped_grad_scale = unzipped_grad_scale.T
         do2_s = torch.empty([unzipped_grad_fp8.shape[0], bw_w2_quant.shape[1]], dtype=torch.bfloat16, device=o1.device)
         if numpy.prod(unzipped_grad_fp8.shape) != 0:
@@ -790,7 +797,7 @@ class FP8GroupGemmMlpFunctionNode:
             do1_fp8, do1_scale = do1
         else:
             do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, output_scale_transpose=True, quant_method="1x128", input_transpose=False,
-                                                        using_pow2_scale=self.use_ue8m0)
+                                                        using_pow2_scale=self.use_ue8m0, ue8m0_scale=self._scale_bytes)
             do1_scale = do1_scale.T
         do1 = do1_fp8
         dx_shape = [do1_fp8.shape[0], bw_w1_quant.shape[1]]
@@ -980,7 +987,8 @@ class FP8GroupGemmMlpFunctionNode:
         fuse = self.fuse_bwd_quant and not self.is_split_group_gemm and len(tokens_per_expert) <= 256
         do3_t = None
         if fuse and not isinstance(out_grad, tuple) and out_grad.dtype == torch.bfloat16:
-            g_fp8, g_scale, g_t_fp8, g_t_scale = F8.quant_and_transpose_split(out_grad, tokens_per_expert, self.use_ue8m0, True)
+            g_fp8, g_scale, g_t_fp8, g_t_scale = F8.quant_and_transpose_split(out_grad, tokens_per_expert, self.use_ue8m0, True,
+                                                                              ue8m0_scale=self._scale_bytes)
             out_grad, do3_t = (g_fp8, g_scale.T), (g_t_fp8, g_t_scale)
         do1, o2_s, probs_grad = self.bwd_dowm_input(expert_w2, out_grad, o1, tokens_per_expert, unzipped_probs=unzipped_probs,
                                                     m_indices=m_indices)
@@ -988,7 +996,8 @@ class FP8GroupGemmMlpFunctionNode:
         self.o1 = None
         do1_rows = do1_t = do1
         if fuse:
-            d_fp8, d_scale, d_t_fp8, d_t_scale = F8.quant_and_transpose_split(do1, tokens_per_expert, self.use_ue8m0, True)
+            d_fp8, d_scale, d_t_fp8, d_t_scale = F8.quant_and_transpose_split(do1, tokens_per_expert, self.use_ue8m0, True,
+                                                                              ue8m0_scale=self._scale_bytes)
             do1_rows, do1_t = (d_fp8, d_scale.T), (d_t_fp8, d_t_scale)
         del do1
         self.bwd_gate_up_weight(do1_t, None, expert_w1, tokens_per_expert, input_fp8_slice=input_fp8_slice,

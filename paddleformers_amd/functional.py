@@ -86,11 +86,14 @@ class GatheredRows:
         return rows.view(FP8), self.scale[idx] * live[:, None].to(torch.float32)
 
 
-def _scale_layout_of(s: torch.Tensor, rows: int, blocks: int, what: str) -> Tuple[torch.Tensor, int]:
+def _scale_layout_of(s: torch.Tensor, rows: int, blocks: int, what: str, allow_ue8m0: bool = False) -> Tuple[torch.Tensor, int]:
     """A logical [rows, blocks] scale tensor -> (tensor, layout flag) without copying when its
-    memory is either row-major (0) or blocks-major, i.e. a transposed view of [blocks, rows] (1)."""
+    memory is either row-major (0) or blocks-major, i.e. a transposed view of [blocks, rows] (1);
+    UE8M0 exponent bytes (uint8, where the caller takes them) are layout 2, blocks-major."""
     if tuple(s.shape) != (rows, blocks):
         raise ValueError(f"{what} must have shape [{rows}, {blocks}], got {list(s.shape)}")
+    if s.dtype == torch.uint8 and allow_ue8m0:          # UE8M0 bytes: blocks-major only
+        return (s if s.stride() == (1, rows) else s.t().contiguous().t()), 2
     if s.dtype != torch.float32:
         raise ValueError(f"{what} must be float32")
     if s.is_contiguous():
@@ -112,6 +115,7 @@ def fp8_quant_blockwise(
     output_scale_transpose: bool = False,
     return_transpose_only: bool = False,
     using_pow2_scale: bool = False,
+    ue8m0_scale: bool = False,
 ):
     """Block-wise e4m3 quantization, scale = amax/448 per tile.
 
@@ -120,6 +124,9 @@ def fp8_quant_blockwise(
     input_transpose, or (q_t, s_t) when also return_transpose_only.
     Scale shapes: 1x128 -> [M, K/128], or [K/128, M] with output_scale_transpose (transposed copy:
     [K, M/128] / [M/128, K]); 128x128 -> [R/128, C/128] (transposed copy [C/128, R/128]).
+    ue8m0_scale (1x128 without input_transpose, power-of-two scales): the scales come back as UE8M0 exponent bytes
+    (uint8, scale = 2^(byte - 127)) of the same logical shape, stored [K/128, M] -- the form the block-scaled GEMMs of
+    `use_ue8m0` (transformers/configuration_utils.py:454-459) read, written by the quantizer itself.
     """
     _dev(x, "x")
     if x.dtype != torch.bfloat16:
@@ -136,6 +143,13 @@ def fp8_quant_blockwise(
         if K % 128 != 0:
             raise ValueError(f"last dimension must be divisible by 128, got {K}")
         lay = 1 if output_scale_transpose else 0
+        if ue8m0_scale:
+            if input_transpose or not pow2:
+                raise ValueError("ue8m0_scale goes with using_pow2_scale=True and input_transpose=False")
+            q = torch.empty((M, K), dtype=FP8, device=dev)
+            s = torch.empty((K // 128, M), dtype=torch.uint8, device=dev)
+            _lib.call("pf8_quant_1x128", _p(x2), M, K, K, _p(q), _p(s), 2, 1, _stream())
+            return q.reshape(x.shape), (s if output_scale_transpose else s.t())
         if not input_transpose:
             q = torch.empty((M, K), dtype=FP8, device=dev)
             s = torch.empty((K // 128, M) if lay else (M, K // 128), dtype=torch.float32, device=dev)
@@ -244,12 +258,13 @@ def fused_stack_quant_both(weight_list: Sequence[torch.Tensor], using_pow2_scale
 
 
 def fused_weighted_swiglu_act_quant(o1: torch.Tensor, probs: Optional[torch.Tensor] = None, using_pow2_scaling: bool = False,
-                                    return_o2: bool = False):
+                                    return_o2: bool = False, ue8m0_scale: bool = False):
     """quant_1x128( bf16( bf16(swiglu(o1)) * probs ) ) in one pass.
 
     transformers/fp8_utils.py:984-986; un-fused equivalent ernie token_dispatcher/fp8_utils.py:996-1004.
     o1 bf16 [M, 2I] with the gate in the first half; probs fp32 [M] (or [M, 1]) or None.
     Returns (q [M, I], s [M, I/128]); with return_o2 also the bf16 activations before quantization.
+    ue8m0_scale (with using_pow2_scaling): s is UE8M0 exponent bytes, uint8 [M, I/128] stored [I/128, M].
     """
     _dev(o1, "o1")
     if o1.dtype != torch.bfloat16 or o1.dim() != 2:
@@ -269,9 +284,16 @@ def fused_weighted_swiglu_act_quant(o1: torch.Tensor, probs: Optional[torch.Tens
             probs = probs.float()
         probs = probs.contiguous()
     q = torch.empty((M, I), dtype=FP8, device=o1.device)
-    s = torch.empty((M, I // 128), dtype=torch.float32, device=o1.device)
     o2 = torch.empty((M, I), dtype=torch.bfloat16, device=o1.device) if return_o2 else None
-    _lib.call("pf8_swiglu_weighted_quant", _p(o1), _p(probs), M, I, _p(q), _p(s), _p(o2), 0, int(bool(using_pow2_scaling)), _stream())
+    if ue8m0_scale:
+        if not using_pow2_scaling:
+            raise ValueError("ue8m0_scale goes with using_pow2_scaling=True")
+        s = torch.empty((I // 128, M), dtype=torch.uint8, device=o1.device)
+        _lib.call("pf8_swiglu_weighted_quant", _p(o1), _p(probs), M, I, _p(q), _p(s), _p(o2), 2, 1, _stream())
+        s = s.t()
+    else:
+        s = torch.empty((M, I // 128), dtype=torch.float32, device=o1.device)
+        _lib.call("pf8_swiglu_weighted_quant", _p(o1), _p(probs), M, I, _p(q), _p(s), _p(o2), 0, int(bool(using_pow2_scaling)), _stream())
     return (q, s, o2) if return_o2 else (q, s)
 
 
@@ -315,7 +337,7 @@ def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], 
         if scale is None:
             raise ValueError("an e4m3 input needs its scale tensor")
         _dev(scale, "scale")
-        scale, xs_layout = _scale_layout_of(scale, Mtot, K // 128, "scale")
+        scale, xs_layout = _scale_layout_of(scale, Mtot, K // 128, "scale", allow_ue8m0=True)
     elif x.dtype != torch.bfloat16:
         raise ValueError("x must be bfloat16 or float8_e4m3fn")
     E = len(rows)
@@ -331,9 +353,13 @@ def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], 
             if n == Mtot:
                 xs_ptr, lay = _p(scale), xs_layout
             else:
-                # more than 256 experts: hand each chunk its own row-major slice of the scales
-                keep = scale[off:off + n].contiguous()
-                xs_ptr, lay = _p(keep), 0
+                # more than 256 experts: hand each chunk its own slice of the scales (row-major fp32, blocks-major bytes)
+                if xs_layout == 2:
+                    keep = scale[off:off + n].t().contiguous()
+                    xs_ptr, lay = _p(keep), 2
+                else:
+                    keep = scale[off:off + n].contiguous()
+                    xs_ptr, lay = _p(keep), 0
         xp = C.c_void_p(x.data_ptr() + off * K * x.element_size())
         qp = C.c_void_p(q_t.data_ptr() + off * K)
         sp = C.c_void_p(s_t.data_ptr() + (off // 128) * K * 4)
@@ -372,12 +398,13 @@ def _transpose_split_quant_gathered(g: GatheredRows, rows: List[int], pow_2_scal
 
 
 def quant_and_transpose_split(x: torch.Tensor, tokens_per_expert: Sequence[int], using_pow2_scale: bool = False,
-                              pow_2_scales: bool = True):
+                              pow_2_scales: bool = True, ue8m0_scale: bool = False):
     """fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True, using_pow2_scale=...) and
     fused_transpose_split_quant(x, None, tokens_per_expert, pow_2_scales) from ONE read of x: the two
     quantizations the MoE node's backward applies to the same gradient (transformers/fp8_utils.py:1030-1036
     with :1115, :1073-1079 with :1168).  Returns (q [M,K], s [K/128,M], q_t list, s_t list), each
-    bit-identical to the separate calls' outputs.  At most 256 experts."""
+    bit-identical to the separate calls' outputs.  At most 256 experts.
+    ue8m0_scale (with using_pow2_scale): s comes back as UE8M0 exponent bytes, uint8 [K/128, M]."""
     _dev(x, "x")
     if x.dim() != 2 or x.dtype != torch.bfloat16:
         raise ValueError("x must be a 2-D bfloat16 tensor")
@@ -393,13 +420,15 @@ def quant_and_transpose_split(x: torch.Tensor, tokens_per_expert: Sequence[int],
         raise ValueError(f"last dimension must be divisible by 128, got {K}")
     if len(rows) > 256:
         raise ValueError("at most 256 experts")
+    if ue8m0_scale and not using_pow2_scale:
+        raise ValueError("ue8m0_scale goes with using_pow2_scale=True")
     q = torch.empty((Mtot, K), dtype=FP8, device=x.device)
-    s = torch.empty((K // 128, Mtot), dtype=torch.float32, device=x.device)
+    s = torch.empty((K // 128, Mtot), dtype=torch.uint8 if ue8m0_scale else torch.float32, device=x.device)
     q_t = torch.empty((K * Mtot,), dtype=FP8, device=x.device)
     s_t = torch.empty(((Mtot // 128) * K,), dtype=torch.float32, device=x.device)
     if Mtot and K:
         arr = (C.c_int64 * len(rows))(*rows)
-        _lib.call("pf8_quant_and_transpose_split", _p(x), arr, len(rows), K, _p(q), _p(s), int(bool(using_pow2_scale)),
+        _lib.call("pf8_quant_and_transpose_split", _p(x), arr, len(rows), K, _p(q), _p(s), 2 if ue8m0_scale else int(bool(using_pow2_scale)),
                   _p(q_t), _p(s_t), int(bool(pow_2_scales)), _stream())
     qs, ss, off = [], [], 0
     for r in rows:
@@ -420,6 +449,8 @@ def scales_to_ue8m0(scale: torch.Tensor, check: bool = True) -> torch.Tensor:
     `use_ue8m0` hands to deep_gemm (transformers/configuration_utils.py:454-459).  With `check` the
     call synchronizes and raises if a scale is not a positive finite power of two."""
     _dev(scale, "scale")
+    if scale.dtype == torch.uint8:            # already exponent bytes (a quantizer wrote them)
+        return scale
     if scale.dtype != torch.float32:
         raise ValueError("scale must be float32")
     dense = scale if scale.is_contiguous() or (scale.dim() == 2 and scale.t().is_contiguous()) else scale.contiguous()

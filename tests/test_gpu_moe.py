@@ -288,6 +288,52 @@ def test_moe_node_ue8m0_needs_a_pow2_weight_cache():
     assert torch.equal(plain.view(torch.int16), cached.view(torch.int16))
 
 
+def test_moe_node_ue8m0_iteration_runs_no_scale_conversion_pass(monkeypatch):
+    """With the weight cache warm, a use_ue8m0 iteration converts no scale tensor: every activation quantizer writes the
+    exponent bytes itself.  Results equal those of the fp32-scale quantizers followed by the conversion, to the bit."""
+    from paddleformers_amd import fp8_utils as U
+    from paddleformers_amd import functional as F8
+
+    E, H, I = 3, 512, 384
+    rows = [256, 0, 384]
+    _, _, experts, x, probs = _make(E, H, I, rows, seed=43)
+    dout = G.bf16_normal((sum(rows), H), seed=44, std=1e-3)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    tx, tdo = G.to_torch_bf16(x), G.to_torch_bf16(dout)
+    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True, using_pow2_scale=True)
+    converted = []
+    real = F8.scales_to_ue8m0
+
+    def counting(scale, check=True):
+        if scale.dtype == torch.float32:
+            converted.append(tuple(scale.shape))
+        return real(scale, check)
+
+    monkeypatch.setattr(F8, "scales_to_ue8m0", counting)
+
+    def run(node):
+        for e in experts:
+            e.w1.main_grad = None
+            e.w2.main_grad = None
+        o3 = node.forward(tx, tp, rows).clone()
+        dx, pg = node.backward(tdo, tp, rows)
+        return o3, dx.clone(), pg.clone(), [e.w1.main_grad.clone() for e in experts if e.w1.main_grad is not None]
+
+    run(U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True))           # warm: the weights' bytes are made here
+    converted.clear()
+    node = U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True)
+    got = run(node)
+    assert converted == [] and node._scale_bytes
+    # the expert-by-expert loop takes fp32 scales; it is the same arithmetic
+    loop = U.FP8GroupGemmMlpFunctionNode(_Map(experts), use_ue8m0=True, is_split_group_gemm=True)
+    assert not loop._scale_bytes
+    ref = run(loop)
+    assert torch.equal(got[0].view(torch.int16), ref[0].view(torch.int16)) and torch.equal(got[1].view(torch.int16), ref[1].view(torch.int16))
+    assert torch.equal(got[2], ref[2])
+    for a, b in zip(got[3], ref[3]):
+        assert G.rel_fro(a.cpu().numpy(), b.cpu().numpy()) < 1e-6
+
+
 def test_moe_node_ue8m0_weight_scale_bytes_follow_the_weight_cache():
     """The node remembers the UE8M0 bytes of the cached weight scales between calls; a new cache (new tensors) and a
     cache rewritten in place (same tensors, new contents) must both be picked up."""

@@ -519,3 +519,68 @@ def test_fused_swiglu_weighted_bwd(F):
     # tolerance 1e-5 of the row's absolute-term sum
     terms = np.abs(O.bf16_bits_to_f32(do2).astype(np.float64)).sum(axis=1) * 8.0
     assert np.all(np.abs(pg.cpu().numpy().astype(np.float64) - epg) <= 1e-5 * terms + 1e-30)
+
+
+# ---------------------------------------------------------------------------------------------
+# UE8M0 exponent bytes written by the quantizers themselves
+# ---------------------------------------------------------------------------------------------
+
+
+def _e8_of(scale_f32):
+    """Power-of-two fp32 scales -> UE8M0 bytes (the biased exponent field)."""
+    bits = np.ascontiguousarray(scale_f32).view(np.uint32)
+    assert (bits & 0x807FFFFF == 0).all(), "not powers of two"
+    return (bits >> 23).astype(np.uint8)
+
+
+@pytest.mark.parametrize("M,K", [(4, 128), (136, 1408), (515, 512)])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_quant_1x128_writes_ue8m0_bytes(F, M, K, transpose):
+    bits = G.bf16_normal((M, K), seed=M + K, outlier_frac=1e-3, outlier_scale=300.0)
+    bits[1, :128] = 0                                   # an all-zero tile: scale 1 = byte 127
+    bits[2, :128] = G.bf16_normal((128,), seed=3, std=1e-30)          # tiny values: the scale rule's division path
+    eq, es = O.quant_1x128(bits, 0, True)
+    x = G.to_torch_bf16(bits)
+    q, s = F.fp8_quant_blockwise(x, quant_method="1x128", using_pow2_scale=True, output_scale_transpose=transpose, ue8m0_scale=True)
+    assert s.dtype == torch.uint8 and tuple(s.shape) == ((K // 128, M) if transpose else (M, K // 128))
+    got = s.cpu().numpy()
+    _same(G.from_torch_fp8(q), eq, "bytes")
+    _same(got.T if transpose else got, _e8_of(es), "exponent bytes")
+    assert got[(0, 1) if transpose else (1, 0)] == 127
+    # the conversion pass is the identity on bytes
+    assert F.scales_to_ue8m0(s) is s
+    with pytest.raises(ValueError):
+        F.fp8_quant_blockwise(x, quant_method="1x128", using_pow2_scale=False, ue8m0_scale=True)
+
+
+def test_swiglu_quant_writes_ue8m0_bytes(F):
+    M, I = 260, 512
+    o1 = G.bf16_normal((M, 2 * I), seed=5, std=2.0)
+    probs = np.random.default_rng(6).random(M).astype(np.float32)
+    eq, es = O.swiglu_weighted_quant(o1, probs, pow2=True)
+    q, s = F.fused_weighted_swiglu_act_quant(G.to_torch_bf16(o1), torch.from_numpy(probs).cuda(), using_pow2_scaling=True, ue8m0_scale=True)
+    assert s.dtype == torch.uint8 and tuple(s.shape) == (M, I // 128) and s.stride() == (1, M)
+    _same(G.from_torch_fp8(q), eq, "bytes")
+    _same(s.cpu().numpy(), _e8_of(es), "exponent bytes")
+    with pytest.raises(ValueError):
+        F.fused_weighted_swiglu_act_quant(G.to_torch_bf16(o1), None, using_pow2_scaling=False, ue8m0_scale=True)
+
+
+def test_quant_and_transpose_split_writes_ue8m0_row_scales_and_reads_them_back(F):
+    rows, K = [128, 0, 256], 640
+    bits = G.bf16_normal((sum(rows), K), seed=8, outlier_frac=1e-3, outlier_scale=100.0)
+    x = G.to_torch_bf16(bits)
+    q0, s0, qt0, st0 = F.quant_and_transpose_split(x, rows, True, True)
+    q1, s1, qt1, st1 = F.quant_and_transpose_split(x, rows, True, True, ue8m0_scale=True)
+    assert s1.dtype == torch.uint8 and s1.shape == s0.shape
+    assert torch.equal(q0.view(torch.uint8), q1.view(torch.uint8))
+    _same(s1.cpu().numpy(), _e8_of(s0.cpu().numpy()), "row-scale exponent bytes")
+    for a, b in zip(qt0 + st0, qt1 + st1):
+        assert torch.equal(a.view(torch.uint8) if a.dtype != torch.float32 else a, b.view(torch.uint8) if b.dtype != torch.float32 else b)
+    # the transposed quantizer of an e4m3 input takes its scales as bytes (what the node caches in that mode)
+    qa, sa = F.fused_transpose_split_quant(q0, s0.T, rows, True)
+    qb, sb = F.fused_transpose_split_quant(q1, s1.T, rows, True)
+    for a, b in zip(qa + sa, qb + sb):
+        assert torch.equal(a.view(torch.uint8) if a.dtype != torch.float32 else a, b.view(torch.uint8) if b.dtype != torch.float32 else b)
+    with pytest.raises(ValueError):
+        F.quant_and_transpose_split(x, rows, False, True, ue8m0_scale=True)
