@@ -412,7 +412,33 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     del am, bm, sam, sbm, om
     torch.cuda.empty_cache()
     # the masked-layout expert node (fixed capacity per expert) end to end: 32 experts x 512 rows, 256..512 valid
+    out["ernie_masked_node_32x512_fwd_bwd"] = bench_masked_node(20, 3)
+    torch.cuda.empty_cache()
+    # the fused FP8 MoE node end to end at config 5: forward + backward (dgrad and wgrad, both GEMMs),
+    # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers; then the same step
+    # with power-of-two scales throughout (use_ue8m0): forward and dgrad GEMMs on the block-scaled MFMA kernel
+    node_flop = 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H)
+    out["moe_node_config5_fwd_bwd"] = dict(bench_moe_node(False, 20, 3), flop=node_flop)
+    out["moe_node_config5_fwd_bwd_ue8m0"] = dict(bench_moe_node(True, 20, 3), flop=node_flop)
+    # the layer around the node (unzip -> node -> zip and back) with FP8 dispatch, the unzip as a copy and as a row map only
+    out["moe_layer_config5_fp8_dispatch_fwd_bwd_unzip_copies"] = dict(bench_moe_layer(False, 10, 2), flop=node_flop)
+    out["moe_layer_config5_fp8_dispatch_fwd_bwd_unzip_maps"] = dict(bench_moe_layer(True, 10, 2), flop=node_flop)
+    torch.cuda.empty_cache()
+    return _finish(out)
+
+
+def bench_masked_node(iters, warmup):
+    """ms per forward + backward of the masked-layout expert node (ernie ExpertsGroupGemmNode: fixed capacity per expert,
+    a count of valid rows per expert): 32 experts x 512 rows with 256..512 valid, H=4096, I=1408, cached stacked FP8
+    weights, weight gradients accumulated into stacked fp32 buffers."""
+    import numpy as np
+    import torch
+
     from paddleformers_amd import ernie_fp8_utils as EU
+    from paddleformers_amd import functional as F8
+
+    Em, Cm = 32, 512
+    mm = torch.from_numpy(np.random.default_rng(7).integers(256, Cm + 1, Em).astype(np.int32)).cuda()
 
     class _Lin:
         def __init__(self, w):
@@ -454,23 +480,13 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
         nodem.forward(xm, prm, mm)
         nodem.backward(dm, mm, None, Cm)
 
-    ms = time_kernel(fwd_bwd_masked, [()], 20, 3)
+    ms = time_kernel(fwd_bwd_masked, [()], iters, warmup)
     valid_rows = float(mm.sum().item())
-    out["ernie_masked_node_32x512_fwd_bwd"] = dict(ms, flop=2 * (2.0 * valid_rows * Hm * 2 * Im + 2.0 * valid_rows * Im * Hm)
-                                               + (2.0 * Em * Cm * Hm * 2 * Im + 2.0 * Em * Cm * Im * Hm))
+    # forward and input-gradient GEMMs on the valid rows, weight-gradient GEMMs over the whole capacity (padding rows are zero)
+    flop = 2 * (2.0 * valid_rows * Hm * 2 * Im + 2.0 * valid_rows * Im * Hm) + (2.0 * Em * Cm * Hm * 2 * Im + 2.0 * Em * Cm * Im * Hm)
     del exm, gm1, gm2, xm, dm, nodem
     torch.cuda.empty_cache()
-    # the fused FP8 MoE node end to end at config 5: forward + backward (dgrad and wgrad, both GEMMs),
-    # cached stacked FP8 weights, weight gradients accumulated into stacked fp32 buffers; then the same step
-    # with power-of-two scales throughout (use_ue8m0): forward and dgrad GEMMs on the block-scaled MFMA kernel
-    node_flop = 3 * (2.0 * ROUTED * H * 2 * I + 2.0 * ROUTED * I * H)
-    out["moe_node_config5_fwd_bwd"] = dict(bench_moe_node(False, 20, 3), flop=node_flop)
-    out["moe_node_config5_fwd_bwd_ue8m0"] = dict(bench_moe_node(True, 20, 3), flop=node_flop)
-    # the layer around the node (unzip -> node -> zip and back) with FP8 dispatch, the unzip as a copy and as a row map only
-    out["moe_layer_config5_fp8_dispatch_fwd_bwd_unzip_copies"] = dict(bench_moe_layer(False, 10, 2), flop=node_flop)
-    out["moe_layer_config5_fp8_dispatch_fwd_bwd_unzip_maps"] = dict(bench_moe_layer(True, 10, 2), flop=node_flop)
-    torch.cuda.empty_cache()
-    return _finish(out)
+    return dict(ms, flop=flop)
 
 
 def bench_moe_node(ue8m0, iters, warmup):
@@ -671,9 +687,10 @@ def main():
                          "readings of the GEMM can be scaled by a kernel of known traffic")
     ap.add_argument("--gemm-analysis", action="store_true",
                     help="run only the analysis of the config 3 up+gate launch (ablations, block cycles, compute-unit budgets) and print it")
-    ap.add_argument("--moe-node", choices=["fp32", "ue8m0"],
+    ap.add_argument("--moe-node", choices=["fp32", "ue8m0", "masked"],
                     help="run only the config 5 MoE node leg (forward + backward, --steps/--warmup iterations) with fp32 or "
-                         "UE8M0 scales and print its time: the run to profile for the node's per-kernel breakdown")
+                         "UE8M0 scales, or the masked-layout (ernie) node's leg, and print its time: the run to profile for the "
+                         "node's per-kernel breakdown")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path uses no collectives and the run has a single MI355X; use --gpus 1",
@@ -700,6 +717,11 @@ def main():
     if args.gemm_legs_only:
         it = args.leg_iters or 50
         print(json.dumps({"other_gemm": bench_other_gemms(it, min(10, it), gemm_only=True)}))
+        return
+    if args.moe_node == "masked":
+        r = bench_masked_node(args.steps, args.warmup)
+        print(json.dumps({"leg": "ernie_masked_node_32x512_fwd_bwd", "steps": args.steps, "warmup": args.warmup, "ms": round(r["ms"], 4),
+                          "TFLOPs": round(r["flop"] / r["ms"] / 1e9, 1)}))
         return
     if args.moe_node:
         ms = bench_moe_node(args.moe_node == "ue8m0", args.steps, args.warmup)["ms"]

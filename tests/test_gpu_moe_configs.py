@@ -127,7 +127,9 @@ def _check_grouped_gemm(call, rows, what):
 
 
 def _check_quant_rows(x, q, s_kmajor, rows, pow2, what):
-    """Row-wise 1x128 quantization of bf16 x (scales stored [K/128, M]) on the slabs, bit-exact."""
+    """Row-wise 1x128 quantization of bf16 x (scales stored [K/128, M], fp32 or the UE8M0 bytes the quantizer wrote in
+    that mode) on the slabs, bit-exact."""
+    s_kmajor = _scales_f32(s_kmajor)
     for lo, _, label in _slab_tiles(rows):
         eq, es = O.quant_1x128(G.from_torch_bf16(x[lo:lo + 128]), 0, pow2=pow2)
         msg = G.mismatch_report(G.from_torch_fp8(q[lo:lo + 128]), eq, f"{what}, {label}: bytes")
@@ -229,7 +231,7 @@ def _check_forward(rec, node, x, probs, rows, pow2_in, tag):
         eq, es = O.swiglu_weighted_quant(G.from_torch_bf16(o1[lo:lo + 128]), probs[lo:lo + 128, 0].cpu().numpy(), 0, True)
         msg = G.mismatch_report(G.from_torch_fp8(o2q[lo:lo + 128]), eq, f"{tag} o2 bytes, {label}")
         assert not msg, msg
-        msg = G.mismatch_report(o2s[lo:lo + 128].cpu().numpy(), es, f"{tag} o2 scales, {label}")
+        msg = G.mismatch_report(_scales_f32(o2s)[lo:lo + 128].contiguous().cpu().numpy(), es, f"{tag} o2 scales, {label}")
         assert not msg, msg
     _check_grouped_gemm(gemms[1], rows, f"{tag} down")
     return o1
@@ -332,7 +334,7 @@ def test_config5_forward_backward_at_full_size(ue8m0):
     by_src = {("fp8" if c[1][0].dtype == torch.float8_e4m3fn else "bf16"): c for c in tsq}
     xt_q, xt_s = by_src["fp8"][3]
     assert by_src["fp8"][1][0] is x_fp8
-    _check_transposed(lambda e: (G.from_torch_fp8(seg(x_fp8, e)), seg(x_scale, e).contiguous().cpu().numpy()), xt_q, xt_s, rows,
+    _check_transposed(lambda e: (G.from_torch_fp8(seg(x_fp8, e)), seg(_scales_f32(x_scale), e).contiguous().cpu().numpy()), xt_q, xt_s, rows,
                       [small] + one, f"{tag} X^T from e4m3")
     o2t_q, o2t_s = by_src["bf16"][3]
     assert by_src["bf16"][1][0] is o2_s
