@@ -148,8 +148,9 @@ def bench_quantizers(iters=60, warmup=10):
         del sets
         torch.cuda.empty_cache()
 
-    # plain copies: the size of config 1's activation quantizer (89 MB moved) and of config 4's (477 MB)
-    for name, half in (("copy_yardstick_89MB", 44498944), ("copy_yardstick_477MB", 238551040)):
+    # plain copies: the size of config 1's weight quantizer (44 MB moved), of its activation quantizer (89 MB) and of
+    # config 4's (477 MB)
+    for name, half in (("copy_yardstick_44MB", 22021888), ("copy_yardstick_89MB", 44498944), ("copy_yardstick_477MB", 238551040)):
         run(name, 2 * half, max(4, (1 << 30) // (2 * half)), lambda h=half: (u8(h).random_(0, 255), u8(h)),
             lambda src, dst: _lib.call("pf8_debug_copy", p(src), p(dst), src.numel(), st))
     # C1a: 1x128 on [4096, 7168]
@@ -165,8 +166,9 @@ def bench_quantizers(iters=60, warmup=10):
     # C3-q: fused SwiGLU + requant on [8192, 4096]
     M, I = 8192, 2048
     for pow2 in (0, 1):
-        run("swiglu_quant_8192x4096" + ("_pow2" if pow2 else ""), 84443136 - 32768, 8, lambda: (bf((M, 2 * I)), u8(M, I), f32(M, I // 128)),
-            lambda o, q, s_, pw=pow2: _lib.call("pf8_swiglu_weighted_quant", p(o), None, M, I, p(q), p(s_), None, 0, pw, st))
+        run("swiglu_quant_8192x4096" + ("_pow2" if pow2 else ""), 84443136, 8,
+            lambda: (bf((M, 2 * I)), u8(M, I), f32(M, I // 128), torch.rand((M,), device="cuda")),
+            lambda o, q, s_, pr, pw=pow2: _lib.call("pf8_swiglu_weighted_quant", p(o), p(pr), M, I, p(q), p(s_), None, 0, pw, st))
     # C4: fused quant + transpose on [16384, 7168]
     M, K = 16384, 7168
     for pow2 in (0, 1):
