@@ -276,6 +276,22 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
             del w2fm
         del a2, w2, o3
     torch.cuda.empty_cache()
+    # beyond the tile table of the persistent plain-weight kernel (2,048 row tiles): config 5's up+gate shapes with 2,304
+    # row tiles (128 experts x 18 tiles), where that kernel walks the row tiles in plain groups of 16 instead of expert by
+    # expert; the fragment-major kernel reads the expert of every tile from m_indices and has no such table
+    Mb = 128 * 18 * 128
+    mib = torch.repeat_interleave(torch.arange(E, dtype=torch.int32), 18 * 128).cuda()
+    a, sa = qact(Mb, H)
+    w1, s1 = qweights(E, 2 * I, H)
+    o1 = torch.empty((Mb, 2 * I), dtype=torch.bfloat16, device="cuda")
+    big_it, big_w = max(4, iters // 4), max(1, warmup // 4)
+    out["grouped_up_gate_2304_row_tiles"] = dict(tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa.T), (w1, s1), o1, mib), big_it, big_w),
+                                                 flop=2.0 * Mb * H * 2 * I, padded_rows=Mb)
+    w1fm = deep_gemm.to_fragment_major(w1)
+    out["grouped_up_gate_2304_row_tiles_fragment_major"] = dict(
+        tkern(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((a, sa.T), (w1fm, s1), o1, mib), big_it, big_w), flop=2.0 * Mb * H * 2 * I, padded_rows=Mb)
+    del a, sa, w1, s1, w1fm, o1, mib
+    torch.cuda.empty_cache()
     # config 5 weight gradient dW1[e] [H, 2I] += x_e^T . do1_e, all experts in one launch
     rows = [int(r) for r in padded]
     x = torch.randn((Mp, H), device="cuda").to(torch.bfloat16)
@@ -766,6 +782,9 @@ def main():
 
     o1 = torch.empty((Mpad, 2 * I), dtype=torch.bfloat16, device="cuda")
     o3 = torch.empty((Mpad, H), dtype=torch.bfloat16, device="cuda")
+    # routing probability of every row (zero on padding rows), applied between SwiGLU and the requantization as the
+    # reference's forward does (transformers/fp8_utils.py:965-987)
+    probs = torch.rand((Mpad,), device="cuda") * (x.float().abs().amax(dim=1) > 0)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
 
     def step(evs=None, w1=w1fm, w2=w2fm):
@@ -775,7 +794,7 @@ def main():
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((xq, xs.T), (w1, w1s), o1, m_idx)
         if evs: evs[2].record()
         # power-of-two scales for the requantised activation, as the reference's fused node asks (transformers/fp8_utils.py:984-986)
-        o2q, o2s = F8.fused_weighted_swiglu_act_quant(o1, None, using_pow2_scaling=True)
+        o2q, o2s = F8.fused_weighted_swiglu_act_quant(o1, probs, using_pow2_scaling=True)
         if evs: evs[3].record()
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2, w2s), o3, m_idx)
         if evs: evs[4].record()
@@ -788,7 +807,7 @@ def main():
         """The same forward with SwiGLU and the requantization in the up+gate GEMM's epilogue (one launch, bit-identical
         o2; the bf16 o1 is never written: what the node does when recompute_fwd_gate_up makes o1 disposable)."""
         xq, xs = F8.fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True)
-        o2q, o2s = deep_gemm.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((xq, xs.T), (w1q, w1s), m_idx, None, using_pow2_scaling=True)
+        o2q, o2s = deep_gemm.m_grouped_fp8_gemm_nt_contiguous_swiglu_quant((xq, xs.T), (w1q, w1s), m_idx, probs, using_pow2_scaling=True)
         deep_gemm.m_grouped_fp8_gemm_nt_contiguous((o2q, o2s), (w2fm, w2s), o3, m_idx)
 
     def timed(fn, n):

@@ -113,6 +113,9 @@ def test_tokens_through_unzip_node_experts_zip_node_and_back(fp8_tokens):
     ref_y, ref_dx, ref_dp, ref_dw1, ref_dw2 = _fp32_layer(x, rm, probs, w1, w2, dy)
     errs = {"y": G.rel_fro(y.float().cpu().numpy(), ref_y), "dx": G.rel_fro(dx.float().cpu().numpy(), ref_dx)}
     print("layer errors vs fp32:", errs)
+    # measured on MI355X: 0.065 for y and for dx (the e4m3 rounding of two GEMM operands in a row; inputs, weights and
+    # routing all come from the seeds above).  The bar is 1.4 times that: a dropped probability factor, a wrong expert or
+    # a missing copy in the sum moves these errors to 0.3 and beyond.
     tol = 0.09
     assert G.rel_fro(y.float().cpu().numpy(), ref_y) < tol
     assert G.rel_fro(dx.float().cpu().numpy(), ref_dx) < tol
