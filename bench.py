@@ -51,7 +51,7 @@ def traffic_from_summary(kernel_name):
 
 
 # the kernel the up+gate grouped GEMM of the headline workload runs on (what rocprofv3 --kernel-trace names it)
-ROOFLINE_KERNEL = "pf8::k_gemm_fm<1, 0>"
+ROOFLINE_KERNEL = "pf8::k_gemm_fm<1, 0, 0>"
 
 
 def zipf_counts(total, E, s, seed, n_empty=2, pad=128):
