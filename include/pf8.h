@@ -235,7 +235,7 @@ int pf8_grouped_gemm_nt_contiguous(const uint8_t* a, const float* sa, int sa_lay
  * N multiple of 64, K multiple of 128. */
 int pf8_weight_to_fragment_major(const uint8_t* w, int E, int64_t N, int64_t K, uint8_t* wf, pf8_stream_t stream);
 
-/* 1 when the *_fm GEMMs take this shape (M % 128 == 0, N % 256 == 0, K % 128 == 0, K >= 384), else 0.  No device access. */
+/* 1 when the *_fm GEMMs take this shape (M % 128 == 0, N % 128 == 0 and N >= 256, K % 128 == 0, K >= 384), else 0.  No device access. */
 int pf8_gemm_fm_supported(int64_t M, int64_t N, int64_t K);
 
 /* deep_gemm.fp8_gemm_nt / m_grouped_fp8_gemm_nt_contiguous (transformers/fp8_utils.py:289-302, 949-954, 1002-1007) on a

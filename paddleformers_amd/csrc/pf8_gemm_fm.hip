@@ -47,7 +47,7 @@
 //     MFMAs of the next block, and a tile's very last behind an explicit wait.
 //   * Epilogue: each wavefront stages 32 rows x 64 columns of bf16 at a time in a private LDS slice and stores
 //     128-byte row pieces.
-// Needs Prows % 256 == 0, Qrows % 128 == 0 and K % 128 == 0, K >= 384; dense and contiguous-grouped layouts.
+// Needs Prows % 128 == 0 and Prows >= 256, Qrows % 128 == 0 and K % 128 == 0, K >= 384; dense and contiguous-grouped layouts.
 #include <atomic>
 
 #include "pf8_gemm_common.h"
@@ -104,7 +104,9 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int x = lane & 31, hh = lane >> 5;
 
-    const int64_t p_tiles = a.Prows / 256, q_tiles = a.Qrows / BQ;
+    // a last column tile may be half new (Prows = 256 t + 128): it covers the LAST 256 weight rows, and the two wavefronts
+    // that repeat the previous tile's columns store nothing
+    const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = a.Qrows / BQ;
     const int64_t KB = a.red / 128, PB = a.Prows / 128, P64 = a.Prows / 64;
     const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, W = gridDim.x >> 3;
     const bool grouped = a.grouped != 0;
@@ -216,8 +218,8 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
     // 32 w + 4 (lane >> 3) + c), of the token row whose scales its scale copy fetches (tile row 64 w + lane, wavefronts 0 / 1)
     // and which of the four rows it accumulates for (tile rows 4 x .. 4 x + 3) are real; c_* current tile, n_* next
     uint32_t c_qoff[4] = {0, 0, 0, 0}, n_qoff[4] = {0, 0, 0, 0}, c_svoff = 0, n_svoff = 0;
-    float c_live[4] = {1.f, 1.f, 1.f, 1.f}, n_live[4] = {1.f, 1.f, 1.f, 1.f};
-    auto gather_setup = [&](int64_t qt, uint32_t (&qoff)[4], uint32_t& svoff, float (&live)[4]) {
+    uint32_t c_live = 15u, n_live = 15u;          // bit t: the lane's accumulate row t of the tile is a token (not a padding row)
+    auto gather_setup = [&](int64_t qt, uint32_t (&qoff)[4], uint32_t& svoff, uint32_t& live) {
         const int32_t* m = a.src_row + qt * BQ;
         const int4 rc = *reinterpret_cast<const int4*>(m + 32 * wave + 4 * crow);
         const int4 rl = *reinterpret_cast<const int4*>(m + 4 * x);
@@ -226,8 +228,8 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             qoff[c] = (uint32_t)(rcv[c] < 0 ? 0 : rcv[c]) * (uint32_t)a.red + q_chunk;     // a padding row reads token 0: finite bytes, zero factor
-            live[c] = rlv[c] < 0 ? 0.f : 1.f;
         }
+        live = (rlv[0] < 0 ? 0u : 1u) | (rlv[1] < 0 ? 0u : 2u) | (rlv[2] < 0 ? 0u : 4u) | (rlv[3] < 0 ? 0u : 8u);
         if (wave < 2) svoff = (uint32_t)(rs < 0 ? 0 : rs) * (uint32_t)(KB * 4);
     };
     auto setup = [&](int64_t qt, int64_t pt, const uint8_t*& pp, const uint8_t*& qp, const uint8_t*& sp_, int& store) {
@@ -235,10 +237,12 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
         store = e >= 0;
         if (e < 0) e = 0;                  // a padding tile is computed on expert 0's weights and not stored
         if constexpr (TRACE & 64) { pt = 0; qt = 0; e = 0; }        // timing experiment: every tile reads the operands of tile (0, 0)
-        pp = a.pf + (((int64_t)e * P64 + pt * 4 + wave) * KB) * 8192;
+        const int64_t p0 = pt * 256 + 256 <= a.Prows ? pt * 256 : a.Prows - 256;       // first weight row of the tile
+        if (pt * 256 != p0 && wave < 2) store = 0;
+        pp = a.pf + (((int64_t)e * P64 + p0 / 64 + wave) * KB) * 8192;
         qp = GATHER ? a.q : a.q + qt * BQ * a.red;
         if (wave < 2) sp_ = reinterpret_cast<const uint8_t*>(GATHER ? a.sq : a.sq + (SQL == 1 ? qt * BQ : qt * BQ * KB));
-        else sp_ = reinterpret_cast<const uint8_t*>(a.sp + ((int64_t)e * PB + pt * 2) * KB);
+        else sp_ = reinterpret_cast<const uint8_t*>(a.sp + ((int64_t)e * PB + p0 / 128) * KB);
     };
     setup(cq, cp, c_p, c_q, c_s, c_store);
     if constexpr (GATHER) gather_setup(cq, c_qoff, c_svoff, c_live);
@@ -338,7 +342,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
         }
         float fq_cur[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) fq_cur[t] = GATHER ? sq_nxt[t] * sp_nxt * c_live[t] : sq_nxt[t] * sp_nxt;
+        for (int t = 0; t < 4; ++t) fq_cur[t] = GATHER && !((c_live >> t) & 1u) ? 0.f : sq_nxt[t] * sp_nxt;
         const int64_t k2 = kb + 2;
         const bool in2 = k2 < KB;
         const int64_t kk = in2 ? k2 : k2 - KB;
@@ -427,7 +431,8 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
             const int lane_e = tid_e & 63, x_e = lane_e & 31, hh_e = lane_e >> 5;
             uint8_t* ep = lds + EP_OFS + wave * (32 * EP_LD);
             const int er = lane_e >> 3, ec = lane_e & 7;
-            uint8_t* tile_out = reinterpret_cast<uint8_t*>(a.out) + ((cq * BQ) * a.ldo + cp * 256 + wave * 64 + ec * 8) * 2;
+            const int64_t p0_e = cp * 256 + 256 <= a.Prows ? cp * 256 : a.Prows - 256;
+            uint8_t* tile_out = reinterpret_cast<uint8_t*>(a.out) + ((cq * BQ) * a.ldo + p0_e + wave * 64 + ec * 8) * 2;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -455,7 +460,8 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
         cq = nq; cp = np; c_p = n_p; c_q = n_q; c_s = n_s; c_store = n_store;
         if constexpr (GATHER) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) { c_qoff[c] = n_qoff[c]; c_live[c] = n_live[c]; }
+            for (int c = 0; c < 4; ++c) c_qoff[c] = n_qoff[c];
+            c_live = n_live;
             c_svoff = n_svoff;
         }
         return false;
@@ -521,7 +527,7 @@ extern "C" int pf8_weight_to_fragment_major(const uint8_t* w, int E, int64_t N, 
 }
 
 extern "C" int pf8_gemm_fm_supported(int64_t M, int64_t N, int64_t K) {
-    return M > 0 && M % 128 == 0 && N >= 256 && N % 256 == 0 && K >= 384 && K % 128 == 0;
+    return M > 0 && M % 128 == 0 && N >= 256 && N % 128 == 0 && K >= 384 && K % 128 == 0;
 }
 
 static int launch_fm(const char* where, const uint8_t* a, const float* sa, int sa_layout, const uint8_t* wf, const float* sb, int E,
@@ -532,7 +538,7 @@ static int launch_fm(const char* where, const uint8_t* a, const float* sa, int s
     FmArgs g = {};
     g.pf = wf; g.q = a; g.sp = sb; g.sq = sa; g.out = out;
     g.Prows = N; g.Qrows = M; g.red = K; g.ldo = ldo; g.grouped = m_indices != nullptr; g.E = E; g.m_indices = m_indices;
-    const int64_t T = (N / 256) * (M / 128), per_xcd = (T + 7) / 8;
+    const int64_t T = ((N + 255) / 256) * (M / 128), per_xcd = (T + 7) / 8;
     if (T > 0x7FFFFFFF) return pf8_fail(PF8_EINVAL, where, "too many tiles");
     int64_t w = pf8_effective_cus() / 8;
     if (w < 1) w = 1;
@@ -568,7 +574,7 @@ extern "C" int pf8_gemm_nt_fm(const uint8_t* a, const float* sa, int sa_layout, 
                               int64_t K, uint16_t* out, int64_t ldo, pf8_stream_t stream) {
     PF8_REQUIRE(M >= 0 && N >= 0 && K >= 0, "negative shape");
     if (M == 0 || N == 0) return PF8_OK;
-    PF8_REQUIRE(pf8_gemm_fm_supported(M, N, K), "needs M % 128 == 0, N % 256 == 0, K % 128 == 0 and K >= 384");
+    PF8_REQUIRE(pf8_gemm_fm_supported(M, N, K), "needs M % 128 == 0, N % 128 == 0, N >= 256, K % 128 == 0 and K >= 384");
     PF8_REQUIRE(a && sa && b_fm && sb && out, "null pointer");
     PF8_REQUIRE(ldo >= N && ldo % 8 == 0, "ldo must be >= N and a multiple of 8");
     PF8_REQUIRE(PF8_ALIGNED16(a) && PF8_ALIGNED16(b_fm) && PF8_ALIGNED16(out), "pointers must be 16-byte aligned");
@@ -582,7 +588,7 @@ extern "C" int pf8_grouped_gemm_nt_contiguous_fm(const uint8_t* a, const float* 
                                                  pf8_stream_t stream) {
     PF8_REQUIRE(E >= 0 && Mtot >= 0 && N >= 0 && K >= 0, "negative shape");
     if (Mtot == 0 || N == 0 || E == 0) return PF8_OK;
-    PF8_REQUIRE(pf8_gemm_fm_supported(Mtot, N, K), "needs Mtot % 128 == 0, N % 256 == 0, K % 128 == 0 and K >= 384");
+    PF8_REQUIRE(pf8_gemm_fm_supported(Mtot, N, K), "needs Mtot % 128 == 0, N % 128 == 0, N >= 256, K % 128 == 0 and K >= 384");
     PF8_REQUIRE(a && sa && b_fm && sb && out && m_indices, "null pointer");
     PF8_REQUIRE(PF8_ALIGNED16(a) && PF8_ALIGNED16(b_fm) && PF8_ALIGNED16(out), "pointers must be 16-byte aligned");
     PF8_REQUIRE(sa_layout == 0 || sa_layout == 1, "sa_layout must be 0 or 1");
@@ -593,7 +599,7 @@ extern "C" int pf8_grouped_gemm_nt_contiguous_fm(const uint8_t* a, const float* 
 extern "C" int pf8_debug_grouped_gemm_fm_cycles(const uint8_t* a, const float* sa, const uint8_t* b_fm, const float* sb, int E, int64_t Mtot,
                                                 int64_t N, int64_t K, const int32_t* m_indices, uint16_t* out, int64_t* cycles,
                                                 int64_t workgroups, int ablate, pf8_stream_t stream) {
-    PF8_REQUIRE(E > 0 && pf8_gemm_fm_supported(Mtot, N, K), "needs Mtot % 128 == 0, N % 256 == 0, K % 128 == 0 and K >= 384");
+    PF8_REQUIRE(E > 0 && pf8_gemm_fm_supported(Mtot, N, K), "needs Mtot % 128 == 0, N % 128 == 0, N >= 256, K % 128 == 0 and K >= 384");
     PF8_REQUIRE(a && sa && b_fm && sb && out && m_indices && cycles, "null pointer");
     PF8_REQUIRE(PF8_ALIGNED16(a) && PF8_ALIGNED16(b_fm) && PF8_ALIGNED16(out), "pointers must be 16-byte aligned");
     return launch_fm(__func__, a, sa, 1, b_fm, sb, E, Mtot, N, K, m_indices, out, N, stream, cycles, workgroups, ablate);
@@ -604,7 +610,7 @@ extern "C" int pf8_grouped_gemm_nt_contiguous_fm_gather(const uint8_t* tokens, c
                                                         const int32_t* m_indices, uint16_t* out, pf8_stream_t stream) {
     PF8_REQUIRE(E >= 0 && Mtot >= 0 && N >= 0 && K >= 0 && T >= 0, "negative shape");
     if (Mtot == 0 || N == 0 || E == 0) return PF8_OK;
-    PF8_REQUIRE(pf8_gemm_fm_supported(Mtot, N, K), "needs Mtot % 128 == 0, N % 256 == 0, K % 128 == 0 and K >= 384");
+    PF8_REQUIRE(pf8_gemm_fm_supported(Mtot, N, K), "needs Mtot % 128 == 0, N % 128 == 0, N >= 256, K % 128 == 0 and K >= 384");
     PF8_REQUIRE(T > 0 && tokens && token_scales && src_row && b_fm && sb && out && m_indices, "null pointer");
     PF8_REQUIRE(PF8_ALIGNED16(tokens) && PF8_ALIGNED16(b_fm) && PF8_ALIGNED16(out) && PF8_ALIGNED16(src_row), "pointers must be 16-byte aligned");
     PF8_REQUIRE(K <= (1ll << 24) && T * K < (1ll << 31), "the token matrix must stay below 2 GiB");

@@ -43,7 +43,8 @@ class FragmentMajor:
 
 
 def fragment_major_supported(M: int, N: int, K: int) -> bool:
-    """Shapes the fragment-major kernels take (whole 128-row and 256-column tiles, at least three K blocks)."""
+    """Shapes the fragment-major kernels take (whole 128-row tiles, 256-column tiles of which the last may be half new, at
+    least three K blocks)."""
     return bool(_lib.lib().pf8_gemm_fm_supported(int(M), int(N), int(K)))
 
 
@@ -142,7 +143,7 @@ def fp8_gemm_nt(a, b, out: torch.Tensor, c: Optional[torch.Tensor] = None, recip
     fm = isinstance(tb, FragmentMajor)
     if fm and (recipe is not None or c is not None or _is_ue8m0(sa) or _is_ue8m0(sb) or not fragment_major_supported(M, N, K)
                or out.dtype != torch.bfloat16 or out.stride(-1) != 1 or out.stride(0) % 8 != 0 or out.data_ptr() % 16 != 0):
-        raise ValueError("a fragment-major weight serves the default recipe with fp32 scales, M % 128 == 0, N % 256 == 0, K % 128 == 0, K >= 384")
+        raise ValueError("a fragment-major weight serves the default recipe with fp32 scales, M % 128 == 0, N % 128 == 0, N >= 256, K % 128 == 0, K >= 384")
     ta = ta if ta.is_contiguous() else ta.contiguous()
     if fm:
         sa, lay = _scale_layout_of(sa, M, K // 128, "a scale")
@@ -244,7 +245,7 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
         return out
     if isinstance(tb, FragmentMajor):
         if _is_ue8m0(sa) or _is_ue8m0(sb) or not fragment_major_supported(Mtot, N, K):
-            raise ValueError("a fragment-major weight serves fp32 scales, Mtot % 128 == 0, N % 256 == 0, K % 128 == 0, K >= 384")
+            raise ValueError("a fragment-major weight serves fp32 scales, Mtot % 128 == 0, N % 128 == 0, N >= 256, K % 128 == 0, K >= 384")
         sa, lay = _scale_layout_of(sa, Mtot, K // 128, "a scale")
         if tuple(sb.shape) != (E, N // 128, K // 128) or sb.dtype != torch.float32:
             raise ValueError(f"b scale must be float32 [{E}, {N // 128}, {K // 128}]")

@@ -97,7 +97,8 @@ def _weights(E, N, K, seed):
     return np.stack(bs), np.stack(sbs)
 
 
-@pytest.mark.parametrize("T,K,N,topk,E", [(300, 512, 512, 2, 5), (1000, 384, 256, 3, 4), (700, 1408, 768, 4, 8), (90, 1024, 512, 1, 6)])
+@pytest.mark.parametrize("T,K,N,topk,E", [(300, 512, 512, 2, 5), (1000, 384, 256, 3, 4), (700, 1408, 768, 4, 8), (90, 1024, 512, 1, 6),
+                                         (400, 512, 640, 2, 3)])
 @pytest.mark.parametrize("cus", [0, 16])
 def test_grouped_gemm_reads_through_the_source_map(F, T, K, N, topk, E, cus):
     from paddleformers_amd import deep_gemm as dg

@@ -57,7 +57,8 @@ def _dense_case(M, N, K, seed):
     return a, sa, b, sb
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 256, 384), (128, 256, 512), (384, 512, 1024), (256, 768, 2048), (1280, 256, 640), (256, 256, 1408)])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 384), (128, 256, 512), (384, 512, 1024), (256, 768, 2048), (1280, 256, 640), (256, 256, 1408),
+                                   (256, 384, 512), (384, 1408, 640), (128, 640, 384)])          # the last three: a half last column tile
 @pytest.mark.parametrize("lay", [0, 1])
 def test_dense_fragment_major_against_oracle_and_plain_kernel(dg, M, N, K, lay):
     a, sa, b, sb = _dense_case(M, N, K, seed=M + N + K)
@@ -112,8 +113,9 @@ def _grouped_case(E, N, K, blocks, seed):
 ])
 @pytest.mark.parametrize("lay", [0, 1])
 @pytest.mark.parametrize("cus", [0, 16])
-def test_grouped_fragment_major_against_oracle_and_plain_kernel(dg, K, blocks, lay, cus):
-    E, N = 4, 512
+@pytest.mark.parametrize("N", [512, 384])
+def test_grouped_fragment_major_against_oracle_and_plain_kernel(dg, K, blocks, lay, cus, N):
+    E = 4
     a, sa, b, sb, m_idx = _grouped_case(E, N, K, blocks, seed=K + len(blocks))
     Mtot = a.shape[0]
     ta, tb = G.to_torch_fp8(a), G.to_torch_fp8(b)
@@ -143,7 +145,8 @@ def test_fragment_major_rejects_other_shapes_and_scales(dg):
     tsa, tsb = torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda()
     fm = dg.to_fragment_major(tb)
     assert dg.fragment_major_supported(128, 256, 512) and dg.fragment_major_supported(128, 256, 384)
-    assert not dg.fragment_major_supported(128, 384, 512) and not dg.fragment_major_supported(128, 256, 256)
+    assert dg.fragment_major_supported(128, 384, 512) and not dg.fragment_major_supported(128, 320, 512)
+    assert not dg.fragment_major_supported(128, 128, 512) and not dg.fragment_major_supported(128, 256, 256)
     assert not dg.fragment_major_supported(100, 256, 512)
     with pytest.raises(ValueError):                             # K = 256: fewer than three K blocks
         dg.fp8_gemm_nt((ta[:, :256].contiguous(), tsa[:, :2].contiguous()),

@@ -553,7 +553,7 @@ def test_moe_node_reads_fragment_major_copies_of_the_cached_weights():
     the plain-weight kernels, and a replaced cache entry is picked up."""
     from paddleformers_amd import fp8_utils as U
 
-    E, H, I = 3, 512, 384                    # 2I = 768 and H = 512 are multiples of 256; I = 384 is not (dgrad-down stays plain)
+    E, H, I = 3, 512, 384                    # 2I = 768 and H = 512 are whole 256-column tiles; I = 384 ends in a half tile (dgrad-down)
     rows = [256, 0, 384]
     _, _, experts, x, probs = _make(E, H, I, rows, seed=41)
     dout = G.bf16_normal((sum(rows), H), seed=42, std=1e-3)
@@ -580,7 +580,7 @@ def test_moe_node_reads_fragment_major_copies_of_the_cached_weights():
     kept = w0.fp8_weight_stacked_transpose_fragment_major
     assert kept[0] is w0.fp8_weight_stacked_transpose and isinstance(kept[2], U.deep_gemm.FragmentMajor)
     assert hasattr(v0, "fp8_weight_stacked_transpose_fragment_major") and hasattr(w0, "fp8_weight_stacked_fragment_major")
-    assert not hasattr(v0, "fp8_weight_stacked_fragment_major")          # [E, I, H] with I = 384: not a shape the kernel takes
+    assert hasattr(v0, "fp8_weight_stacked_fragment_major")              # [E, I, H] with I = 384: a whole tile and a half one
     run(True)
     assert w0.fp8_weight_stacked_transpose_fragment_major is kept        # made once
     # a new cache entry (next optimizer step) is another tensor: its copy replaces the old one
