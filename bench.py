@@ -350,7 +350,6 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     # readers of the unzipped tokens (up+gate grouped GEMM, transposed quantizer of the weight gradient) on the copied rows
     # and through the map
     xq, xs = F8.fp8_quant_blockwise(xt, quant_method="1x128")
-    del xt
     ms = time_kernel(lambda: F8.moe_permute(xq, xs, rm_t, pr_t, Et, cnts, 128), [()], 20, 3)
     cq, _, _, cs = F8.moe_permute(xq, xs, rm_t, pr_t, Et, cnts, 128)
     Mp5 = cq.shape[0]
@@ -366,7 +365,8 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     midx5 = torch.repeat_interleave(torch.arange(Et, dtype=torch.int32), torch.tensor(pad5)).cuda()
     o15 = torch.empty((Mp5, N5), dtype=torch.bfloat16, device="cuda")
     flop5 = 2.0 * Tt * tk * Ht * N5
-    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((cq, cs), (wfm5, ws5), o15, midx5), [()], iters, warmup)
+    cs_k = cs.t().contiguous().t()          # scales stored [H/128, rows], as the node hands them to the GEMM
+    ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((cq, cs_k), (wfm5, ws5), o15, midx5), [()], iters, warmup)
     out["grouped_config5_up_gate_fragment_major_copied_rows"] = dict(ms, flop=flop5)
     ms = time_kernel(lambda: deep_gemm.m_grouped_fp8_gemm_nt_contiguous((gq, None), (wfm5, ws5), o15, midx5), [()], iters, warmup)
     out["grouped_config5_up_gate_fragment_major_through_row_map"] = dict(ms, flop=flop5)
@@ -375,6 +375,15 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     out["transpose_split_quant_fp8_config5_copied_rows"] = dict(ms, bytes=tsq_bytes)
     ms = time_kernel(lambda: F8.fused_transpose_split_quant(gq, None, pad5, True), [()], 20, 3)
     out["transpose_split_quant_fp8_config5_through_row_map"] = dict(ms, bytes=tsq_bytes)
+    # the gradient side: bf16 tokens copied into expert order and quantized (row-wise and transposed, one read), against
+    # the tokens quantized row-wise once and the transposed copy quantized through the row map
+    cb = F8.moe_permute(xt, None, rm_t, pr_t, Et, cnts, 128)[0]
+    gb = F8.moe_permute(xt, None, rm_t, pr_t, Et, cnts, 128, do_gather=False)[0]
+    ms = time_kernel(lambda: F8.quant_and_transpose_split(cb, pad5, False, True), [()], 20, 3)
+    out["quant_and_transpose_split_bf16_config5_copied_rows"] = dict(ms, bytes=Mp5 * Ht * 4 + 2 * Mp5 * (Ht // 128) * 4)
+    ms = time_kernel(lambda: (gb.quantize(False), F8.fused_transpose_split_quant(gb, None, pad5, True)), [()], 20, 3)
+    out["quantize_tokens_and_transpose_split_bf16_config5_through_row_map"] = dict(ms, bytes=Tt * Ht * 3 + Mp5 * Ht * 3)
+    del xt, cb, gb
     del xq, xs, cq, cs, gq, wfm5, ws5, o15, midx5
     torch.cuda.empty_cache()
     # the RMSNorm the dense FP8 MLP recomputes: forward and backward on [16384, 7168] bf16

@@ -107,13 +107,14 @@ int pf8_transpose_split_quant(const void* x, const float* xs, int x_is_fp8, int 
                               const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q_t, float* s_t,
                               int pow2, pf8_stream_t stream);
 
-/* pf8_transpose_split_quant of an e4m3 input with UnZipNode.forward's row copy folded into the read: row r of the
- * expert-sorted input is row src_row[r] of tokens [T, K] with that row's scales (xs_layout 0 = [T, K/128], 1 = [K/128, T]);
- * src_row[r] < 0 is a row of zeros.  src_row int32 [sum rows_per_expert], entries below T.  Outputs bit-identical to
+/* pf8_transpose_split_quant with the row copy of UnZipNode.forward / ZipNode.backward (moe_utils.py:141-186, 217-261)
+ * folded into the read: row r of the expert-sorted input is row src_row[r] of tokens [T, K] -- bf16 (x_is_fp8 = 0), or
+ * e4m3 with that row's scales (xs_layout 0 = [T, K/128], 1 = [K/128, T], 2 = UE8M0 bytes [K/128, T]); src_row[r] < 0 is a
+ * row of zeros.  src_row int32 [sum rows_per_expert], 16-byte aligned, entries below T.  Outputs bit-identical to
  * pf8_transpose_split_quant on the rows pf8_moe_permute copies out. */
-int pf8_transpose_split_quant_gather(const uint8_t* tokens, const float* token_scales, int xs_layout, int64_t T,
-                                     const int32_t* src_row, const int64_t* rows_per_expert, int E, int64_t K,
-                                     uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream);
+int pf8_transpose_split_quant_gather(const void* tokens, const float* token_scales, int x_is_fp8, int xs_layout,
+                                     int64_t T, const int32_t* src_row, const int64_t* rows_per_expert, int E,
+                                     int64_t K, uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream);
 
 /* The two quantizations the MoE node's backward applies to the SAME bf16 gradient, from one read:
  * fp8_quant_blockwise(x, quant_method="1x128", output_scale_transpose=True, using_pow2_scale=pow2_rows)
@@ -250,15 +251,21 @@ int pf8_grouped_gemm_nt_contiguous_fm(const uint8_t* a, const float* sa, int sa_
                                       const float* sb, int E, int64_t Mtot, int64_t N, int64_t K,
                                       const int32_t* m_indices, uint16_t* out, pf8_stream_t stream);
 
-/* pf8_grouped_gemm_nt_contiguous_fm with UnZipNode.forward's row copy (moe_utils.py:141-186) folded into the read of the
- * activation operand: row r of the expert-sorted operand is row src_row[r] of tokens [T, K] (e4m3) with the scales of that
- * row of token_scales [T, K/128] (fp32, row-major); src_row[r] < 0 (see pf8_moe_permute_map) is a row of zeros.  out is
- * bit-identical to pf8_grouped_gemm_nt_contiguous_fm on the rows pf8_moe_permute copies out.  src_row: int32 [Mtot],
- * 16-byte aligned, every entry below T; tokens below 2 GiB. */
-int pf8_grouped_gemm_nt_contiguous_fm_gather(const uint8_t* tokens, const float* token_scales, int64_t T,
-                                             const int32_t* src_row, const uint8_t* b_fm, const float* sb, int E,
-                                             int64_t Mtot, int64_t N, int64_t K, const int32_t* m_indices,
-                                             uint16_t* out, pf8_stream_t stream);
+/* pf8_grouped_gemm_nt_contiguous_fm with the row copy of UnZipNode.forward / ZipNode.backward (moe_utils.py:141-186,
+ * 217-261) folded into the read of the activation operand: row r of the expert-sorted operand is row src_row[r] of
+ * tokens [T, K] (e4m3); src_row[r] < 0 (see pf8_moe_permute_map) is a row of zeros.  sa holds the scales of the
+ * EXPERT-SORTED rows, [Mtot, K/128] in either layout, as pf8_gather_row_scales makes them from the token scales (zero
+ * for a negative src_row).  out is bit-identical to pf8_grouped_gemm_nt_contiguous_fm on the rows pf8_moe_permute copies
+ * out.  src_row: int32 [Mtot], 16-byte aligned, every entry below T; tokens below 2 GiB. */
+int pf8_grouped_gemm_nt_contiguous_fm_gather(const uint8_t* tokens, int64_t T, const int32_t* src_row, const float* sa,
+                                             int sa_layout, const uint8_t* b_fm, const float* sb, int E, int64_t Mtot,
+                                             int64_t N, int64_t K, const int32_t* m_indices, uint16_t* out,
+                                             pf8_stream_t stream);
+
+/* out[r, kb] = xs[src_row[r], kb] (0 for a negative src_row): the 1x128 scales of rows that are read through a source map,
+ * gathered on their own.  xs fp32 [T, KB] row-major; out [rows, KB] row-major (out_layout 0) or [KB, rows] (1). */
+int pf8_gather_row_scales(const float* xs, int64_t T, int64_t KB, const int32_t* src_row, int64_t rows, float* out,
+                          int out_layout, pf8_stream_t stream);
 
 /* The up+gate grouped GEMM with the activation quantizer of the down projection in its epilogue: the two calls of
  * FP8GroupGemmMlpFunctionNode.forward -- deep_gemm.m_grouped_fp8_gemm_nt_contiguous (transformers/fp8_utils.py:949-954)

@@ -28,7 +28,7 @@ SIGNATURES = {
     "pf8_stack_quant_both": [_vp, _i32, _i64, _i64, _vp, _vp, _vp, _vp, _i32, _vp],
     "pf8_swiglu_weighted_quant": [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i32, _i32, _vp],
     "pf8_transpose_split_quant": [_vp, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp, _i32, _vp],
-    "pf8_transpose_split_quant_gather": [_vp, _vp, _i32, _i64, _vp, _vp, _i32, _i64, _vp, _vp, _i32, _vp],
+    "pf8_transpose_split_quant_gather": [_vp, _vp, _i32, _i32, _i64, _vp, _vp, _i32, _i64, _vp, _vp, _i32, _vp],
     "pf8_quant_and_transpose_split": [_vp, _vp, _i32, _i64, _vp, _vp, _i32, _vp, _vp, _i32, _vp],
     "pf8_act_dequant": [_vp, _vp, _i32, _i64, _i64, _vp, _vp],
     "pf8_weight_dequant": [_vp, _vp, _i64, _i64, _vp, _vp],
@@ -47,7 +47,8 @@ SIGNATURES = {
     "pf8_gemm_fm_supported": [_i64, _i64, _i64],
     "pf8_gemm_nt_fm": [_vp, _vp, _i32, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
     "pf8_grouped_gemm_nt_contiguous_fm": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp],
-    "pf8_grouped_gemm_nt_contiguous_fm_gather": [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp],
+    "pf8_grouped_gemm_nt_contiguous_fm_gather": [_vp, _i64, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp],
+    "pf8_gather_row_scales": [_vp, _i64, _i64, _vp, _i64, _vp, _i32, _vp],
     "pf8_grouped_gemm_swiglu_quant_nt_contiguous": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i32, _vp],
     "pf8_gemm_nt_ue8m0": [_vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
     "pf8_grouped_gemm_nt_contiguous_ue8m0": [_vp, _vp, _i64, _vp, _vp, _i32, _i64, _i64, _i64, _vp, _vp, _vp, _vp],

@@ -66,8 +66,9 @@ struct FmArgs {
     int64_t Prows, Qrows, red, ldo;
     int grouped, E;
     const int32_t* m_indices;
-    // GATHER instantiation: q is the token matrix [T, red], sq its scales [T, KB] (sq_layout 0) and output row r multiplies
-    // token src_row[r] (negative = a padding row: its output is zero); Qrows counts output rows
+    // GATHER instantiation: q is the token matrix [T, red] and output row r multiplies token src_row[r]; sq holds the scales
+    // of the OUTPUT rows (gathered beforehand: 4 bytes per row and K block against 128), zero for a row whose src_row is
+    // negative (a padding row: it reads token 0's bytes with a zero factor, its output is zero); Qrows counts output rows
     const int32_t* src_row;
     int64_t* cycles;       // TRACE instantiation only: [workgroups][8] cycle sums of wavefront 0 (see pf8_debug_grouped_gemm_fm_cycles)
 };
@@ -94,7 +95,6 @@ __device__ __forceinline__ void fm_mfma_second(f32x16& d, const i32x8& q) {
 
 template <int SQL, int TRACE = 0, int GATHER = 0>
 __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
-    static_assert(!GATHER || SQL == 0, "gathered tokens carry row-major scales");
     constexpr int BQ = 128;
     constexpr int STAGE = kFmStage, S_OFS = 16384, SP_OFS = 16384 + 512, EP_OFS = kFmStages * kFmStage, EP_LD = kFmEpLd;
     constexpr int BAR = 12;
@@ -215,22 +215,13 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
     int c_store, n_store = 0;
     bool n_valid = false;
     // GATHER: per tile and lane, the byte offsets of the four token rows its activation copies fetch (copy c: tile row
-    // 32 w + 4 (lane >> 3) + c), of the token row whose scales its scale copy fetches (tile row 64 w + lane, wavefronts 0 / 1)
-    // and which of the four rows it accumulates for (tile rows 4 x .. 4 x + 3) are real; c_* current tile, n_* next
-    uint32_t c_qoff[4] = {0, 0, 0, 0}, n_qoff[4] = {0, 0, 0, 0}, c_svoff = 0, n_svoff = 0;
-    uint32_t c_live = 15u, n_live = 15u;          // bit t: the lane's accumulate row t of the tile is a token (not a padding row)
-    auto gather_setup = [&](int64_t qt, uint32_t (&qoff)[4], uint32_t& svoff, uint32_t& live) {
-        const int32_t* m = a.src_row + qt * BQ;
-        const int4 rc = *reinterpret_cast<const int4*>(m + 32 * wave + 4 * crow);
-        const int4 rl = *reinterpret_cast<const int4*>(m + 4 * x);
-        const int rs = wave < 2 ? m[64 * wave + lane] : 0;
-        const int rcv[4] = {rc.x, rc.y, rc.z, rc.w}, rlv[4] = {rl.x, rl.y, rl.z, rl.w};
+    // 32 w + 4 (lane >> 3) + c); c_* current tile, n_* next
+    uint32_t c_qoff[4] = {0, 0, 0, 0}, n_qoff[4] = {0, 0, 0, 0};
+    auto gather_setup = [&](int64_t qt, uint32_t (&qoff)[4]) {
+        const int4 rc = *reinterpret_cast<const int4*>(a.src_row + qt * BQ + 32 * wave + 4 * crow);
+        const int rcv[4] = {rc.x, rc.y, rc.z, rc.w};
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            qoff[c] = (uint32_t)(rcv[c] < 0 ? 0 : rcv[c]) * (uint32_t)a.red + q_chunk;     // a padding row reads token 0: finite bytes, zero factor
-        }
-        live = (rlv[0] < 0 ? 0u : 1u) | (rlv[1] < 0 ? 0u : 2u) | (rlv[2] < 0 ? 0u : 4u) | (rlv[3] < 0 ? 0u : 8u);
-        if (wave < 2) svoff = (uint32_t)(rs < 0 ? 0 : rs) * (uint32_t)(KB * 4);
+        for (int c = 0; c < 4; ++c) qoff[c] = (uint32_t)(rcv[c] < 0 ? 0 : rcv[c]) * (uint32_t)a.red + q_chunk;
     };
     auto setup = [&](int64_t qt, int64_t pt, const uint8_t*& pp, const uint8_t*& qp, const uint8_t*& sp_, int& store) {
         int e = expert_of(qt);
@@ -241,19 +232,19 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
         if (pt * 256 != p0 && wave < 2) store = 0;
         pp = a.pf + (((int64_t)e * P64 + p0 / 64 + wave) * KB) * 8192;
         qp = GATHER ? a.q : a.q + qt * BQ * a.red;
-        if (wave < 2) sp_ = reinterpret_cast<const uint8_t*>(GATHER ? a.sq : a.sq + (SQL == 1 ? qt * BQ : qt * BQ * KB));
+        if (wave < 2) sp_ = reinterpret_cast<const uint8_t*>(a.sq + (SQL == 1 ? qt * BQ : qt * BQ * KB));
         else sp_ = reinterpret_cast<const uint8_t*>(a.sp + ((int64_t)e * PB + p0 / 128) * KB);
     };
     setup(cq, cp, c_p, c_q, c_s, c_store);
-    if constexpr (GATHER) gather_setup(cq, c_qoff, c_svoff, c_live);
+    if constexpr (GATHER) gather_setup(cq, c_qoff);
     n_p = c_p; n_q = c_q; n_s = c_s;
 
     // the 13 memory instructions that bring in one K block, for ring position TT: 0 = scales, 1..8 = weight fragments
     // (1 KB each, in the order they lie in memory), 9..12 = activation copies
-    auto issue = [&](auto tc, auto ic, const uint8_t* pp, const uint8_t* qp, const uint8_t* sp_, const uint32_t (&qoff)[4], uint32_t svoff) {
+    auto issue = [&](auto tc, auto ic, const uint8_t* pp, const uint8_t* qp, const uint8_t* sp_, const uint32_t (&qoff)[4]) {
         constexpr int TT = decltype(tc)::value, I = decltype(ic)::value;
         if constexpr (I == 0) {
-            if constexpr (!(TRACE & 4)) dma4_s(GATHER && wave < 2 ? svoff : s_voff, sp_, lds_base + TT * STAGE + s_lds);
+            if constexpr (!(TRACE & 4)) dma4_s(s_voff, sp_, lds_base + TT * STAGE + s_lds);
         } else if constexpr (I <= 8) {
             constexpr int t = I - 1;
             if constexpr (!(TRACE & 2)) fm_pload<32 * TT + 4 * t, (t & 3) * 1024>(t < 4 ? p_voff0 : p_voff1, pp);
@@ -266,7 +257,7 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
         }
     };
     auto issue_all = [&](auto tc, const uint8_t* pp, const uint8_t* qp, const uint8_t* sp_) {
-        static_for<13>([&](auto ic) { issue(tc, ic, pp, qp, sp_, c_qoff, c_svoff); });
+        static_for<13>([&](auto ic) { issue(tc, ic, pp, qp, sp_, c_qoff); });
     };
     auto qfrag = [&](const uint8_t* base, int j, int kh) -> i32x8 {
         return ld_frag_lds(base + j * 4096 + (fq_ofs0 ^ (kh * 64)), base + j * 4096 + (fq_ofs1 ^ (kh * 64)));
@@ -332,28 +323,26 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
             if (n_valid) setup(nq, np, n_p, n_q, n_s, n_store);
             else { n_p = c_p; n_q = c_q; n_s = c_s; n_store = 0; }      // past the last tile the prefetch re-reads this tile's first blocks
             if constexpr (GATHER) {
-                if (n_valid) gather_setup(nq, n_qoff, n_svoff, n_live);
+                if (n_valid) gather_setup(nq, n_qoff);
                 else {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) n_qoff[c] = c_qoff[c];
-                    n_svoff = c_svoff;
                 }
             }
         }
         float fq_cur[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) fq_cur[t] = GATHER && !((c_live >> t) & 1u) ? 0.f : sq_nxt[t] * sp_nxt;
+        for (int t = 0; t < 4; ++t) fq_cur[t] = sq_nxt[t] * sp_nxt;
         const int64_t k2 = kb + 2;
         const bool in2 = k2 < KB;
         const int64_t kk = in2 ? k2 : k2 - KB;
         const uint8_t* pp = (in2 ? c_p : n_p) + kk * 8192;
         const uint8_t* qp = (in2 ? c_q : n_q) + kk * 128;
         const uint8_t* sp_ = (in2 ? c_s : n_s) + kk * s_kstep;
-        uint32_t p_qoff[4] = {0, 0, 0, 0}, p_svoff = 0;          // GATHER: the lane offsets of the tile the prefetched block belongs to
+        uint32_t p_qoff[4] = {0, 0, 0, 0};                        // GATHER: the lane offsets of the tile the prefetched block belongs to
         if constexpr (GATHER) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) p_qoff[c] = in2 ? c_qoff[c] : n_qoff[c];
-            p_svoff = in2 ? c_svoff : n_svoff;
         }
         const uint8_t* sbase = lds + PH * STAGE;
         const uint8_t* nbase = lds + NX * STAGE;
@@ -382,8 +371,8 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
             else fm_mfma_second<32 * PH + 16 * pf + 8>(d[t & 1], qf[(2 * j + 1) & 3]);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (m < 12) {
-                if constexpr (m == 0) issue(std::integral_constant<int, PT>{}, std::integral_constant<int, 0>{}, pp, qp, sp_, p_qoff, p_svoff);
-                issue(std::integral_constant<int, PT>{}, std::integral_constant<int, m + 1>{}, pp, qp, sp_, p_qoff, p_svoff);
+                if constexpr (m == 0) issue(std::integral_constant<int, PT>{}, std::integral_constant<int, 0>{}, pp, qp, sp_, p_qoff);
+                issue(std::integral_constant<int, PT>{}, std::integral_constant<int, m + 1>{}, pp, qp, sp_, p_qoff);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (m == 12 && !(TRACE & 16)) { qf[0] = qfrag(nbase, 0, 0); __builtin_amdgcn_sched_barrier(0); }
@@ -461,8 +450,6 @@ __global__ __launch_bounds__(256, 1) void k_gemm_fm(const FmArgs a) {
         if constexpr (GATHER) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) c_qoff[c] = n_qoff[c];
-            c_live = n_live;
-            c_svoff = n_svoff;
         }
         return false;
     };
@@ -509,6 +496,7 @@ static int fm_lds_attr() {
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fm<1>), hipFuncAttributeMaxDynamicSharedMemorySize, kFmDynLds);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fm<1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, kFmDynLds);
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fm<0, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, kFmDynLds);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_fm<1, 0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, kFmDynLds);
     if (e != hipSuccess) return pf8_fail(PF8_ELAUNCH, "pf8_gemm_fm", hipGetErrorString(e));
     done.fetch_or(bit, std::memory_order_release);
     return PF8_OK;
@@ -564,7 +552,8 @@ static int launch_fm(const char* where, const uint8_t* a, const float* sa, int s
     }
     if (src_row) {
         g.src_row = src_row;
-        hipLaunchKernelGGL((k_gemm_fm<0, 0, 1>), dim3((unsigned)(8 * w)), dim3(256), kFmDynLds, (hipStream_t)stream, g);
+        if (sa_layout == 0) hipLaunchKernelGGL((k_gemm_fm<0, 0, 1>), dim3((unsigned)(8 * w)), dim3(256), kFmDynLds, (hipStream_t)stream, g);
+        else hipLaunchKernelGGL((k_gemm_fm<1, 0, 1>), dim3((unsigned)(8 * w)), dim3(256), kFmDynLds, (hipStream_t)stream, g);
     } else if (sa_layout == 0) hipLaunchKernelGGL(k_gemm_fm<0>, dim3((unsigned)(8 * w)), dim3(256), kFmDynLds, (hipStream_t)stream, g);
     else hipLaunchKernelGGL(k_gemm_fm<1>, dim3((unsigned)(8 * w)), dim3(256), kFmDynLds, (hipStream_t)stream, g);
     return pf8_check_launch(where);
@@ -605,14 +594,15 @@ extern "C" int pf8_debug_grouped_gemm_fm_cycles(const uint8_t* a, const float* s
     return launch_fm(__func__, a, sa, 1, b_fm, sb, E, Mtot, N, K, m_indices, out, N, stream, cycles, workgroups, ablate);
 }
 
-extern "C" int pf8_grouped_gemm_nt_contiguous_fm_gather(const uint8_t* tokens, const float* token_scales, int64_t T, const int32_t* src_row,
+extern "C" int pf8_grouped_gemm_nt_contiguous_fm_gather(const uint8_t* tokens, int64_t T, const int32_t* src_row, const float* sa, int sa_layout,
                                                         const uint8_t* b_fm, const float* sb, int E, int64_t Mtot, int64_t N, int64_t K,
                                                         const int32_t* m_indices, uint16_t* out, pf8_stream_t stream) {
     PF8_REQUIRE(E >= 0 && Mtot >= 0 && N >= 0 && K >= 0 && T >= 0, "negative shape");
     if (Mtot == 0 || N == 0 || E == 0) return PF8_OK;
     PF8_REQUIRE(pf8_gemm_fm_supported(Mtot, N, K), "needs Mtot % 128 == 0, N % 128 == 0, N >= 256, K % 128 == 0 and K >= 384");
-    PF8_REQUIRE(T > 0 && tokens && token_scales && src_row && b_fm && sb && out && m_indices, "null pointer");
+    PF8_REQUIRE(T > 0 && tokens && sa && src_row && b_fm && sb && out && m_indices, "null pointer");
     PF8_REQUIRE(PF8_ALIGNED16(tokens) && PF8_ALIGNED16(b_fm) && PF8_ALIGNED16(out) && PF8_ALIGNED16(src_row), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(sa_layout == 0 || sa_layout == 1, "sa_layout must be 0 or 1");
     PF8_REQUIRE(K <= (1ll << 24) && T * K < (1ll << 31), "the token matrix must stay below 2 GiB");
-    return launch_fm(__func__, tokens, token_scales, 0, b_fm, sb, E, Mtot, N, K, m_indices, out, N, stream, nullptr, 0, 0, src_row);
+    return launch_fm(__func__, tokens, sa, sa_layout, b_fm, sb, E, Mtot, N, K, m_indices, out, N, stream, nullptr, 0, 0, src_row);
 }

@@ -158,6 +158,20 @@ __global__ __launch_bounds__(256) void k_permute_source_rows(const int32_t* __re
     if (out_probs) out_probs[r] = probs ? probs[i] : 0.0f;
 }
 
+// The scales of rows that are read through a source map, gathered on their own (4 bytes per row and K block against the 128
+// bytes they scale): out[r, kb] = xs[src_row[r], kb], 0 for a negative src_row; one thread per output element, row fastest.
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void k_gather_row_scales(const float* __restrict__ xs, const int32_t* __restrict__ src_row, int64_t rows,
+                                                           int64_t KB, float* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * KB) return;
+    const int64_t kb = i / rows, r = i % rows;
+    const int t = src_row[r];
+    const float v = t < 0 ? 0.0f : xs[(int64_t)t * KB + kb];
+    if (LAYOUT == 1) out[kb * rows + r] = v;
+    else out[r * KB + kb] = v;
+}
+
 // One workgroup per token: fp32 sum of its routed copies in slot order, bf16 out; probabilities back
 // into [T, topk] order.
 __global__ __launch_bounds__(256) void k_unpermute(const uint16_t* __restrict__ u, const int32_t* __restrict__ rowmap,
@@ -293,6 +307,19 @@ extern "C" int pf8_moe_permute_map(const int32_t* routemap, const float* probs, 
     if (rc || T == 0) return rc;
     hipLaunchKernelGGL(k_permute_source_rows, dim3((unsigned)((T * topk + 255) / 256)), dim3(256), 0, st, routemap, probs, rowmap, T, topk, E,
                        src_row, out_probs);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_gather_row_scales(const float* xs, int64_t T, int64_t KB, const int32_t* src_row, int64_t rows, float* out, int out_layout,
+                                     pf8_stream_t stream) {
+    PF8_REQUIRE(T >= 0 && KB >= 0 && rows >= 0, "negative shape");
+    PF8_REQUIRE(out_layout == 0 || out_layout == 1, "out_layout must be 0 or 1");
+    if (rows == 0 || KB == 0) return PF8_OK;
+    PF8_REQUIRE(src_row && out && (xs || T == 0), "null pointer");
+    PF8_REQUIRE(rows * KB <= 0x7FFFFFFFll * 256, "too many scales");
+    const dim3 grid((unsigned)((rows * KB + 255) / 256));
+    if (out_layout == 1) hipLaunchKernelGGL(k_gather_row_scales<1>, grid, dim3(256), 0, (hipStream_t)stream, xs, src_row, rows, KB, out);
+    else hipLaunchKernelGGL(k_gather_row_scales<0>, grid, dim3(256), 0, (hipStream_t)stream, xs, src_row, rows, KB, out);
     return pf8_check_launch(__func__);
 }
 

@@ -225,7 +225,7 @@ struct TileSrc {
     int64_t ld;            // row stride in elements
     int64_t rows;          // total rows (for xs_layout 1)
     int xs_layout;
-    const int32_t* src_row;   // e4m3 source only: row r of the tile grid is row src_row[r] of xq / xs (negative = a row of zeros); null = r
+    const int32_t* src_row;   // row r of the tile grid is row src_row[r] of the source (negative = a row of zeros); null = r
 };
 
 // load this thread's 8x8 patch as fp32 values; amax bit patterns per row chunk go to rmax[i]
@@ -334,16 +334,30 @@ struct SplitArgs {
 // to bf16 first (q * s rounded to nearest even), which is what the un-fused chain feeds the quantizer
 __device__ __forceinline__ void load_patch_packed(const TileSrc& src, int64_t row0, int64_t col0, int g, int l, uint4 (&w)[8]) {
     if (src.x) {
+        if (src.src_row) {
+            // the thread's eight rows are consecutive: their sources are two 16-byte loads (row0 is a multiple of 128)
+            const int4 r0 = *reinterpret_cast<const int4*>(src.src_row + row0 + 8 * g), r1 = *reinterpret_cast<const int4*>(src.src_row + row0 + 8 * g + 4);
+            const int rr[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) w[i] = ld16(src.x + (row0 + 8 * g + i) * src.ld + col0 + 8 * l);
+            for (int i = 0; i < 8; ++i)
+                w[i] = rr[i] < 0 ? make_uint4(0, 0, 0, 0) : ld16(src.x + (int64_t)rr[i] * src.ld + col0 + 8 * l);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) w[i] = ld16(src.x + (row0 + 8 * g + i) * src.ld + col0 + 8 * l);
+        }
     } else {
         uint2 q[8];
         float sc[8];
         const int64_t KB = src.ld / 128;
+        int rr[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (src.src_row) {
+            const int4 r0 = *reinterpret_cast<const int4*>(src.src_row + row0 + 8 * g), r1 = *reinterpret_cast<const int4*>(src.src_row + row0 + 8 * g + 4);
+            rr[0] = r0.x; rr[1] = r0.y; rr[2] = r0.z; rr[3] = r0.w; rr[4] = r1.x; rr[5] = r1.y; rr[6] = r1.z; rr[7] = r1.w;
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             int64_t r = row0 + 8 * g + i;
-            if (src.src_row) r = src.src_row[r];
+            if (src.src_row) r = rr[i];
             if (r < 0) {                // a zero byte times a zero scale, as the copied padding row holds them
                 q[i] = make_uint2(0, 0);
                 sc[i] = 0.0f;
@@ -808,13 +822,13 @@ extern "C" int pf8_transpose_split_quant(const void* x, const float* xs, int x_i
     return transpose_split_quant(__func__, x, xs, x_is_fp8, xs_layout, rows_per_expert, E, K, nullptr, nullptr, q_t, s_t, pow2 ? 1 : 0, stream);
 }
 
-extern "C" int pf8_transpose_split_quant_gather(const uint8_t* tokens, const float* token_scales, int xs_layout, int64_t T,
+extern "C" int pf8_transpose_split_quant_gather(const void* tokens, const float* token_scales, int x_is_fp8, int xs_layout, int64_t T,
                                                 const int32_t* src_row, const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q_t,
                                                 float* s_t, int pow2, pf8_stream_t stream) {
     PF8_REQUIRE(T > 0, "the token matrix is empty");
-    PF8_REQUIRE(src_row, "null pointer");
-    return transpose_split_quant(__func__, tokens, token_scales, 1, xs_layout, rows_per_expert, E, K, nullptr, nullptr, q_t, s_t, pow2 ? 1 : 0,
-                                 stream, src_row, T);
+    PF8_REQUIRE(src_row && PF8_ALIGNED16(src_row), "src_row must be a 16-byte aligned device pointer");
+    return transpose_split_quant(__func__, tokens, token_scales, x_is_fp8, xs_layout, rows_per_expert, E, K, nullptr, nullptr, q_t, s_t,
+                                 pow2 ? 1 : 0, stream, src_row, T);
 }
 
 extern "C" int pf8_quant_and_transpose_split(const uint16_t* x, const int64_t* rows_per_expert, int E, int64_t K, uint8_t* q, float* s,

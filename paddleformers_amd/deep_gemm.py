@@ -238,9 +238,12 @@ def m_grouped_fp8_gemm_nt_contiguous(a, b, out: torch.Tensor, m_indices: torch.T
         if tuple(sb.shape) != (E, N // 128, K // 128) or sb.dtype != torch.float32:
             raise ValueError(f"b scale must be float32 [{E}, {N // 128}, {K // 128}]")
         T = ta.tokens.shape[0]
+        if ta.tokens.dtype != FP8:
+            raise ValueError("gathered bfloat16 tokens have to be quantized first (GatheredRows.quantize)")
         if T == 0 or T * K >= 2 ** 31 or ta.src_row.data_ptr() % 16:
             raise ValueError("gathered rows: the token matrix must be non-empty and below 2 GiB, the source map 16-byte aligned")
-        _lib.call("pf8_grouped_gemm_nt_contiguous_fm_gather", _p(ta.tokens), _p(ta.scale), T, _p(ta.src_row), _p(tb.data), _p(sb.contiguous()),
+        rs, lay = _scale_layout_of(ta.row_scales(), Mtot, K // 128, "row scales")
+        _lib.call("pf8_grouped_gemm_nt_contiguous_fm_gather", _p(ta.tokens), T, _p(ta.src_row), _p(rs), lay, _p(tb.data), _p(sb.contiguous()),
                   E, Mtot, N, K, _p(m_indices), _p(out), _stream())
         return out
     if isinstance(tb, FragmentMajor):

@@ -771,7 +771,14 @@ class FP8GroupGemmMlpFunctionNode:
     def bwd_dowm_input(self, expert_w2, unzipped_grad, o1, tokens_per_expert, m_indices=None, unzipped_probs=None):
         """do2_s [m_sum, I] = do3 . w2^T, then the SwiGLU backward (fp8_utils.py:1011-1052)."""
         bw_w2_quant, bw_w2_scale, bw_w2_cache = self._stacked(expert_w2, False, len(expert_w2))
-        if isinstance(unzipped_grad, tuple):
+        if isinstance(unzipped_grad, F8.GatheredRows):
+            # gradient rows that were never copied: quantized per token, read through their source map where the GEMM can
+            unzipped_grad = unzipped_grad.quantize(self.use_ue8m0)
+            if self._reads_gathered(unzipped_grad, bw_w2_quant, bw_w2_cache):
+                unzipped_grad_fp8, unzipped_grad_scale = unzipped_grad.contiguous(), None
+            else:
+                unzipped_grad_fp8, unzipped_grad_scale = unzipped_grad.materialize()
+        elif isinstance(unzipped_grad, tuple):
             unzipped_grad_fp8, unzipped_grad_scale = unzipped_grad
             unzipped_grad_scale = unzipped_grad_scale.t().contiguous().t()
         else:
@@ -966,15 +973,16 @@ class FP8GroupGemmMlpFunctionNode:
     @torch.no_grad()
     def backward(self, out_grad, unzipped_probs, tokens_per_expert, input_fp8_slice=None, input_scale_slice=None, m_indices=None,
                  reset_status=False):
-        """fp8_utils.py:1234-1321.  Returns (dx, probs_grad); weight gradients are accumulated
-        into each expert weight's main_grad (or grad)."""
+        """fp8_utils.py:1234-1321.  out_grad: bf16 rows, an (fp8, scale) pair, or the `GatheredRows` of
+        moe_permute(..., do_gather=False) on the gradient tokens.  Returns (dx, probs_grad); weight gradients are
+        accumulated into each expert weight's main_grad (or grad)."""
         if self.bwd_subbatch:
             assert m_indices is not None and input_fp8_slice is not None and tokens_per_expert is not None
             assert input_scale_slice is not None or isinstance(input_fp8_slice, F8.GatheredRows)
         dtype = torch.bfloat16
         g0 = extract_first_if_tuple(out_grad)
         if g0.shape[0] == 0:
-            return torch.zeros_like(g0, dtype=dtype), torch.zeros_like(unzipped_probs)
+            return torch.zeros(list(g0.shape), dtype=dtype, device=g0.device), torch.zeros_like(unzipped_probs)
         expert_w1 = [x.w1 for x in self.experts if x is not None]
         expert_w2 = [x.w2 for x in self.experts if x is not None]
         if self.recompute_fwd_gate_up:
@@ -986,7 +994,11 @@ class FP8GroupGemmMlpFunctionNode:
         # per-expert tensors, nor beyond the 256 experts one launch of the quantizer takes)
         fuse = self.fuse_bwd_quant and not self.is_split_group_gemm and len(tokens_per_expert) <= 256
         do3_t = None
-        if fuse and not isinstance(out_grad, tuple) and out_grad.dtype == torch.bfloat16:
+        if isinstance(out_grad, F8.GatheredRows):
+            # ZipNode.backward handed over the gradient tokens and their row map instead of copied rows: the transposed
+            # copy for the weight gradient is quantized through the map, the row-wise copy per token (bwd_dowm_input)
+            do3_t = self.fused_transpose_split_quant(out_grad, None, tokens_per_expert, True)
+        elif fuse and not isinstance(out_grad, tuple) and out_grad.dtype == torch.bfloat16:
             g_fp8, g_scale, g_t_fp8, g_t_scale = F8.quant_and_transpose_split(out_grad, tokens_per_expert, self.use_ue8m0, True,
                                                                               ue8m0_scale=self._scale_bytes)
             out_grad, do3_t = (g_fp8, g_scale.T), (g_t_fp8, g_t_scale)

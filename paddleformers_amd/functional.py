@@ -38,22 +38,43 @@ def _as2d(x: torch.Tensor) -> torch.Tensor:
 
 
 class GatheredRows:
-    """The expert-sorted, padded rows `moe_permute` would write, not copied: row r is row src_row[r] of `tokens`
-    (float8_e4m3fn [T, H]) with that row of `scale` (fp32 [T, H/128]); src_row[r] < 0 is a row of zeros.
-    What `moe_permute(..., do_gather=False)` returns in place of the copied rows; `m_grouped_fp8_gemm_nt_contiguous` (on a
-    fragment-major weight) and `fused_transpose_split_quant` take it where they take the copied rows and read the tokens
-    through the map, with bit-identical results.  A slice `g[a:b]` is the same tokens behind a slice of the map."""
+    """The expert-sorted, padded rows `moe_permute` would write, not copied: row r is row src_row[r] of `tokens`;
+    src_row[r] < 0 is a row of zeros.  `tokens` is float8_e4m3fn [T, H] with `scale` fp32 [T, H/128] (dispatched FP8
+    tokens, quantized gradients), or bfloat16 [T, H] with `scale` None (gradient tokens before quantization).
+    What `moe_permute(..., do_gather=False)` returns in place of the copied rows; `m_grouped_fp8_gemm_nt_contiguous` (e4m3
+    tokens, on a fragment-major weight) and `fused_transpose_split_quant` take it where they take the copied rows and read
+    the tokens through the map, with bit-identical results.  A slice `g[a:b]` is the same tokens behind a slice of the map."""
 
-    __slots__ = ("tokens", "scale", "src_row")
+    __slots__ = ("tokens", "scale", "src_row", "_row_scale")
 
-    def __init__(self, tokens: torch.Tensor, scale: torch.Tensor, src_row: torch.Tensor):
-        if tokens.dtype != FP8 or tokens.dim() != 2 or not tokens.is_contiguous():
-            raise ValueError("tokens must be a contiguous float8_e4m3fn [T, H] tensor")
-        if scale.dtype != torch.float32 or tuple(scale.shape) != (tokens.shape[0], tokens.shape[1] // 128) or not scale.is_contiguous():
-            raise ValueError("scale must be a contiguous float32 [T, H/128] tensor")
+    def __init__(self, tokens: torch.Tensor, scale: Optional[torch.Tensor], src_row: torch.Tensor):
+        if tokens.dim() != 2 or not tokens.is_contiguous() or tokens.dtype not in (FP8, torch.bfloat16):
+            raise ValueError("tokens must be a contiguous float8_e4m3fn or bfloat16 [T, H] tensor")
+        if tokens.dtype == FP8:
+            if scale is None or scale.dtype != torch.float32 or tuple(scale.shape) != (tokens.shape[0], tokens.shape[1] // 128) \
+                    or not scale.is_contiguous():
+                raise ValueError("float8 tokens come with a contiguous float32 [T, H/128] scale tensor")
+        elif scale is not None:
+            raise ValueError("bfloat16 tokens carry no scale")
         if src_row.dtype != torch.int32 or src_row.dim() != 1:
             raise ValueError("src_row must be int32 [rows]")
         self.tokens, self.scale, self.src_row = tokens, scale, src_row
+        self._row_scale = None
+
+    def row_scales(self) -> torch.Tensor:
+        """The scales of the expert-sorted rows, fp32 logical [rows, H/128] stored [H/128, rows] (what the GEMMs read
+        without a copy), zero on rows of zeros: gathered from the token scales on first use (4 bytes per row and block
+        against the 128 bytes they scale) and kept."""
+        if self.tokens.dtype != FP8:
+            raise ValueError("bfloat16 tokens carry no scales (quantize() first)")
+        if self._row_scale is None:
+            rows, KB = self.src_row.shape[0], self.scale.shape[1]
+            src = self.src_row if self.src_row.is_contiguous() else self.src_row.contiguous()
+            out = torch.empty((KB, rows), dtype=torch.float32, device=self.device)
+            if rows and KB:
+                _lib.call("pf8_gather_row_scales", _p(self.scale), self.tokens.shape[0], KB, _p(src), rows, _p(out), 1, _stream())
+            self._row_scale = out.t()
+        return self._row_scale
 
     @property
     def shape(self):
@@ -73,17 +94,33 @@ class GatheredRows:
     def __getitem__(self, sl):
         if not isinstance(sl, slice) or sl.step not in (None, 1):
             raise TypeError("only contiguous row slices of gathered rows can be taken")
-        return GatheredRows(self.tokens, self.scale, self.src_row[sl])
+        return GatheredRows(self.tokens, self.scale, self.src_row[sl])       # (its row scales are gathered anew: they are stored per slice)
 
     def contiguous(self):
-        return self if self.src_row.is_contiguous() else GatheredRows(self.tokens, self.scale, self.src_row.contiguous())
+        if self.src_row.is_contiguous():
+            return self
+        g = GatheredRows(self.tokens, self.scale, self.src_row.contiguous())
+        g._row_scale = self._row_scale
+        return g
 
-    def materialize(self) -> Tuple[torch.Tensor, torch.Tensor]:
-        """(rows e4m3 [rows, H], scales fp32 [rows, H/128]): the copy, for a consumer that cannot read through the map."""
+    def quantize(self, using_pow2_scale: bool = False) -> "GatheredRows":
+        """bfloat16 tokens -> the same rows behind their 1x128-quantized tokens.  The rule is per row, so quantizing the T
+        tokens once gives every copy the bytes and scales that quantizing the copied rows would (and a row of zeros stays
+        one)."""
+        if self.tokens.dtype == FP8:
+            return self
+        q, s = fp8_quant_blockwise(self.tokens, quant_method="1x128", using_pow2_scale=using_pow2_scale)
+        return GatheredRows(q, s, self.src_row)
+
+    def materialize(self):
+        """The copy, for a consumer that cannot read through the map: (rows e4m3 [rows, H], scales fp32 [rows, H/128]) for
+        float8 tokens, rows bfloat16 [rows, H] for bfloat16 tokens."""
         live = self.src_row >= 0
         idx = self.src_row.clamp(min=0).long()
-        rows = self.tokens.view(torch.uint8)[idx] * live[:, None].to(torch.uint8)
-        return rows.view(FP8), self.scale[idx] * live[:, None].to(torch.float32)
+        if self.tokens.dtype == FP8:
+            rows = self.tokens.view(torch.uint8)[idx] * live[:, None].to(torch.uint8)
+            return rows.view(FP8), self.scale[idx] * live[:, None].to(torch.float32)
+        return torch.where(live[:, None], self.tokens[idx], torch.zeros((), dtype=torch.bfloat16, device=self.device))
 
 
 def _scale_layout_of(s: torch.Tensor, rows: int, blocks: int, what: str, allow_ue8m0: bool = False) -> Tuple[torch.Tensor, int]:
@@ -387,7 +424,8 @@ def _transpose_split_quant_gathered(g: GatheredRows, rows: List[int], pow_2_scal
         if sum(chunk) == 0:
             continue
         arr = (C.c_int64 * len(chunk))(*chunk)
-        _lib.call("pf8_transpose_split_quant_gather", _p(g.tokens), _p(g.scale), 0, T, C.c_void_p(src.data_ptr() + off * 4), arr, len(chunk), K,
+        _lib.call("pf8_transpose_split_quant_gather", _p(g.tokens), _p(g.scale), int(g.tokens.dtype == FP8), 0, T,
+                  C.c_void_p(src.data_ptr() + off * 4), arr, len(chunk), K,
                   C.c_void_p(q_t.data_ptr() + off * K), C.c_void_p(s_t.data_ptr() + (off // 128) * K * 4), int(bool(pow_2_scales)), _stream())
     qs, ss, off = [], [], 0
     for r in rows:
@@ -726,8 +764,8 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
     expert_routemap_topk int32 [T, topk] (negative = unused slot); expert_prob_topk fp32 [T, topk].
     Returns (hidden_states_unzipped [Mpad, H], zipped_expertwise_rowmap int32 [T, num_experts],
     token_prob_unzipped fp32 [Mpad, 1], scale_unzipped fp32 [Mpad, H/128] or None).
-    do_gather=False (float8 hidden_states only) copies no row: the first result is a `GatheredRows` (the tokens, their
-    scales and the source token of every output row), the last is None.
+    do_gather=False copies no row: the first result is a `GatheredRows` (the tokens, their scales if they are float8, and
+    the source token of every output row), the last is None.
     Counts that do not match the routing (a token routed to an expert beyond its `tokens_per_expert` count is
     dropped; rows of an overstated count are written as zeros) set a sticky flag word that lives on the device for
     the life of the process: the call itself neither allocates nor reads it back, as the reference's operator has no
@@ -765,8 +803,6 @@ def moe_permute(hidden_states: torch.Tensor, scale: Optional[torch.Tensor], expe
     overflow = _permute_flag(dev)
     cnt = (C.c_int64 * num_experts)(*counts)
     if not do_gather:
-        if not is_fp8:
-            raise ValueError("do_gather=False serves float8 hidden_states (the consumers of gathered rows read e4m3 tokens)")
         src_row = torch.empty((mpad,), dtype=torch.int32, device=dev)
         _lib.call("pf8_moe_permute_map", _p(rm), _p(pr), T, topk, num_experts, cnt, a, _p(rowmap), _p(src_row), _p(out_p), _p(overflow),
                   _stream())

@@ -68,9 +68,11 @@ class FusionMlpNode:
         self.output_subbatch_rows = output_subbatch_rows     # granularity of the reference's fp32 zip; unused here (see module text)
         self.unzipped_probs = None
         self.m_indices = None
-        # with FP8 dispatch and one grouped launch per GEMM (is_split_group_gemm=False) the unzip copies no token row: the
-        # up+gate GEMM and the transposed quantizer of the weight gradient read the dispatched tokens through the row map
-        # (same results to the bit; the expert-sorted copy of the tokens and of their scales never exists).  False = copy.
+        # with one grouped launch per GEMM (is_split_group_gemm=False) the reordering copies no row.  Forward, FP8 dispatch:
+        # the up+gate GEMM and the transposed quantizer of the weight gradient read the dispatched tokens through the row
+        # map.  Backward: the gradient tokens are quantized per token, the dgrad GEMM reads them through the map and the
+        # transposed quantizer reads the bf16 tokens through it.  Same results to the bit; the expert-sorted copies of the
+        # tokens, of the gradients and of their scales never exist.  False = copy.
         self.fuse_unzip = True
 
     def set_recompute_fwd_gate_up(self, recompute_fwd_gate_up):
@@ -188,14 +190,16 @@ class FusionMlpNode:
     def backward(self, hidden_states_out_grad: _Tokens):
         """hidden_states_out_grad: bf16 [T, H] or (e4m3, scales).  Returns (gradient of the dispatched tokens bf16 [T, H],
         gradient of the dispatch probabilities fp32 [T, topk]) and drops the node's state."""
+        node = self.experts_group_gemm_node
+        map_only = self.fuse_unzip and not node.is_split_group_gemm and not node.use_ue8m0 and \
+            extract_first_if_tuple(hidden_states_out_grad).shape[0] > 0
         unzipped_grad = self.zip_node.backward(hidden_states_out_grad, self.dispatched_indices, self.dispatched_probs,
                                                top_k=self.router_topk, num_experts=len(self.tokens_per_expert),
-                                               tokens_per_expert=self.tokens_per_expert)
+                                               tokens_per_expert=self.tokens_per_expert, do_gather=not map_only)
         total_zipped_tokens = extract_first_if_tuple(hidden_states_out_grad).shape[0]
         total_unzipped_tokens = extract_first_if_tuple(unzipped_grad).shape[0]
         num_experts = len(self.tokens_per_expert)
         padding_token_per_experts = [(x + 127) // 128 * 128 for x in self.tokens_per_expert]
-        node = self.experts_group_gemm_node
         if self.mlp_bwd_subbatch_rows != 0 and total_unzipped_tokens > self.mlp_bwd_subbatch_rows * 2:
             subbatch_rows = self._subbatch_rows(total_unzipped_tokens, num_experts, self.mlp_bwd_subbatch_rows)
             hidden = extract_first_if_tuple(hidden_states_out_grad).shape[-1]

@@ -78,6 +78,10 @@ class ZipNode:
 
     @torch.no_grad()
     def backward(self, grad_output: _Tokens, dispatched_indices: torch.Tensor, dispatched_probs: Optional[torch.Tensor],
-                 top_k: int, num_experts: int, tokens_per_expert: Sequence[int]):
-        rows, _, _, scale = _permute(grad_output, dispatched_indices, dispatched_probs, num_experts, tokens_per_expert)
+                 top_k: int, num_experts: int, tokens_per_expert: Sequence[int], do_gather: bool = True):
+        """do_gather=False: no row is copied; the result is the `GatheredRows` (gradient tokens behind the row map) the
+        expert MLP node's backward reads through."""
+        rows, _, _, scale = _permute(grad_output, dispatched_indices, dispatched_probs, num_experts, tokens_per_expert, do_gather=do_gather)
+        if not do_gather:
+            return rows
         return (rows, scale) if isinstance(grad_output, tuple) else rows

@@ -88,8 +88,28 @@ def test_source_map_flags_counts_that_disagree_with_the_routing(F):
     # the rows of the overstated count read as zeros, as the copy writes them
     rows, scales = g.materialize()
     assert torch.equal(rows.view(torch.uint8), cx.view(torch.uint8)) and torch.equal(scales, cs) and torch.equal(gp, cp)
-    with pytest.raises(ValueError):                 # bf16 tokens have no consumer that reads through the map
-        F.moe_permute(G.to_torch_bf16(G.bf16_normal((T, H), seed=1)), None, trm, tpr, E, counts, 128, do_gather=False)
+
+
+def test_source_map_of_bf16_tokens_and_their_per_token_quantization(F):
+    """Gradient tokens: bf16 rows behind the map; quantizing the T tokens gives every copy the bytes and scales that
+    quantizing the copied rows gives (the 1x128 rule is per row)."""
+    T, H, topk, E = 333, 512, 3, 5
+    rm, probs, counts = routing(T, topk, E, seed=12)
+    bits = G.bf16_normal((T, H), seed=13, outlier_frac=1e-3, outlier_scale=50.0)
+    tx, trm, tpr = G.to_torch_bf16(bits), torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda()
+    cx, crow, cp, _ = F.moe_permute(tx, None, trm, tpr, E, counts, 128)
+    g, grow, gp, gs = F.moe_permute(tx, None, trm, tpr, E, counts, 128, do_gather=False)
+    assert gs is None and g.scale is None and g.dtype == torch.bfloat16 and torch.equal(grow, crow) and torch.equal(gp, cp)
+    assert torch.equal(g.materialize().view(torch.int16), cx.view(torch.int16))
+    for pow2 in (False, True):
+        cq, cs = F.fp8_quant_blockwise(cx, quant_method="1x128", using_pow2_scale=pow2)
+        gq = g.quantize(pow2)
+        assert gq.dtype == F.FP8 and gq.quantize(pow2) is gq
+        rows, scales = gq.materialize()
+        live = (g.src_row >= 0)
+        assert torch.equal(rows.view(torch.uint8), cq.view(torch.uint8))
+        assert torch.equal(scales[live], cs[live])          # (the copy gives a padding row the scale of an all-zero tile, 1)
+        assert (scales[~live] == 0).all() and (cs[~live] == 1).all()
 
 
 def _weights(E, N, K, seed):
@@ -152,11 +172,18 @@ def test_grouped_gemm_through_the_map_rejects_what_it_cannot_read(F):
 
 @pytest.mark.parametrize("T,K,topk,E", [(300, 512, 2, 5), (1000, 128, 3, 4), (260, 1408, 4, 8)])
 @pytest.mark.parametrize("pow2", [True, False])
-def test_transposed_quantizer_reads_through_the_source_map(F, T, K, topk, E, pow2):
+@pytest.mark.parametrize("bf16", [False, True])
+def test_transposed_quantizer_reads_through_the_source_map(F, T, K, topk, E, pow2, bf16):
     rm, probs, counts = routing(T, topk, E, seed=T + K + 1, drop=0.1)
-    q, s = _tokens(T, K, seed=K + 7)
-    (cx, _, _, cs), (g, _, _, _) = _both(F, q, s, rm, probs, E, counts)
     padded = [(c + 127) // 128 * 128 for c in counts]
+    if bf16:
+        tx = G.to_torch_bf16(G.bf16_normal((T, K), seed=K + 9, outlier_frac=1e-3, outlier_scale=30.0))
+        trm, tpr = torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda()
+        cx, cs = F.moe_permute(tx, None, trm, tpr, E, counts, 128)[0], None
+        g = F.moe_permute(tx, None, trm, tpr, E, counts, 128, do_gather=False)[0]
+    else:
+        q, s = _tokens(T, K, seed=K + 7)
+        (cx, _, _, cs), (g, _, _, _) = _both(F, q, s, rm, probs, E, counts)
     qc, sc = F.fused_transpose_split_quant(cx, cs, padded, pow2)
     qg, sg = F.fused_transpose_split_quant(g, None, padded, pow2)
     assert len(qc) == len(qg) == E
@@ -164,8 +191,9 @@ def test_transposed_quantizer_reads_through_the_source_map(F, T, K, topk, E, pow
         assert qc[e].shape == qg[e].shape and sc[e].shape == sg[e].shape
         assert torch.equal(qc[e].view(torch.uint8), qg[e].view(torch.uint8)), f"expert {e} bytes"
         assert torch.equal(sc[e], sg[e]), f"expert {e} scales"
-    with pytest.raises(ValueError):
-        F.fused_transpose_split_quant(g, g.scale, padded, pow2)
+    if not bf16:
+        with pytest.raises(ValueError):
+            F.fused_transpose_split_quant(g, g.scale, padded, pow2)
 
 
 @pytest.mark.parametrize("recompute", [False, True])
@@ -181,7 +209,10 @@ def test_expert_mlp_node_on_gathered_rows_equals_the_node_on_copied_rows(F, reco
     cx, _, cp, cs = F.moe_permute(tq, ts, trm, tpr, E, counts, 128)
     g, _, gp, _ = F.moe_permute(tq, ts, trm, tpr, E, counts, 128, do_gather=False)
     padded = [(c + 127) // 128 * 128 for c in counts]
-    grad = torch.randn((sum(padded), H), generator=torch.Generator(device="cuda").manual_seed(5), device="cuda").to(torch.bfloat16)
+    # the gradient arrives as tokens too (ZipNode.backward): copied rows for the one node, the map for the other
+    tg = torch.randn((T, H), generator=torch.Generator(device="cuda").manual_seed(6), device="cuda").to(torch.bfloat16)
+    grad = F.moe_permute(tg, None, trm, tpr, E, counts, 128)[0]
+    grad_map = F.moe_permute(tg, None, trm, tpr, E, counts, 128, do_gather=False)[0]
     results = []
     for rows in ((cx, cs), g):
         experts = _fresh_experts(w1, w2)
@@ -190,7 +221,7 @@ def test_expert_mlp_node_on_gathered_rows_equals_the_node_on_copied_rows(F, reco
         o3 = node.forward(rows, cp, padded)
         if rows is g:
             assert isinstance(node.input_fp8, F.GatheredRows) and node.input_scale is None     # nothing was copied
-        dx, pg = node.backward(grad, cp, padded)
+        dx, pg = node.backward(grad_map if rows is g else grad, cp, padded)
         results.append((o3, dx, pg, [e.w1.main_grad for e in experts], [e.w2.main_grad for e in experts]))
     a, b = results
     assert torch.equal(a[0].view(torch.int16), b[0].view(torch.int16)) and torch.equal(a[1].view(torch.int16), b[1].view(torch.int16))
@@ -199,7 +230,8 @@ def test_expert_mlp_node_on_gathered_rows_equals_the_node_on_copied_rows(F, reco
         assert (ga is None) == (gb is None) and (ga is None or torch.equal(ga, gb))
 
 
-def test_fusion_mlp_node_copies_no_token_row_and_matches_the_copying_layer():
+@pytest.mark.parametrize("fp8_dispatch", [True, False])
+def test_fusion_mlp_node_copies_no_token_row_and_matches_the_copying_layer(fp8_dispatch):
     from paddleformers_amd import functional as F8
     from paddleformers_amd.fp8_utils import fp8_quant_weight
     from paddleformers_amd.moe_layer import FusionMlpNode
@@ -209,18 +241,24 @@ def test_fusion_mlp_node_copies_no_token_row_and_matches_the_copying_layer():
     T, H, I, E, topk = 900, 512, 256, 4, 2
     rm, probs, counts, w1, w2, _, x, dy = _layer(T, H, I, E, topk, seed=91)
     trm, tpr = torch.from_numpy(rm).cuda(), torch.from_numpy(probs).cuda()
-    tokens = F8.fp8_quant_blockwise(G.to_torch_bf16(x), quant_method="1x128")
+    tokens = F8.fp8_quant_blockwise(G.to_torch_bf16(x), quant_method="1x128") if fp8_dispatch else G.to_torch_bf16(x)
     tdy = G.to_torch_bf16(dy)
     out = []
     for fuse, fwd_rows, bwd_rows in ((False, 0, 0), (True, 0, 0), (False, 256, 256), (True, 256, 256)):
         experts = _fresh_experts(w1, w2)
         fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True)
         layer = FusionMlpNode(_custom_map(experts, counts), topk, is_split_group_gemm=False, recompute_fwd_gate_up=True,
-                              mlp_fwd_subbatch_rows=fwd_rows, mlp_bwd_subbatch_rows=bwd_rows)
+                              dsv3_use_fp8_dispatch=fp8_dispatch, mlp_fwd_subbatch_rows=fwd_rows if fp8_dispatch else 0,
+                              mlp_bwd_subbatch_rows=bwd_rows)
         layer.fuse_unzip = fuse
         y = layer.forward(tokens, trm, tpr)
-        assert isinstance(layer.experts_group_gemm_node.input_fp8, F8.GatheredRows) == fuse
+        # forward: only FP8 tokens are read through the map (bf16 tokens are copied, then quantized); backward: always
+        assert isinstance(layer.experts_group_gemm_node.input_fp8, F8.GatheredRows) == (fuse and fp8_dispatch)
+        seen = []
+        real = layer.experts_group_gemm_node.backward
+        layer.experts_group_gemm_node.backward = lambda g, *a, **k: (seen.append(type(g)), real(g, *a, **k))[1]
         dx, dp = layer.backward(tdy)
+        assert all((t is F8.GatheredRows) == fuse for t in seen) and seen
         out.append((y, dx, dp, [e.w1.main_grad for e in experts] + [e.w2.main_grad for e in experts]))
     for other in out[1:]:
         assert torch.equal(out[0][0].view(torch.int16), other[0].view(torch.int16))
@@ -229,3 +267,15 @@ def test_fusion_mlp_node_copies_no_token_row_and_matches_the_copying_layer():
     for a, b in ((out[0], out[1]), (out[2], out[3])):
         for ga, gb in zip(a[3], b[3]):
             assert (ga is None) == (gb is None) and (ga is None or torch.equal(ga, gb))
+
+
+def test_row_scales_of_gathered_rows(F):
+    T, H, topk, E = 150, 640, 2, 4
+    rm, probs, counts = routing(T, topk, E, seed=21)
+    q, s = _tokens(T, H, seed=22)
+    (cx, _, _, cs), (g, _, _, _) = _both(F, q, s, rm, probs, E, counts)
+    rs = g.row_scales()
+    assert tuple(rs.shape) == tuple(cs.shape) and rs.stride() == (1, rs.shape[0]) and g.row_scales() is rs      # stored [H/128, rows], made once
+    assert torch.equal(rs, cs)                       # zero on padding rows, as the copy writes them
+    part = g[128:256]
+    assert torch.equal(part.row_scales(), cs[128:256]) and part.row_scales().stride() == (1, 128)
