@@ -68,9 +68,9 @@ class FusionMlpNode:
         self.output_subbatch_rows = output_subbatch_rows     # granularity of the reference's fp32 zip; unused here (see module text)
         self.unzipped_probs = None
         self.m_indices = None
-        # with one grouped launch per GEMM (is_split_group_gemm=False) the reordering copies no row.  Forward, FP8 dispatch:
-        # the up+gate GEMM and the transposed quantizer of the weight gradient read the dispatched tokens through the row
-        # map.  Backward: the gradient tokens are quantized per token, the dgrad GEMM reads them through the map and the
+        # with one grouped launch per GEMM (is_split_group_gemm=False) the reordering copies no row.  Forward: the up+gate
+        # GEMM and the transposed quantizer of the weight gradient read the dispatched tokens (bf16 tokens quantized per
+        # token first) through the row map.  Backward: the gradient tokens are quantized per token, the dgrad GEMM reads them through the map and the
         # transposed quantizer reads the bf16 tokens through it.  Same results to the bit; the expert-sorted copies of the
         # tokens, of the gradients and of their scales never exist.  False = copy.
         self.fuse_unzip = True
@@ -155,12 +155,15 @@ class FusionMlpNode:
         self.dispatched_indices = dispatched_indices.to(torch.int32)
         total_zipped_tokens = extract_first_if_tuple(hs_2d_dispatched).shape[0]
         node = self.experts_group_gemm_node
-        map_only = (self.fuse_unzip and isinstance(hs_2d_dispatched, tuple) and not node.is_split_group_gemm and not node.use_ue8m0
-                    and total_zipped_tokens > 0)
+        map_only = self.fuse_unzip and not node.is_split_group_gemm and not node.use_ue8m0 and total_zipped_tokens > 0
         unzipped_tokens, zipped_expertwise_rowmap, unzipped_probs, unzipped_tokens_scale = self.unzip_node.forward(
             hs_2d_dispatched, self.dispatched_indices, dispatched_probs, topk=self.router_topk, num_experts=num_experts,
             tokens_per_expert=self.tokens_per_expert, do_gather=not map_only)
         self.unzipped_probs = unzipped_probs          # [rows, 1] already
+        if map_only and not isinstance(hs_2d_dispatched, tuple):
+            # bf16 dispatch: the node would quantize every expert-sorted copy of a token (fp8_utils.py:938-941); the 1x128
+            # rule is per row, so the T tokens are quantized once instead and read through the map like dispatched FP8 tokens
+            unzipped_tokens = unzipped_tokens.quantize(False)
         total_unzipped_tokens = unzipped_tokens.shape[0]
         # adaptive recompute of the up+gate output: on when this rank received more rows than the balanced share times a ratio
         if self.recompute_fwd_gate_up == -1:
