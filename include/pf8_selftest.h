@@ -24,6 +24,9 @@ int pf8_debug_encode(const float* v, int64_t n, uint8_t* out, pf8_stream_t strea
 int pf8_debug_div_encode(const float* x, const float* s, int64_t n, uint8_t* out, pf8_stream_t stream);
 /* Self-test hook: out[i] = silu(x[i]) with the device restatement of the oracle's expf. */
 int pf8_debug_silu(const float* x, int64_t n, float* out, pf8_stream_t stream);
+/* Self-test hook: the two quotients of the SwiGLU backward, out_silu[i] = x / (1 + exp(-x)) and out_sigmoid[i] = 1 / (1 + exp(-x)),
+ * as the kernel forms them (one hardware reciprocal, exact residuals). */
+int pf8_debug_silu_sigmoid(const float* x, int64_t n, float* out_silu, float* out_sigmoid, pf8_stream_t stream);
 
 /* Measurement hook: pf8_grouped_gemm_nt_contiguous_fm (sa_layout 1) from an instantiation that reads the shader clock
  * at four points of every K block.  cycles int64 [workgroups][8], workgroups >= the launch's grid (at most one per

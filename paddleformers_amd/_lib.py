@@ -63,6 +63,7 @@ SIGNATURES = {
     "pf8_debug_encode": [_vp, _i64, _vp, _vp],
     "pf8_debug_div_encode": [_vp, _vp, _i64, _vp, _vp],
     "pf8_debug_silu": [_vp, _i64, _vp, _vp],
+    "pf8_debug_silu_sigmoid": [_vp, _i64, _vp, _vp, _vp],
 }
 
 

@@ -246,6 +246,20 @@ __device__ __forceinline__ float silu_exact(float g, const ExpPoly& k) {
 }
 __device__ __forceinline__ float silu_exact(float g) { return silu_exact(g, exp_poly()); }
 
+// The two quotients of the SwiGLU backward from one hardware reciprocal: g / den (silu_exact's sequence) and 1 / den
+// (y = v_rcp_f32(den), r = fma(-y, den, 1), y + r y), den = 1 + exp(-g).  Both are the correctly rounded quotients for
+// every bf16 g: the GPU test suite compares them with the CPU checker's divisions on all 65,536 inputs.
+struct SiluSigmoid { float silu, sigmoid; };
+__device__ __forceinline__ SiluSigmoid silu_and_sigmoid(float g, const ExpPoly& k) {
+    const float den = 1.0f + expf_fixed(-g, k);
+    const float y = __builtin_amdgcn_rcpf(den);
+    const float q0 = g * y;
+    SiluSigmoid o;
+    o.silu = __builtin_copysignf(__builtin_fmaf(__builtin_fmaf(-q0, den, g), y, q0), g);
+    o.sigmoid = __builtin_fmaf(__builtin_fmaf(-y, den, 1.0f), y, y);
+    return o;
+}
+
 // Contiguous-grouped GEMM with UE8M0 scales: which of the two kernels takes an expert load, from the
 // work-item list's header {paired 256-row items, 128-row blocks}.  Rounds of tiles per compute unit,
 // a 256x256 block costing 1.6 times a 128x256 one (measured): few blocks per expert leave many

@@ -88,11 +88,12 @@ __global__ __launch_bounds__(256) void k_quant_1x128(const uint16_t* __restrict_
 // Per output the kernel spends about 29 vector instructions, 17 of them SiLU (the exponential's short fixed sequence, one
 // v_rcp_f32 and the three-instruction exact quotient).  Products are rounded to bf16 in pairs by the hardware convert and
 // stay packed: the optional bf16 copy is stored as they are and amax runs on packed 16-bit magnitudes.
-template <int LAYOUT, bool HAS_P>
+// U: 128-column blocks per lane group (a wavefront covers 4 U of them); the host picks the U that leaves fewer idle lane
+// groups in a row's last wavefront (I = 1408: 11 blocks are three wavefronts of 4, not two of 8 with five groups idle).
+template <int LAYOUT, bool HAS_P, int U>
 __global__ __launch_bounds__(256) void k_swiglu_quant(const uint16_t* __restrict__ o1, const float* __restrict__ probs,
                                                       int64_t M, int64_t m0, int IB, uint8_t* __restrict__ q,
                                                       float* __restrict__ s, uint16_t* __restrict__ o2, int pow2) {
-    constexpr int U = 2;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, l = lane & 15;
     const int64_t r = m0 + (int64_t)blockIdx.y * 4 + wave;
     if (r >= M) return;
@@ -161,6 +162,7 @@ __global__ __launch_bounds__(256) void k_swiglu_bwd(const uint16_t* __restrict__
     uint4* dur = reinterpret_cast<uint4*>(do1 + r * 2 * I + I);
     uint4* osr = reinterpret_cast<uint4*>(o2_s + r * I);
     const int chunks = (int)(I / 8);
+    const ExpPoly poly = exp_poly_in_registers();
     float pg = 0.0f;
     for (int c = lane; c < chunks; c += 64) {
         const uint4 wg = ld16(gr + c), wu = ld16(ur + c), wd = ld16(dr + c);
@@ -170,14 +172,13 @@ __global__ __launch_bounds__(256) void k_swiglu_bwd(const uint16_t* __restrict__
         unpack8(wd, dv);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float e = expf_fixed(-gv[i]);
-            float den = 1.0f + e;
-            float sl = gv[i] / den;
+            const SiluSigmoid ss = silu_and_sigmoid(gv[i], poly);       // g / den and 1 / den without the IEEE division sequence
+            const float sl = ss.silu;
             float o2f = round_bf16(sl * uv[i]);
             os[i] = o2f * p;
             float do2 = round_bf16(dv[i] * p);
             pg += dv[i] * o2f;
-            float sig = 1.0f / den;
+            const float sig = ss.sigmoid;
             float t1 = 1.0f - sig;
             float t2 = gv[i] * t1;
             float t3 = 1.0f + t2;
@@ -646,9 +647,11 @@ __global__ void k_debug_div_encode(const float* x, const float* s, int64_t n, ui
     uint2 o = quant8(v, t);
     out[i] = (uint8_t)(o.x & 0xFFu);
 }
-__global__ void k_debug_silu(const float* x, int64_t n, float* out) {
+__global__ void k_debug_silu(const float* x, int64_t n, float* out, float* out_sigmoid) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = silu_exact(x[i]);
+    if (i >= n) return;
+    out[i] = silu_exact(x[i]);
+    if (out_sigmoid) out_sigmoid[i] = silu_and_sigmoid(x[i], exp_poly()).sigmoid;
 }
 
 }  // namespace pf8
@@ -853,19 +856,16 @@ extern "C" int pf8_swiglu_weighted_quant(const uint16_t* o1, const float* probs,
     const int64_t slab = (int64_t)65535 * 4;
     for (int64_t m0 = 0; m0 < M; m0 += slab) {
         const int64_t m = M - m0 < slab ? M - m0 : slab;
-        dim3 grid((unsigned)((IB + 7) / 8), (unsigned)((m + 3) / 4)), block(256);
-        if (scale_layout == 0 && probs)
-            hipLaunchKernelGGL((k_swiglu_quant<0, true>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
-        else if (scale_layout == 0)
-            hipLaunchKernelGGL((k_swiglu_quant<0, false>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
-        else if (scale_layout == 1 && probs)
-            hipLaunchKernelGGL((k_swiglu_quant<1, true>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
-        else if (scale_layout == 1)
-            hipLaunchKernelGGL((k_swiglu_quant<1, false>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
-        else if (probs)
-            hipLaunchKernelGGL((k_swiglu_quant<2, true>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
-        else
-            hipLaunchKernelGGL((k_swiglu_quant<2, false>), grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
+        // blocks per wavefront: 8, or 4 when that wastes fewer lane groups on the row's last wavefront
+        const int u = ((IB + 7) / 8) * 8 > ((IB + 3) / 4) * 4 ? 1 : 2;
+        dim3 grid((unsigned)((IB + 4 * u - 1) / (4 * u)), (unsigned)((m + 3) / 4)), block(256);
+        void (*k)(const uint16_t*, const float*, int64_t, int64_t, int, uint8_t*, float*, uint16_t*, int) = nullptr;
+#define PF8_PICK(L, P) (u == 2 ? k_swiglu_quant<L, P, 2> : k_swiglu_quant<L, P, 1>)
+        if (scale_layout == 0) k = probs ? PF8_PICK(0, true) : PF8_PICK(0, false);
+        else if (scale_layout == 1) k = probs ? PF8_PICK(1, true) : PF8_PICK(1, false);
+        else k = probs ? PF8_PICK(2, true) : PF8_PICK(2, false);
+#undef PF8_PICK
+        hipLaunchKernelGGL(k, grid, block, 0, (hipStream_t)stream, o1, probs, M, m0, IB, q, s, o2, pow2);
         int rc = pf8_check_launch(__func__);
         if (rc) return rc;
     }
@@ -953,6 +953,12 @@ extern "C" int pf8_debug_div_encode(const float* x, const float* s, int64_t n, u
 extern "C" int pf8_debug_silu(const float* x, int64_t n, float* out, pf8_stream_t stream) {
     if (n <= 0) return PF8_OK;
     PF8_REQUIRE(x && out, "null pointer");
-    hipLaunchKernelGGL(k_debug_silu, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, n, out);
+    hipLaunchKernelGGL(k_debug_silu, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, n, out, (float*)nullptr);
+    return pf8_check_launch(__func__);
+}
+extern "C" int pf8_debug_silu_sigmoid(const float* x, int64_t n, float* out_silu, float* out_sigmoid, pf8_stream_t stream) {
+    if (n <= 0) return PF8_OK;
+    PF8_REQUIRE(x && out_silu && out_sigmoid, "null pointer");
+    hipLaunchKernelGGL(k_debug_silu, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, n, out_silu, out_sigmoid);
     return pf8_check_launch(__func__);
 }

@@ -47,6 +47,22 @@ def _call_debug(name, *tensors_and_n):
     _lib.call(name, *args, C.c_void_p(torch.cuda.current_stream().cuda_stream))
 
 
+def test_device_sigmoid_of_the_swiglu_backward_matches_the_division(F):
+    """1 / (1 + exp(-g)) as the backward kernel forms it (hardware reciprocal, exact residual, one fused correction) against
+    the IEEE division of the same denominator, on every finite bf16 g; g / (1 + exp(-g)) from the same reciprocal too."""
+    h = np.arange(65536, dtype=np.uint16)
+    f = O.bf16_bits_to_f32(h)
+    f = f[np.isfinite(f)]
+    d = torch.from_numpy(f).cuda()
+    sl, sg = torch.empty_like(d), torch.empty_like(d)
+    _call_debug("pf8_debug_silu_sigmoid", d, f.size, sl, sg)
+    den = (np.float32(1.0) + O.expf_array(-f)).astype(np.float32)
+    with np.errstate(all="ignore"):
+        want = (np.float32(1.0) / den).astype(np.float32)
+    _same(sg.cpu().numpy().view(np.uint32), want.view(np.uint32), "sigmoid over all finite bf16 inputs")
+    _same(sl.cpu().numpy().view(np.uint32), O.silu_array(f).view(np.uint32), "silu over all finite bf16 inputs")
+
+
 def test_hw_encode_matches_oracle_sweep(F):
     """The hardware OCP convert vs the oracle's RNE encoder: every bf16 pattern times a scale
     sweep, the e4m3 grid points, the midpoints between them and their fp32 neighbours."""
