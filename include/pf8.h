@@ -276,8 +276,9 @@ int pf8_gather_row_scales(const float* xs, int64_t T, int64_t KB, const int32_t*
  * [Mtot] or NULL.  Outputs: q e4m3 [Mtot, I] and s fp32 [Mtot, I/128] of
  * quant_1x128( bf16( bf16(silu(o1[:, :I]) * o1[:, I:]) * probs ) ), bit-identical to the two separate calls, and,
  * when o1 is not NULL, the bf16 GEMM result o1 [Mtot, 2I] itself (the node keeps it for backward unless
- * recompute_fwd_gate_up is set, :1263-1267).  Mtot and I multiples of 128, K a multiple of 128 and >= 384; other shapes
- * return PF8_EINVAL (make the two calls). */
+ * recompute_fwd_gate_up is set, :1263-1267).  pow2: bit 0 = power-of-two scales, bit 1 = s is stored [I/128, Mtot] (the
+ * layout the down GEMM reads fastest, scale_layout 1).  Mtot and I multiples of 128, K a multiple of 128 and >= 384;
+ * other shapes return PF8_EINVAL (make the two calls). */
 int pf8_grouped_gemm_swiglu_quant_nt_contiguous(const uint8_t* a, const float* sa, int sa_layout, const uint8_t* b,
                                                 const float* sb, int E, int64_t Mtot, int64_t I, int64_t K,
                                                 const int32_t* m_indices, const float* probs, uint16_t* o1,

@@ -671,13 +671,16 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fwd_deep(const GemmArgs a) {
                         pk[i] = pack_bf16(bf16_lo(w) * pr, bf16_hi(w) * pr);         // pr = 1 without probabilities: the product is exact
                     }
                     const uint32_t m = pkmax_u16(pkmax_u16(pk[0] & 0x7FFF7FFFu, pk[1] & 0x7FFF7FFFu), pkmax_u16(pk[2] & 0x7FFF7FFFu, pk[3] & 0x7FFF7FFFu));
-                    const TileScale t = make_scale(row16_max(umax(m << 16, m & 0xFFFF0000u)), a.pow2_out != 0);
+                    const TileScale t = make_scale(row16_max(umax(m << 16, m & 0xFFFF0000u)), (a.pow2_out & 1) != 0);
                     float v[8];
                     unpack8(make_uint4(pk[0], pk[1], pk[2], pk[3]), v);
                     const uint2 o = quant8(v, t);
                     if (c_rows) {
                         st8(a.q2 + row * a.inter + cp * 128 + ec * 8, o);
-                        if (ec == 0) a.s2[row * IB + cp] = t.s;
+                        if (ec == 0) {
+                            if (a.pow2_out & 2) a.s2[(int64_t)cp * a.Qrows + row] = t.s;      // scales stored [I/128, rows]
+                            else a.s2[row * IB + cp] = t.s;
+                        }
                     }
                 }
                 if (half == 0) __syncthreads();      // everyone has read the first pass's rows before they are overwritten

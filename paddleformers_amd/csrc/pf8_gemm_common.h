@@ -36,7 +36,7 @@ struct GemmArgs {
     const float* probs;         // per-row factor or null
     uint8_t* q2;                // e4m3 [Qrows, inter]
     float* s2;                  // fp32 [Qrows, inter / 128]
-    int pow2_out;               // scale rule of the requantization
+    int pow2_out;               // bit 0: power-of-two scale rule of the requantization; bit 1: s2 stored [inter / 128, Qrows]
 };
 
 // 16-byte chunk c of LDS row `row` lives at chunk c ^ swz_key(row): the 16 rows a fragment read touches

@@ -325,10 +325,10 @@ def m_grouped_fp8_gemm_nt_contiguous_swiglu_quant(a, b, m_indices: torch.Tensor,
         raise ValueError(f"b scale must be float32 [{E}, {N // 128}, {K // 128}]")
     sb = sb if sb.is_contiguous() else sb.contiguous()
     q = torch.empty((Mtot, I), dtype=FP8, device=ta.device)
-    s = torch.empty((Mtot, I // 128), dtype=torch.float32, device=ta.device)
+    s = torch.empty((I // 128, Mtot), dtype=torch.float32, device=ta.device)        # handed back as its transpose (see the quantizer)
     _lib.call("pf8_grouped_gemm_swiglu_quant_nt_contiguous", _p(ta), _p(sa), lay, _p(tb), _p(sb), E, Mtot, I, K, _p(m_indices),
-              _p(probs), _p(out), _p(q), _p(s), int(bool(using_pow2_scaling)), _stream())
-    return q, s
+              _p(probs), _p(out), _p(q), _p(s), int(bool(using_pow2_scaling)) | 2, _stream())
+    return q, s.t()
 
 
 def m_grouped_fp8_gemm_nt_masked(a, b, out: torch.Tensor, masked_m: torch.Tensor, expected_m: int):

@@ -329,8 +329,11 @@ def fused_weighted_swiglu_act_quant(o1: torch.Tensor, probs: Optional[torch.Tens
         _lib.call("pf8_swiglu_weighted_quant", _p(o1), _p(probs), M, I, _p(q), _p(s), _p(o2), 2, 1, _stream())
         s = s.t()
     else:
-        s = torch.empty((M, I // 128), dtype=torch.float32, device=o1.device)
-        _lib.call("pf8_swiglu_weighted_quant", _p(o1), _p(probs), M, I, _p(q), _p(s), _p(o2), 0, int(bool(using_pow2_scaling)), _stream())
+        # stored [I/128, M] and handed back as its transpose: the same [M, I/128] tensor to every consumer, in the layout the
+        # grouped GEMM that follows reads fastest (one 256-byte piece per 64 rows and K block instead of 64 separate words)
+        s = torch.empty((I // 128, M), dtype=torch.float32, device=o1.device)
+        _lib.call("pf8_swiglu_weighted_quant", _p(o1), _p(probs), M, I, _p(q), _p(s), _p(o2), 1, int(bool(using_pow2_scaling)), _stream())
+        s = s.t()
     return (q, s, o2) if return_o2 else (q, s)
 
 
