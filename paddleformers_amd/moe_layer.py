@@ -67,6 +67,7 @@ class FusionMlpNode:
         self.mlp_bwd_subbatch_rows = mlp_bwd_subbatch_rows
         self.output_subbatch_rows = output_subbatch_rows     # granularity of the reference's fp32 zip; unused here (see module text)
         self.unzipped_probs = None
+        self._src_row = None
         self.m_indices = None
         # with one grouped launch per GEMM (is_split_group_gemm=False) the reordering copies no row.  Forward: the up+gate
         # GEMM and the transposed quantizer of the weight gradient read the dispatched tokens (bf16 tokens quantized per
@@ -160,6 +161,8 @@ class FusionMlpNode:
             hs_2d_dispatched, self.dispatched_indices, dispatched_probs, topk=self.router_topk, num_experts=num_experts,
             tokens_per_expert=self.tokens_per_expert, do_gather=not map_only)
         self.unzipped_probs = unzipped_probs          # [rows, 1] already
+        # the routing is the same in backward: the row map built here also places the gradient tokens
+        self._src_row = unzipped_tokens.src_row if map_only else None
         if map_only and not isinstance(hs_2d_dispatched, tuple):
             # bf16 dispatch: the node would quantize every expert-sorted copy of a token (fp8_utils.py:938-941); the 1x128
             # rule is per row, so the T tokens are quantized once instead and read through the map like dispatched FP8 tokens
@@ -196,9 +199,13 @@ class FusionMlpNode:
         node = self.experts_group_gemm_node
         map_only = self.fuse_unzip and not node.is_split_group_gemm and not node.use_ue8m0 and \
             extract_first_if_tuple(hidden_states_out_grad).shape[0] > 0
-        unzipped_grad = self.zip_node.backward(hidden_states_out_grad, self.dispatched_indices, self.dispatched_probs,
-                                               top_k=self.router_topk, num_experts=len(self.tokens_per_expert),
-                                               tokens_per_expert=self.tokens_per_expert, do_gather=not map_only)
+        if map_only and getattr(self, "_src_row", None) is not None:
+            tok, sc = hidden_states_out_grad if isinstance(hidden_states_out_grad, tuple) else (hidden_states_out_grad, None)
+            unzipped_grad = F8.GatheredRows(tok.contiguous(), None if sc is None else sc.contiguous(), self._src_row)
+        else:
+            unzipped_grad = self.zip_node.backward(hidden_states_out_grad, self.dispatched_indices, self.dispatched_probs,
+                                                   top_k=self.router_topk, num_experts=len(self.tokens_per_expert),
+                                                   tokens_per_expert=self.tokens_per_expert, do_gather=not map_only)
         total_zipped_tokens = extract_first_if_tuple(hidden_states_out_grad).shape[0]
         total_unzipped_tokens = extract_first_if_tuple(unzipped_grad).shape[0]
         num_experts = len(self.tokens_per_expert)
