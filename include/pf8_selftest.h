@@ -41,6 +41,11 @@ int pf8_debug_grouped_gemm_fm_cycles(const uint8_t* a, const float* sa, const ui
                                      int64_t Mtot, int64_t N, int64_t K, const int32_t* m_indices, uint16_t* out,
                                      int64_t* cycles, int64_t workgroups, int ablate, pf8_stream_t stream);
 
+/* Measurement hook: pf8_grouped_wgrad_pow2 sends the experts whose reduction axis is at least `blocks` 128-row blocks long
+ * to the kernel with the 256x256 accumulator tile and the others to the 128x128-tile kernel (both give the same bits);
+ * 0 = every expert to the 128x128-tile kernel.  Returns the previous setting (default 6). */
+int pf8_debug_set_wgrad_tile256_min_blocks(int blocks);
+
 #ifdef __cplusplus
 }
 #endif

@@ -64,6 +64,7 @@ SIGNATURES = {
     "pf8_debug_div_encode": [_vp, _vp, _i64, _vp, _vp],
     "pf8_debug_silu": [_vp, _i64, _vp, _vp],
     "pf8_debug_silu_sigmoid": [_vp, _i64, _vp, _vp, _vp],
+    "pf8_debug_set_wgrad_tile256_min_blocks": [_i32],
 }
 
 

@@ -14,8 +14,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libpf8.so")
-SOURCES = ["pf8_api.hip", "pf8_quant.hip", "pf8_gemm.hip", "pf8_gemm_fm.hip", "pf8_gemm_e8.hip", "pf8_permute.hip", "pf8_norm.hip"]
-HEADERS = ["pf8_device.h", "pf8_host.h", "pf8_gemm_common.h", os.path.join("..", "..", "include", "pf8.h"),
+SOURCES = ["pf8_api.hip", "pf8_quant.hip", "pf8_gemm.hip", "pf8_gemm_fm.hip", "pf8_gemm_e8.hip", "pf8_wgrad_e8.hip", "pf8_permute.hip", "pf8_norm.hip"]
+HEADERS = ["pf8_device.h", "pf8_host.h", "pf8_gemm_common.h", "pf8_e8_common.h", os.path.join("..", "..", "include", "pf8.h"),
            os.path.join("..", "..", "include", "pf8_selftest.h")]
 
 FLAGS = [
@@ -107,10 +107,76 @@ def check_fragment_ring(flags) -> None:
         text = open(out).read()
     if "k_gemm_fm" not in text or "v_mfma_f32_32x32x64_f8f6f4" not in text:
         raise RuntimeError("the device assembly of pf8_gemm_fm.hip does not look as expected; the AGPR check cannot run")
+    hz = sgpr_address_hazards(text)
+    if hz:
+        raise RuntimeError(f"pf8_gemm_fm.hip: {len(hz)} memory instructions read a scalar address register too soon after the vector "
+                           f"unit wrote it, e.g. line {hz[0][0]}: {hz[0][1]}")
     n = text.count("v_accvgpr")
     if n:
         raise RuntimeError(f"pf8_gemm_fm.hip: the compiler placed {n} accumulation-register copies of its own; they would "
                            "overwrite the weight-fragment ring (lower the register pressure of k_gemm_fm)")
+
+
+def sgpr_address_hazards(asm_text: str, need: int = 5):
+    """[(line, instruction, sgpr, wait states)] where a vector-memory instruction reads, as its scalar address, a register
+    the vector unit wrote (v_readlane / v_readfirstlane: restored spills, uniform values computed on the vector unit)
+    fewer than `need` wait states earlier.  The hardware needs five; the compiler pads its own instructions with s_nop
+    but not the text of inline assembly, so a kernel whose memory instructions are written by hand can be handed an
+    address register that is not yet readable.  Every instruction counts as one wait state, s_nop N as N + 1."""
+    import re
+
+    bad, last, n = [], {}, 0
+    for ln, l in enumerate(asm_text.splitlines(), 1):
+        t = l.strip()
+        if not l.startswith("\t") or not t or t.startswith((".", ";")):
+            continue
+        op = t.split()[0]
+        if op == "s_nop":
+            n += int(t.split()[1]) + 1
+            continue
+        n += 1
+        m = re.match(r"v_(?:readlane|readfirstlane)_b32 s(\d+)", t)
+        if m:
+            last[int(m.group(1))] = n
+        if op.startswith(("global_", "buffer_", "flat_", "scratch_")):
+            for a, b in re.findall(r"s\[(\d+):(\d+)\]", t):
+                for r in range(int(a), int(b) + 1):
+                    if r in last and n - last[r] - 1 < need:
+                        bad.append((ln, t, r, n - last[r] - 1))
+    return bad
+
+
+def check_accumulator_tiles(flags) -> None:
+    """pf8_gemm_e8.hip and pf8_wgrad_e8.hip keep a 256x256 accumulator tile in the whole AGPR file, named only by their
+    inline assembly.  The compiler sees those registers as free and, under register pressure, parks values of its own
+    there (v_accvgpr_write_b32 aN, vM), which would overwrite accumulators.  The kernels' own accesses are writes of the
+    constant 0 and reads by the epilogues (256 per copy of the epilogue): anything else fails the build."""
+    import re
+    import tempfile
+
+    for name, reads in (("pf8_gemm_e8.hip", None), ("pf8_wgrad_e8.hip", 1024)):
+        src = os.path.join(CSRC, name)
+        with tempfile.TemporaryDirectory() as tmp:
+            out = os.path.join(tmp, name + ".s")
+            cmd = [hipcc()] + [f for f in flags if f not in ("-shared", "-fPIC") and not f.startswith("-Rpass")] + \
+                  ["--offload-device-only", "-S", src, "-o", out]
+            proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+            if proc.returncode != 0:
+                raise RuntimeError(f"hipcc -S failed on {name}:\n" + proc.stdout)
+            text = open(out).read()
+        if "v_mfma_scale_f32_16x16x128_f8f6f4" not in text:
+            raise RuntimeError(f"the device assembly of {name} does not look as expected; the AGPR check cannot run")
+        hz = sgpr_address_hazards(text)
+        if hz:
+            raise RuntimeError(f"{name}: {len(hz)} memory instructions read a scalar address register too soon after the vector unit "
+                               f"wrote it, e.g. line {hz[0][0]}: {hz[0][1]} (s{hz[0][2]} after {hz[0][3]} wait states; put an s_nop in "
+                               "front of the instruction in its inline assembly)")
+        parked = [l.strip() for l in text.splitlines() if re.search(r"v_accvgpr_write_b32 a\d+, [vs]", l) or "v_accvgpr_mov" in l]
+        n_reads = text.count("v_accvgpr_read_b32")
+        if parked or (reads is not None and n_reads != reads):
+            raise RuntimeError(f"{name}: the compiler uses accumulation registers of its own ({len(parked)} copies in, {n_reads} reads"
+                               f"{'' if reads is None else ' where the epilogues make ' + str(reads)}); they would overwrite the "
+                               "accumulator tile (lower the kernel's register pressure)")
 
 
 def build(force: bool = False, verbose: bool = False) -> str:
@@ -135,6 +201,7 @@ def build(force: bool = False, verbose: bool = False) -> str:
     try:
         warning = check_scratch(lines)
         check_fragment_ring(FLAGS)
+        check_accumulator_tiles(FLAGS)
     except RuntimeError:
         os.remove(LIB)
         raise

@@ -61,4 +61,9 @@ extern "C" int pf8_set_num_cus(int n) {
     return prev;
 }
 extern "C" int pf8_get_num_cus(void) { return g_num_cus.load(); }
+
+// experts at least this many 128-row blocks long take the 256x256-tile weight-gradient kernel
+static std::atomic<int> g_wgrad_tile256_min_blocks{6};
+int pf8_wgrad_tile256_min_blocks() { return g_wgrad_tile256_min_blocks.load(); }
+extern "C" int pf8_debug_set_wgrad_tile256_min_blocks(int blocks) { return g_wgrad_tile256_min_blocks.exchange(blocks < 0 ? 0 : blocks); }
 extern "C" int pf8_effective_num_cus(void) { return pf8_effective_cus(); }

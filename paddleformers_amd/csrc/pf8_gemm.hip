@@ -768,6 +768,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
     int64_t KB = a.red / 128;
     if (a.group == GROUP_WGRAD) {
         const int e = blockIdx.y;
+        if ((a.wgrad_skip[e >> 5] >> (e & 31)) & 1u) return;
         const int64_t t0 = a.tile_start[e], t1 = a.tile_start[e + 1];
         // packed per-expert operands: [rows, M_e] at rows*128*t0, scales [M_e/128, rows] at t0*rows
         pbase += a.Prows * 128 * t0;
@@ -1211,6 +1212,32 @@ static int grouped_wgrad(const char* where, const uint8_t* a_t, const float* sa_
     g.Prows = N; g.Qrows = Kin; g.red = 0; g.ldo = N; g.accumulate = accumulate; g.group = GROUP_WGRAD; g.E = E; g.pow2_scales = pow2;
     const int64_t tiles = ((N + 127) / 128) * ((Kin + 127) / 128);
     PF8_REQUIRE_AT(where, tiles <= 0x7FFFFFFF, "too many tiles");
+    // The experts with a long reduction axis (power-of-two scales, shapes the 256x256 tile takes) go to the kernel that
+    // holds the tile in the AGPR file, longest first; the others stay here, where two workgroups per compute unit
+    // overlap one tile's gradient read-modify-write with the other's blocks.  Only when the long experts fill the
+    // device at least once: a handful of 256x256 tiles would leave most compute units idle.
+    const int min_blocks = pf8_wgrad_tile256_min_blocks();
+    if (pow2 && min_blocks > 0 && N % 128 == 0 && N >= 256 && Kin % 128 == 0 && Kin >= 256 && PF8_ALIGNED16(sa_t) &&
+        N * 128 * 4 <= 0x7FFFFFFFll) {
+        int32_t t0[kWgE8MaxItems], kb[kWgE8MaxItems];
+        uint8_t ex[kWgE8MaxItems];
+        int n = 0;
+        for (int e = 0; e < E; ++e) {
+            const int32_t blocks = g.tile_start[e + 1] - g.tile_start[e];
+            if (blocks < (min_blocks < 4 ? 4 : min_blocks) || (int64_t)blocks * 128 > (1ll << 24)) continue;
+            int i = n++;
+            for (; i > 0 && kb[i - 1] < blocks; --i) { t0[i] = t0[i - 1]; kb[i] = kb[i - 1]; ex[i] = ex[i - 1]; }   // longest first
+            t0[i] = g.tile_start[e]; kb[i] = blocks; ex[i] = (uint8_t)e;
+        }
+        const int cus = pf8_effective_cus();
+        const int64_t tiles256 = ((N + 255) / 256) * ((Kin + 255) / 256);
+        if (n > 0 && tiles256 * n >= cus) {
+            rc = pf8_launch_wgrad_e8(b_t, a_t, sb_t, sa_t, out, N, Kin, N, accumulate, n, t0, kb, ex, cus, (hipStream_t)stream, where);
+            if (rc) return rc;
+            if (n == E) return PF8_OK;
+            for (int i = 0; i < n; ++i) g.wgrad_skip[ex[i] >> 5] |= 1u << (ex[i] & 31);
+        }
+    }
     return launch_gemm(g, MODE_WGRAD, dim3((unsigned)tiles, (unsigned)E), (hipStream_t)stream, where);
 }
 

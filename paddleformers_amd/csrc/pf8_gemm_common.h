@@ -30,6 +30,7 @@ struct GemmArgs {
     const int32_t* pair_list;   // UE8M0 forward: when set, the kernel runs only if the paired-tile kernel declines
     int cus;                    //   (header of its work-item list, compute units both assume)
     int pow2_scales;            // wgrad: every scale is a power of two (applied inside the MFMA)
+    uint32_t wgrad_skip[8];     // GROUP_WGRAD: bit e set = expert e is another kernel's (the 256x256-tile launch)
     // fused up+gate -> SwiGLU -> 1x128 requantization (k_gemm_fwd_deep<.., .., 1>): P holds [gate rows | up rows],
     // Prows = 2 * inter; `out` (bf16 [Qrows, 2 inter]) may be null
     int64_t inter;              // I: columns of the quantized activation

@@ -31,6 +31,7 @@
 #include <type_traits>
 
 #include "pf8_device.h"
+#include "pf8_e8_common.h"
 #include "pf8_host.h"
 
 namespace pf8 {
@@ -49,18 +50,6 @@ struct E8Args {
     int force;              // with items: run them here whatever the list's header says
 };
 
-__device__ __forceinline__ int e8_keyp(int row) { return (row & 7) ^ ((row >> 3) & 1); }
-
-// 16 bytes per lane global -> LDS, scalar base + 32-bit lane offset; tracked by vmcnt only
-__device__ __forceinline__ void e8_dma16(uint32_t voff, const uint8_t* sbase, uint32_t lds_dst) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase), "s"(lds_dst) : "memory");
-}
-__device__ __forceinline__ i32x8 e8_frag(const uint8_t* p0, const uint8_t* p1) {
-    i32x4 lo = *reinterpret_cast<const i32x4*>(p0);
-    i32x4 hi = *reinterpret_cast<const i32x4*>(p1);
-    return (i32x8){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-}
-
 // acc[IDX] += (2^(sa-127) A) (2^(sb.byte[OB]-127) B): A = P fragment (one scale per block), B = Q fragment
 template <int IDX, int OB>
 __device__ __forceinline__ void e8_mfma(const i32x8& a, const i32x8& b, int sa, int sb) {
@@ -68,24 +57,6 @@ __device__ __forceinline__ void e8_mfma(const i32x8& a, const i32x8& b, int sa, 
     if constexpr (OB == 1) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel:[0,1,0] op_sel_hi:[0,0,0]" : : "v"(a), "v"(b), "v"(sa), "v"(sb), "n"(4 * IDX), "n"(4 * IDX + 3));
     if constexpr (OB == 2) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel_hi:[0,1,0]" : : "v"(a), "v"(b), "v"(sa), "v"(sb), "n"(4 * IDX), "n"(4 * IDX + 3));
     if constexpr (OB == 3) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%4:%5], %0, %1, a[%4:%5], %2, %3 op_sel:[0,1,0] op_sel_hi:[0,1,0]" : : "v"(a), "v"(b), "v"(sa), "v"(sb), "n"(4 * IDX), "n"(4 * IDX + 3));
-}
-template <int IDX>
-__device__ __forceinline__ void e8_acc_zero4() {
-    asm volatile("v_accvgpr_write_b32 a[%0], 0\n\tv_accvgpr_write_b32 a[%1], 0\n\tv_accvgpr_write_b32 a[%2], 0\n\tv_accvgpr_write_b32 a[%3], 0"
-                 : : "n"(4 * IDX), "n"(4 * IDX + 1), "n"(4 * IDX + 2), "n"(4 * IDX + 3));
-}
-template <int R>
-__device__ __forceinline__ float e8_acc_get() {
-    float v;
-    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v) : "n"(R));
-    return v;
-}
-template <int N, typename F>
-__device__ __forceinline__ void e8_static_for(F&& f) {
-    if constexpr (N > 0) {
-        e8_static_for<N - 1>(f);
-        f(std::integral_constant<int, N - 1>{});
-    }
 }
 
 __global__ __launch_bounds__(256, 1) void k_gemm_e8(const E8Args a) {

@@ -28,3 +28,13 @@ enum { PF8_NOTE_GROUPED_ORDER = 0, PF8_NOTE_MASKED_TABLE = 1 };
 int pf8_launch_deep_ue8m0(const uint8_t* p, const uint8_t* q, const uint8_t* sp8, const uint8_t* sq8, int64_t ldsq, void* out,
                           int64_t Prows, int64_t Qrows, int64_t red, int E, const int32_t* m_indices, const int32_t* pair_list,
                           int cus, hipStream_t stream, const char* where);
+
+// Launches the 256x256-tile weight-gradient kernel (pf8_wgrad_e8.hip) on the listed experts of a grouped weight gradient
+// whose scales are powers of two: item i is expert item_e[i], item_t0[i] 128-row blocks into the packed operands and
+// item_kb[i] >= 4 blocks long; the list is ordered longest first.  Prows, Qrows: multiples of 128, at least 256.
+constexpr int kWgE8MaxItems = 256;
+int pf8_launch_wgrad_e8(const uint8_t* p, const uint8_t* q, const float* sp, const float* sq, float* out, int64_t Prows, int64_t Qrows,
+                        int64_t ldo, int accumulate, int n_items, const int32_t* item_t0, const int32_t* item_kb, const uint8_t* item_e,
+                        int cus, hipStream_t stream, const char* where);
+// experts at least this many 128-row blocks long go to that kernel (0 = none); pf8_debug_set_wgrad_tile256_min_blocks
+int pf8_wgrad_tile256_min_blocks();
