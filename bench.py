@@ -309,6 +309,13 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     out["grouped_wgrad_config5_dw1_pow2"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
     ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=False, scales_pow2=True), [()], min(iters, 20), min(warmup, 3))
     out["grouped_wgrad_config5_dw1_pow2_overwrite"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
+    # the same launch with every expert on the 128x128-tile kernel (by default the experts at least six 128-row blocks long
+    # take the kernel with the 256x256 accumulator tile)
+    from paddleformers_amd import _lib
+    prev = _lib.lib().pf8_debug_set_wgrad_tile256_min_blocks(0)
+    ms = time_kernel(lambda: F8.grouped_wgrad(a_t, sa_t, b_t, sb_t, g, accumulate=True, scales_pow2=True), [()], min(iters, 20), min(warmup, 3))
+    out["grouped_wgrad_config5_dw1_pow2_tile128_only"] = dict(ms, flop=2.0 * ROUTED * H * 2 * I)
+    _lib.lib().pf8_debug_set_wgrad_tile256_min_blocks(prev)
     del a_t, sa_t, b_t, sb_t, g
     torch.cuda.empty_cache()
     if gemm_only:       # the legs a profiler run of the GEMM kernels wants: config 2, 3 (UE8M0), 5 forward and weight gradient
