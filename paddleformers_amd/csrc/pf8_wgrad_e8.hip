@@ -37,6 +37,7 @@ struct WgE8Args {
     int64_t Prows, Qrows, ldo;
     int accumulate;
     int n_items;
+    int gq;                // q-tiles per group of the tile order
     int32_t* tickets;      // [0..7] per-XCD ticket counters, [8] workgroups finished; all zero at launch
     int32_t item_t0[kWgE8MaxItems];   // first 128-row block of the item's expert along the reduction axis
     int32_t item_kb[kWgE8MaxItems];   // its number of blocks (>= 4)
@@ -82,9 +83,12 @@ __global__ __launch_bounds__(256, 1) void k_wgrad_e8(const WgE8Args a) {
     // Prows / Qrows = 256 t + 128: the last tile along that axis has one 128-row half; its second half re-reads the
     // first and the wavefronts that own it store nothing
     const int64_t p_tiles = (a.Prows + 255) / 256, q_tiles = (a.Qrows + 255) / 256;
-    const int64_t T_item = p_tiles * q_tiles;
     const int64_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, W = gridDim.x >> 3;
-    // this XCD's slice of every item's tile grid, and its queue: the slices of all items, longest reduction first
+    // this XCD's slice of every item's tile grid: an eighth of its tiles in the order "groups of gq q-tiles x all p-tiles,
+    // q fastest", so a slice is about gq q-tiles x T / (8 gq) p-tiles and every XCD gets the same number of tiles (the
+    // host picks the gq that makes the slice squarest: fewest operand panels per tile).  Its queue: the slices of all
+    // items, longest reduction first.
+    const int64_t T_item = p_tiles * q_tiles;
     const int64_t lo_x = xcd * T_item / 8, n_x = (xcd + 1) * T_item / 8 - lo_x;
     const int64_t total_x = n_x * a.n_items;
     if (slot >= total_x) { finish(); return; }
@@ -105,10 +109,11 @@ __global__ __launch_bounds__(256, 1) void k_wgrad_e8(const WgE8Args a) {
         // (32-bit divisions run on the vector unit: their wave-uniform results are moved to scalar registers by hand)
         const uint32_t item = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)u / (uint32_t)n_x));
         const uint32_t v = (uint32_t)lo_x + ((uint32_t)u - item * (uint32_t)n_x);
-        // the shorter axis runs fastest: an XCD's slice is then a few whole strips along it
-        const uint32_t fast = (uint32_t)(p_tiles <= q_tiles ? p_tiles : q_tiles);
-        const uint32_t v_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(v / fast)), v_lo = v - v_hi * fast;
-        const int64_t pt = p_tiles <= q_tiles ? v_lo : v_hi, qt = p_tiles <= q_tiles ? v_hi : v_lo;
+        const uint32_t per_group = (uint32_t)(a.gq * p_tiles);
+        const uint32_t grp = (uint32_t)__builtin_amdgcn_readfirstlane((int)(v / per_group)), r = v - grp * per_group;
+        const uint32_t left = (uint32_t)q_tiles - grp * (uint32_t)a.gq, gsize = left < (uint32_t)a.gq ? left : (uint32_t)a.gq;
+        const uint32_t r_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(r / gsize)), r_lo = r - r_hi * gsize;
+        const int64_t qt = (int64_t)grp * a.gq + r_lo, pt = r_hi;
         const int64_t t0 = a.item_t0[item], kbn = a.item_kb[item], e = a.item_e[item];
         const int64_t red = kbn * 128;
         const bool pt_tail = p_tail(pt), qt_tail = q_tail(qt);
@@ -409,7 +414,15 @@ int pf8_launch_wgrad_e8(const uint8_t* p, const uint8_t* q, const float* sp, con
     }
     int rc = wg8_ticket_slot(where, &g.tickets);
     if (rc) return rc;
-    const int64_t T_item = ((Prows + 255) / 256) * ((Qrows + 255) / 256);
+    // q-tiles per group: a slice of T / 8 tiles touches about gq Q panels and T / (8 gq) P panels; the divisor of the q-tile
+    // count that makes that sum smallest
+    const int64_t tq = (Qrows + 255) / 256, tp = (Prows + 255) / 256, T_item = tq * tp;
+    double best = -1.0;
+    for (int64_t gq = 1; gq <= tq; ++gq) {
+        if (tq % gq) continue;
+        const double cost = (double)gq + (double)T_item / (8.0 * (double)gq);
+        if (best < 0 || cost < best) { best = cost; g.gq = (int)gq; }
+    }
     const int64_t per_xcd = ((T_item + 7) / 8) * n_items;
     int64_t w = cus / 8;
     if (w < 1) w = 1;
