@@ -747,16 +747,19 @@ __global__ __launch_bounds__(256, 2) void k_gemm_wgrad(const GemmArgs a) {
     const int wq = wave >> 1, wp = wave & 1;
     const int li = lane & 15, kg = lane >> 4;
 
-    const int64_t p_tiles = (a.Prows + 127) / 128, q_tiles = (a.Qrows + 127) / 128;
-    const int64_t T = p_tiles * q_tiles;
-    const int64_t per_xcd = (T + 7) / 8;
-    const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    // (tile arithmetic in 32 bits: the host admits at most 2^31 tiles, and 64-bit divisions are hundreds of dependent scalar
+    // instructions in front of every tile)
+    const uint32_t p_tiles = (uint32_t)((a.Prows + 127) / 128), q_tiles = (uint32_t)((a.Qrows + 127) / 128);
+    const uint32_t T = p_tiles * q_tiles;
+    const uint32_t per_xcd = (T + 7u) / 8u;
+    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
     if (logical >= T) return;
     // tiles are walked in strips eight P tiles wide, P fastest inside a strip: the 64 workgroups an XCD
     // runs at a time then cover about 8 x 8 tiles and share 16 operand panels in its L2 instead of 34
-    const int64_t strip_w = 8 * q_tiles, strip = logical / strip_w, in_strip = logical - strip * strip_w;
-    const int64_t strip_p = p_tiles - strip * 8 < 8 ? p_tiles - strip * 8 : 8;
-    const int64_t p_tile = strip * 8 + in_strip % strip_p, q_tile = in_strip / strip_p;
+    const uint32_t strip_w = 8u * q_tiles, strip = logical / strip_w, in_strip = logical - strip * strip_w;
+    const uint32_t strip_p = p_tiles - strip * 8u < 8u ? p_tiles - strip * 8u : 8u;
+    const uint32_t q_tile32 = in_strip / strip_p;
+    const int64_t p_tile = strip * 8u + (in_strip - q_tile32 * strip_p), q_tile = q_tile32;
     const int64_t p0 = p_tile * 128, q0 = q_tile * 128;
 
     const uint8_t* pbase = a.p;

@@ -402,11 +402,15 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
     // adjacent 128-byte pieces of every transposed row and four consecutive row bands of the row-scaled copy, which its L2
     // hands to memory as longer runs than the 128-byte pieces of a plain grid (adjacent column tiles on eight different
     // XCDs): 103 -> 95 us on [16384, 7168].
-    const int64_t nt = KB * MB, per_xcd = (nt + 7) / 8;
-    const int64_t logical = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if ((int64_t)(blockIdx.x >> 3) >= per_xcd || logical >= nt) return;
-    const int64_t band = logical / (4 * KB), in_band = logical % (4 * KB), band_h = MB - band * 4 < 4 ? MB - band * 4 : 4;
-    const int64_t tr = band * 4 + in_band % band_h, tc = in_band / band_h;
+    // (32-bit arithmetic: the host admits at most 2^31 tiles, and four 64-bit divisions are several hundred dependent
+    // scalar instructions in front of every tile)
+    const uint32_t nt = (uint32_t)(KB * MB), per_xcd = (nt + 7u) / 8u;
+    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if ((blockIdx.x >> 3) >= per_xcd || logical >= nt) return;
+    const uint32_t band_w = 4u * (uint32_t)KB, band = logical / band_w, in_band = logical - band * band_w;
+    const uint32_t band_h = (uint32_t)MB - band * 4u < 4u ? (uint32_t)MB - band * 4u : 4u;
+    const uint32_t tc32 = in_band / band_h;
+    const int64_t tr = band * 4u + (in_band - tc32 * band_h), tc = tc32;
     const int64_t row0 = tr * 128, col0 = tc * 128;
     const bool want_rows = q != nullptr;
 
@@ -496,9 +500,12 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
     // destination of the transposed tile
     int64_t qt_base, ldq;
     if (SPLIT) {
-        // expert of this row tile: linear scan of the prefix table (E <= 256, uniform per workgroup)
+        // expert of this row tile: the last e with tile_start[e] <= tr, by bisection of the prefix table (E <= 256, uniform
+        // per workgroup; a linear scan is up to 255 dependent scalar loads)
         int e = 0;
-        while (e + 1 < sp.E && (int64_t)sp.tile_start[e + 1] <= tr) ++e;
+#pragma unroll
+        for (int step = 128; step >= 1; step >>= 1)
+            if (e + step < sp.E && (int64_t)sp.tile_start[e + step] <= tr) e += step;
         const int64_t off = (int64_t)sp.tile_start[e] * 128;                       // rows before this expert
         const int64_t Me = (int64_t)(sp.tile_start[e + 1] - sp.tile_start[e]) * 128;
         qt_base = off * K + (row0 - off);      // + c*Me
@@ -530,17 +537,19 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
 // dequantizers
 // ---------------------------------------------------------------------------------------------
 
-// 1x128 dequant: one thread per 8 bytes
-template <int LAYOUT>
+// 1x128 dequant: one thread per 8 bytes.  IDX: integer type of the index arithmetic, 32-bit whenever the tensor allows it
+// (a 64-bit division per thread is emulated and costs more than the data movement)
+template <int LAYOUT, typename IDX>
 __global__ __launch_bounds__(256) void k_act_dequant(const uint8_t* __restrict__ q, const float* __restrict__ s, int64_t M,
                                                      int64_t K, uint16_t* __restrict__ out) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;   // 8-byte chunk index
-    const int64_t cpr = K / 8;
-    if (idx >= M * cpr) return;
-    const int64_t r = idx / cpr, c8 = idx % cpr;
+    const IDX idx = (IDX)blockIdx.x * 256 + threadIdx.x;   // 8-byte chunk index
+    const IDX cpr = (IDX)(K / 8);
+    if ((int64_t)idx >= M * (K / 8)) return;
+    const IDX r32 = idx / cpr, c8 = idx - r32 * cpr;
+    const int64_t r = r32;
     const int64_t kb = c8 / 16, KB = K / 128;
     const float sc = LAYOUT == 0 ? s[r * KB + kb] : s[kb * M + r];
-    const uint2 w = ld8(q + idx * 8);
+    const uint2 w = ld8(q + (int64_t)idx * 8);
     float f[8];
     e4m3x4_to_f32(w.x, f);
     e4m3x4_to_f32(w.y, f + 4);
@@ -548,7 +557,7 @@ __global__ __launch_bounds__(256) void k_act_dequant(const uint8_t* __restrict__
     for (int j = 0; j < 8; ++j) f[j] *= sc;
     uint4 o;
     o.x = pack_bf16(f[0], f[1]); o.y = pack_bf16(f[2], f[3]); o.z = pack_bf16(f[4], f[5]); o.w = pack_bf16(f[6], f[7]);
-    st16(out + idx * 8, o);
+    st16(out + (int64_t)idx * 8, o);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -895,8 +904,13 @@ extern "C" int pf8_act_dequant(const uint8_t* q, const float* s, int scale_layou
     PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 or 1");
     const int64_t chunks = M * (K / 8);
     dim3 grid((unsigned)((chunks + 255) / 256)), block(256);
-    if (scale_layout == 0) hipLaunchKernelGGL(k_act_dequant<0>, grid, block, 0, (hipStream_t)stream, q, s, M, K, out);
-    else hipLaunchKernelGGL(k_act_dequant<1>, grid, block, 0, (hipStream_t)stream, q, s, M, K, out);
+    if (chunks < 0x7FFFFF00ll) {
+        if (scale_layout == 0) hipLaunchKernelGGL((k_act_dequant<0, uint32_t>), grid, block, 0, (hipStream_t)stream, q, s, M, K, out);
+        else hipLaunchKernelGGL((k_act_dequant<1, uint32_t>), grid, block, 0, (hipStream_t)stream, q, s, M, K, out);
+    } else {
+        if (scale_layout == 0) hipLaunchKernelGGL((k_act_dequant<0, int64_t>), grid, block, 0, (hipStream_t)stream, q, s, M, K, out);
+        else hipLaunchKernelGGL((k_act_dequant<1, int64_t>), grid, block, 0, (hipStream_t)stream, q, s, M, K, out);
+    }
     return pf8_check_launch(__func__);
 }
 
