@@ -7,6 +7,7 @@ kernel on the current stream.  There is no CPU path: a CPU tensor raises.
 """
 from __future__ import annotations
 
+import collections.abc
 import ctypes as C
 from typing import List, Optional, Sequence, Tuple
 
@@ -342,6 +343,48 @@ def fused_weighted_swiglu_act_quant(o1: torch.Tensor, probs: Optional[torch.Tens
 # ---------------------------------------------------------------------------------------------
 
 
+class _PackedExperts(collections.abc.Sequence):
+    """The per-expert tensors fused_transpose_split_quant returns (one q_t [K, M_e] or s_t [M_e/128, K] per expert, empty
+    tensors for experts without rows), as views of the one packed buffer the kernel wrote.  The views are made when an
+    entry is asked for: with 128 experts, slicing 256 of them up front costs more host time than the kernel runs.
+    `grouped_wgrad` takes the buffer as it is."""
+
+    def __init__(self, buf: torch.Tensor, rows: List[int], K: int, scales: bool):
+        self.buf, self.rows, self.K, self.scales = buf, rows, K, scales
+        self._start = None
+        self._views = {}
+
+    def __len__(self):
+        return len(self.rows)
+
+    def __add__(self, other):          # list + list, as code written for the reference's lists may do
+        return list(self) + list(other)
+
+    def __radd__(self, other):
+        return list(other) + list(self)
+
+    def __getitem__(self, i):
+        if isinstance(i, slice):
+            return [self[j] for j in range(*i.indices(len(self.rows)))]
+        if i < 0:
+            i += len(self.rows)
+        if not 0 <= i < len(self.rows):
+            raise IndexError(i)
+        v = self._views.get(i)
+        if v is None:
+            if self._start is None:
+                self._start = [0]
+                for r in self.rows:
+                    self._start.append(self._start[-1] + r)
+            off, r, K = self._start[i], self.rows[i], self.K
+            if self.scales:
+                v = self.buf[(off // 128) * K:((off + r) // 128) * K].view(r // 128, K)
+            else:
+                v = self.buf[off * K:(off + r) * K].view(K, r)
+            self._views[i] = v
+        return v
+
+
 def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], tokens_per_expert: Sequence[int],
                                 pow_2_scales: bool = False) -> Tuple[List[torch.Tensor], List[torch.Tensor]]:
     """Per-expert split along rows -> transpose -> 1x128 quantization along the token axis.
@@ -404,12 +447,7 @@ def fused_transpose_split_quant(x: torch.Tensor, scale: Optional[torch.Tensor], 
         qp = C.c_void_p(q_t.data_ptr() + off * K)
         sp = C.c_void_p(s_t.data_ptr() + (off // 128) * K * 4)
         _lib.call("pf8_transpose_split_quant", xp, xs_ptr, int(is_fp8), lay, arr, len(chunk), K, qp, sp, int(bool(pow_2_scales)), _stream())
-    qs, ss, off = [], [], 0
-    for r in rows:
-        qs.append(q_t[off * K:(off + r) * K].view(K, r))
-        ss.append(s_t[(off // 128) * K:((off + r) // 128) * K].view(r // 128, K))
-        off += r
-    return qs, ss
+    return _PackedExperts(q_t, rows, K, False), _PackedExperts(s_t, rows, K, True)
 
 
 def _transpose_split_quant_gathered(g: GatheredRows, rows: List[int], pow_2_scales: bool):
@@ -430,12 +468,7 @@ def _transpose_split_quant_gathered(g: GatheredRows, rows: List[int], pow_2_scal
         _lib.call("pf8_transpose_split_quant_gather", _p(g.tokens), _p(g.scale), int(g.tokens.dtype == FP8), 0, T,
                   C.c_void_p(src.data_ptr() + off * 4), arr, len(chunk), K,
                   C.c_void_p(q_t.data_ptr() + off * K), C.c_void_p(s_t.data_ptr() + (off // 128) * K * 4), int(bool(pow_2_scales)), _stream())
-    qs, ss, off = [], [], 0
-    for r in rows:
-        qs.append(q_t[off * K:(off + r) * K].view(K, r))
-        ss.append(s_t[(off // 128) * K:((off + r) // 128) * K].view(r // 128, K))
-        off += r
-    return qs, ss
+    return _PackedExperts(q_t, rows, K, False), _PackedExperts(s_t, rows, K, True)
 
 
 def quant_and_transpose_split(x: torch.Tensor, tokens_per_expert: Sequence[int], using_pow2_scale: bool = False,
@@ -471,12 +504,7 @@ def quant_and_transpose_split(x: torch.Tensor, tokens_per_expert: Sequence[int],
         arr = (C.c_int64 * len(rows))(*rows)
         _lib.call("pf8_quant_and_transpose_split", _p(x), arr, len(rows), K, _p(q), _p(s), 2 if ue8m0_scale else int(bool(using_pow2_scale)),
                   _p(q_t), _p(s_t), int(bool(pow_2_scales)), _stream())
-    qs, ss, off = [], [], 0
-    for r in rows:
-        qs.append(q_t[off * K:(off + r) * K].view(K, r))
-        ss.append(s_t[(off // 128) * K:((off + r) // 128) * K].view(r // 128, K))
-        off += r
-    return q, s, qs, ss
+    return q, s, _PackedExperts(q_t, rows, K, False), _PackedExperts(s_t, rows, K, True)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -625,13 +653,24 @@ def grouped_wgrad(a_t_list, sa_t_list, b_t_list, sb_t_list, out: torch.Tensor, a
     scales_pow2 says they were made with pow_2_scales=True (see fp8_gemm_blockwise).
     """
     E = len(a_t_list)
-    rows = [int(t.shape[1]) for t in a_t_list]
-    Kin = int(a_t_list[0].shape[0])
-    N = int(b_t_list[0].shape[0])
+    packed = all(isinstance(l, _PackedExperts) for l in (a_t_list, sa_t_list, b_t_list, sb_t_list))
+    if packed:
+        # the quantizer's own result objects: the packing is known, no view has to be made
+        rows = list(a_t_list.rows)
+        Kin, N = a_t_list.K, b_t_list.K
+        if list(b_t_list.rows) != rows or list(sa_t_list.rows) != rows or list(sb_t_list.rows) != rows or \
+                sa_t_list.K != Kin or sb_t_list.K != N or a_t_list.scales or b_t_list.scales or not sa_t_list.scales or not sb_t_list.scales:
+            raise ValueError("operands do not belong together (rows per expert, widths or roles differ)")
+    else:
+        rows = [int(t.shape[1]) for t in a_t_list]
+        Kin = int(a_t_list[0].shape[0])
+        N = int(b_t_list[0].shape[0])
     if tuple(out.shape) != (E, Kin, N) or out.dtype != torch.float32 or not out.is_contiguous():
         raise ValueError("out must be a contiguous float32 [E, Kin, N] tensor")
 
     def base(lst):
+        if packed:
+            return _p(lst.buf)
         t0 = lst[0]
         st = t0.untyped_storage()
         p = st.data_ptr() + t0.storage_offset() * t0.element_size()
