@@ -53,6 +53,8 @@ CASES = [
     (640, 384, [1024, 512, 0, 768], 8, 4),
     # every expert long: the 128x128-tile kernel is not launched at all
     (512, 512, [768, 1024], 8, 4),
+    # 256 experts (the most one call takes), one 256x256 tile each: most XCDs get an empty slice of every expert
+    (256, 256, [512] * 256, 8, 4),
     # the whole device, shapes of the MoE node's two weight gradients (I = 1408, H = 4096)
     (1408, 4096, [2048, 1024, 128, 3072, 0, 512, 1536], 0, 8),
     (4096, 2816, [2048, 1024, 128, 3072], 0, 8),
