@@ -207,3 +207,51 @@ def test_build_scratch_check_on_canned_remarks(monkeypatch):
         B.check_scratch(reworded)
     with pytest.raises(RuntimeError, match="resource remarks not found"):
         B.check_scratch(["clang: warning: something else"])
+
+
+def test_packed_expert_results_behave_like_the_lists_the_reference_returns():
+    """fused_transpose_split_quant hands its per-expert tensors out as views made on demand; code written for the
+    reference's Python lists (indexing, negative indices, slices, iteration, len, concatenation) must not notice."""
+    import torch
+
+    from paddleformers_amd.functional import _PackedExperts
+
+    rows, K = [256, 0, 128, 384], 4
+    q = torch.arange(sum(rows) * K, dtype=torch.int32)
+    s = torch.arange((sum(rows) // 128) * K, dtype=torch.float32)
+    pq, ps = _PackedExperts(q, rows, K, False), _PackedExperts(s, rows, K, True)
+    assert len(pq) == len(ps) == 4
+    off = 0
+    for e, r in enumerate(rows):
+        assert pq[e].shape == (K, r) and ps[e].shape == (r // 128, K)
+        assert torch.equal(pq[e].reshape(-1), q[off * K:(off + r) * K])
+        assert torch.equal(ps[e].reshape(-1), s[(off // 128) * K:((off + r) // 128) * K])
+        assert pq[e].data_ptr() == q.data_ptr() + off * K * 4 or r == 0        # views, not copies
+        off += r
+    assert pq[-1] is pq[3] and pq[1].numel() == 0
+    assert [t.shape for t in pq[1:3]] == [(K, 0), (K, 128)]
+    assert [t.shape[1] for t in pq] == rows
+    both = pq + ps
+    assert isinstance(both, list) and len(both) == 8 and both[4] is ps[0]
+    assert ([pq[0]] + ps)[1] is ps[0]
+    with pytest.raises(IndexError):
+        pq[4]
+    (only,), = [_PackedExperts(q[:128 * K], [128], K, False)]
+    assert only.shape == (K, 128)
+
+
+
+def test_build_scans_inline_assembly_for_scalar_address_hazards():
+    """A vector-memory instruction may read a scalar address register the vector unit wrote only five wait states later;
+    the compiler pads its own instructions but not inline assembly, so the build scans the device assembly itself."""
+    from paddleformers_amd.build import sgpr_address_hazards
+
+    bad = "\tv_readlane_b32 s0, v225, 47\n\tv_readlane_b32 s1, v225, 48\n\tglobal_atomic_add v196, v178, v198, s[0:1] sc0\n"
+    hz = sgpr_address_hazards(bad)
+    assert [(h[2], h[3]) for h in hz] == [(0, 1), (1, 0)]
+    padded = "\tv_readlane_b32 s0, v225, 47\n\tv_readlane_b32 s1, v225, 48\n\ts_nop 4\n\tglobal_atomic_add v196, v178, v198, s[0:1] sc0\n"
+    assert sgpr_address_hazards(padded) == []
+    far = "\tv_readfirstlane_b32 s4, v1\n" + "\tv_mov_b32_e32 v2, v3\n" * 5 + "\tglobal_load_dwordx4 v[0:3], v8, s[4:5]\n"
+    assert sgpr_address_hazards(far) == []
+    near = "\tv_readfirstlane_b32 s4, v1\n" + "\tv_mov_b32_e32 v2, v3\n" * 4 + "\tglobal_load_dwordx4 v[0:3], v8, s[4:5]\n"
+    assert len(sgpr_address_hazards(near)) == 1
