@@ -387,36 +387,40 @@ __device__ __forceinline__ void load_patch_packed(const TileSrc& src, int64_t ro
 // Per element the kernel spends one masked copy, two packed-u16 max (row and column amax), one
 // unpack and two reciprocal-based quantizations; the 128 row scales and 128 column scales are each computed
 // once (threads 0..127 / 128..255) and handed round through LDS instead of sixteen times over.
+// LDS of one tile's quantization: the transposed byte tile, the per-wave packed column maxima, the row maxima and
+// (s, 1/s, -, slow) for rows 0..127 / columns 128..255
+struct RowColLds {
+    uint32_t t[128 * LDT];
+    uint32_t cm[4 * 64];
+    uint32_t rm[128];
+    float4 sc[256];
+};
+
+// expert of row tile tr: the last e with tile_start[e] <= tr, by bisection of the prefix table (E <= 256, uniform per
+// workgroup; a linear scan is up to 255 dependent scalar loads)
+__device__ __forceinline__ int split_expert_of(const SplitArgs& sp, int64_t tr) {
+    int e = 0;
+#pragma unroll
+    for (int step = 128; step >= 1; step >>= 1)
+        if (e + step < sp.E && (int64_t)sp.tile_start[e + step] <= tr) e += step;
+    return e;
+}
+
+// The quantization of one tile whose packed bf16 patch the thread holds in w (rows 8g..8g+7, columns 8l..8l+7 of tile
+// (tr, tc)), as k_quant_rowcol describes it.  Three barriers; a caller that runs it again on another patch needs none in
+// between (the arrays a call writes first are read last two barriers earlier).  SPLIT: e_known is the expert of the row
+// tile when the caller has looked it up already (-1: looked up here); the expert is returned.
 template <bool SPLIT, int LAYOUT>
-__global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M, int64_t K, uint8_t* __restrict__ q,
-                                                      float* __restrict__ s, uint8_t* __restrict__ qt, float* __restrict__ st,
-                                                      SplitArgs sp, int pow2) {
-    __shared__ uint32_t lds_t[128 * LDT];      // transposed byte tile
-    __shared__ uint32_t lds_cm[4 * 64];        // per-wave packed column maxima
-    __shared__ uint32_t lds_rm[128];           // row maxima
-    __shared__ float4 lds_sc[256];             // (s, 1/s, -, slow) for rows 0..127, columns 128..255
+__device__ __forceinline__ int quant_rowcol_tile(const uint4 (&w)[8], int64_t tr, int64_t tc, int64_t M, int64_t K, uint8_t* __restrict__ q,
+                                                  float* __restrict__ s, uint8_t* __restrict__ qt, float* __restrict__ st,
+                                                  const SplitArgs& sp, int pow2, bool want_rows, RowColLds& L, int e_known = -1) {
+    uint32_t* const lds_t = L.t;
+    uint32_t* const lds_cm = L.cm;
+    uint32_t* const lds_rm = L.rm;
+    float4* const lds_sc = L.sc;
     const int tid = threadIdx.x, g = tid >> 4, l = tid & 15, wave = tid >> 6, lane = tid & 63;
     const int64_t KB = K / 128, MB = M / 128;
-    // Consecutive workgroups go round-robin to the 8 XCDs: every XCD gets a contiguous run of tiles, walked in bands of four
-    // row tiles x all column tiles, row tile fastest.  The four workgroups that run side by side on an XCD then write four
-    // adjacent 128-byte pieces of every transposed row and four consecutive row bands of the row-scaled copy, which its L2
-    // hands to memory as longer runs than the 128-byte pieces of a plain grid (adjacent column tiles on eight different
-    // XCDs): 103 -> 95 us on [16384, 7168].
-    // (32-bit arithmetic: the host admits at most 2^31 tiles, and four 64-bit divisions are several hundred dependent
-    // scalar instructions in front of every tile)
-    const uint32_t nt = (uint32_t)(KB * MB), per_xcd = (nt + 7u) / 8u;
-    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-    if ((blockIdx.x >> 3) >= per_xcd || logical >= nt) return;
-    const uint32_t band_w = 4u * (uint32_t)KB, band = logical / band_w, in_band = logical - band * band_w;
-    const uint32_t band_h = (uint32_t)MB - band * 4u < 4u ? (uint32_t)MB - band * 4u : 4u;
-    const uint32_t tc32 = in_band / band_h;
-    const int64_t tr = band * 4u + (in_band - tc32 * band_h), tc = tc32;
     const int64_t row0 = tr * 128, col0 = tc * 128;
-    const bool want_rows = q != nullptr;
-
-    uint4 w[8];
-    load_patch_packed(src, row0, col0, g, l, w);
-
     // ---- amax on the packed magnitudes ----
     uint32_t cmx = 0, cmy = 0, cmz = 0, cmw = 0;
 #pragma unroll
@@ -499,13 +503,9 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
 
     // destination of the transposed tile
     int64_t qt_base, ldq;
+    int e = e_known;
     if (SPLIT) {
-        // expert of this row tile: the last e with tile_start[e] <= tr, by bisection of the prefix table (E <= 256, uniform
-        // per workgroup; a linear scan is up to 255 dependent scalar loads)
-        int e = 0;
-#pragma unroll
-        for (int step = 128; step >= 1; step >>= 1)
-            if (e + step < sp.E && (int64_t)sp.tile_start[e + step] <= tr) e += step;
+        if (e < 0) e = split_expert_of(sp, tr);
         const int64_t off = (int64_t)sp.tile_start[e] * 128;                       // rows before this expert
         const int64_t Me = (int64_t)(sp.tile_start[e + 1] - sp.tile_start[e]) * 128;
         qt_base = off * K + (row0 - off);      // + c*Me
@@ -531,6 +531,131 @@ __global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M,
             for (int j = 0; j < 8; ++j) st[(col0 + 8 * l + j) * MB + tr] = cs[j];
         }
     }
+    return e;
+}
+
+template <bool SPLIT, int LAYOUT>
+__global__ __launch_bounds__(256, 4) void k_quant_rowcol(TileSrc src, int64_t M, int64_t K, uint8_t* __restrict__ q,
+                                                      float* __restrict__ s, uint8_t* __restrict__ qt, float* __restrict__ st,
+                                                      SplitArgs sp, int pow2) {
+    __shared__ RowColLds L;
+    const int tid = threadIdx.x, g = tid >> 4, l = tid & 15;
+    const int64_t KB = K / 128, MB = M / 128;
+    // Consecutive workgroups go round-robin to the 8 XCDs: every XCD gets a contiguous run of tiles, walked in bands of four
+    // row tiles x all column tiles, row tile fastest.  The four workgroups that run side by side on an XCD then write four
+    // adjacent 128-byte pieces of every transposed row and four consecutive row bands of the row-scaled copy, which its L2
+    // hands to memory as longer runs than the 128-byte pieces of a plain grid (adjacent column tiles on eight different
+    // XCDs): 103 -> 95 us on [16384, 7168].
+    // (32-bit arithmetic: the host admits at most 2^31 tiles, and four 64-bit divisions are several hundred dependent
+    // scalar instructions in front of every tile)
+    const uint32_t nt = (uint32_t)(KB * MB), per_xcd = (nt + 7u) / 8u;
+    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if ((blockIdx.x >> 3) >= per_xcd || logical >= nt) return;
+    const uint32_t band_w = 4u * (uint32_t)KB, band = logical / band_w, in_band = logical - band * band_w;
+    const uint32_t band_h = (uint32_t)MB - band * 4u < 4u ? (uint32_t)MB - band * 4u : 4u;
+    const uint32_t tc32 = in_band / band_h;
+    const int64_t tr = band * 4u + (in_band - tc32 * band_h), tc = tc32;
+    uint4 w[8];
+    load_patch_packed(src, tr * 128, tc * 128, g, l, w);
+    quant_rowcol_tile<SPLIT, LAYOUT>(w, tr, tc, M, K, q, s, qt, st, sp, pow2, q != nullptr, L);
+}
+
+// makes the four words values the compiler has to hold in registers at this point of the program
+__device__ __forceinline__ void pin_words(uint4& w) {
+    asm volatile("" : "+v"(w.x), "+v"(w.y), "+v"(w.z), "+v"(w.w));
+}
+
+// SwiGLU backward with probs on one 128x128 tile of the [M, I] grid, its three results quantized where they are made:
+// do1 = [d gate | d up] ([M, 2I]) row-scaled (q, s) and column-scaled, transposed per expert (qt, st); o2_s ([M, I])
+// column-scaled, transposed per expert (oqt, ost).  Every value takes the arithmetic of k_swiglu_bwd and is rounded to
+// bf16 before it is quantized, so the bytes and scales are those of k_quant_rowcol<true, 1> on the tensors k_swiglu_bwd
+// writes; neither tensor exists in memory here.  probs_grad leaves as one partial sum per row and column tile
+// (pg_part [I/128, M]) that k_sum_row_partials adds up in the order of the tiles.
+__global__ __launch_bounds__(256, 3) void k_swiglu_bwd_quant(const uint16_t* __restrict__ o1, const uint16_t* __restrict__ do2_s,
+                                                          const float* __restrict__ probs, int64_t M, int64_t I,
+                                                          uint8_t* __restrict__ q, float* __restrict__ s, uint8_t* __restrict__ qt,
+                                                          float* __restrict__ st, uint8_t* __restrict__ oqt, float* __restrict__ ost,
+                                                          float* __restrict__ pg_part, SplitArgs sp, int pow2) {
+    __shared__ RowColLds L;
+    const int tid = threadIdx.x, g = tid >> 4, l = tid & 15;
+    const int64_t IB = I / 128, MB = M / 128;
+    // tile order of k_quant_rowcol: a contiguous run of tiles per XCD, bands of four row tiles, row tile fastest
+    const uint32_t nt = (uint32_t)(IB * MB), per_xcd = (nt + 7u) / 8u;
+    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if ((blockIdx.x >> 3) >= per_xcd || logical >= nt) return;
+    const uint32_t band_w = 4u * (uint32_t)IB, band = logical / band_w, in_band = logical - band * band_w;
+    const uint32_t band_h = (uint32_t)MB - band * 4u < 4u ? (uint32_t)MB - band * 4u : 4u;
+    const uint32_t tc32 = in_band / band_h;
+    const int64_t tr = band * 4u + (in_band - tc32 * band_h), tc = tc32;
+    const int64_t r0 = tr * 128 + 8 * g, c0 = tc * 128 + 8 * l;       // this thread's first row and column
+
+    uint4 wg[8], wu[8], wd[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        wg[i] = ld16(o1 + (r0 + i) * 2 * I + c0);
+        wu[i] = ld16(o1 + (r0 + i) * 2 * I + I + c0);
+        wd[i] = ld16(do2_s + (r0 + i) * I + c0);
+    }
+    const float4 p0 = *reinterpret_cast<const float4*>(probs + r0), p1 = *reinterpret_cast<const float4*>(probs + r0 + 4);
+    const float pr[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+    const int e = split_expert_of(sp, tr);
+    const ExpPoly poly = exp_poly_in_registers();
+
+    uint4 a[8], b[8], o[8];       // d gate, d up and o2_s of the patch, packed bf16
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float gv[8], uv[8], dv[8], dg[8], du[8], os[8];
+        unpack8(wg[i], gv);
+        unpack8(wu[i], uv);
+        unpack8(wd[i], dv);
+        const float p = pr[i];
+        float pg = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const SiluSigmoid ss = silu_and_sigmoid(gv[j], poly);
+            const float sl = ss.silu;
+            const float o2f = round_bf16(sl * uv[j]);
+            os[j] = o2f * p;
+            const float do2 = round_bf16(dv[j] * p);
+            pg += dv[j] * o2f;
+            const float sig = ss.sigmoid;
+            const float t1 = 1.0f - sig;
+            const float t2 = gv[j] * t1;
+            const float t3 = 1.0f + t2;
+            const float t4 = sig * t3;
+            const float t5 = do2 * uv[j];
+            dg[j] = t5 * t4;
+            du[j] = do2 * sl;
+        }
+        a[i].x = pack_bf16(dg[0], dg[1]); a[i].y = pack_bf16(dg[2], dg[3]); a[i].z = pack_bf16(dg[4], dg[5]); a[i].w = pack_bf16(dg[6], dg[7]);
+        b[i].x = pack_bf16(du[0], du[1]); b[i].y = pack_bf16(du[2], du[3]); b[i].z = pack_bf16(du[4], du[5]); b[i].w = pack_bf16(du[6], du[7]);
+        o[i].x = pack_bf16(os[0], os[1]); o[i].y = pack_bf16(os[2], os[3]); o[i].z = pack_bf16(os[4], os[5]); o[i].w = pack_bf16(os[6], os[7]);
+        // the packed words are made here: left to itself the compiler sinks the arithmetic behind them into the three
+        // quantizations and keeps every element's intermediate values alive instead (hundreds of registers)
+        pin_words(a[i]);
+        pin_words(b[i]);
+        pin_words(o[i]);
+        // the row's 128 terms of this tile: eight per lane, then the sixteen lanes of the row group
+        pg += __shfl_xor(pg, 1);
+        pg += __shfl_xor(pg, 2);
+        pg += __shfl_xor(pg, 4);
+        pg += __shfl_xor(pg, 8);
+        if (l == i) pg_part[tc * M + r0 + i] = pg;
+        // one row at a time: interleaved, the eight rows' temporaries do not fit the register file next to the patches
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    quant_rowcol_tile<true, 1>(a, tr, tc, M, 2 * I, q, s, qt, st, sp, pow2, true, L, e);
+    quant_rowcol_tile<true, 1>(b, tr, tc + IB, M, 2 * I, q, s, qt, st, sp, pow2, true, L, e);
+    quant_rowcol_tile<true, 1>(o, tr, tc, M, I, nullptr, nullptr, oqt, ost, sp, pow2 & 1, false, L, e);
+}
+
+// out[r] = part[0][r] + part[1][r] + ... + part[n-1][r], added in that order
+__global__ __launch_bounds__(256) void k_sum_row_partials(const float* __restrict__ part, int n, int64_t M, float* __restrict__ out) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= M) return;
+    float acc = part[r];
+    for (int k = 1; k < n; ++k) acc += part[(int64_t)k * M + r];
+    out[r] = acc;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -891,6 +1016,42 @@ extern "C" int pf8_swiglu_weighted_bwd(const uint16_t* o1, const uint16_t* do2_s
     PF8_REQUIRE(PF8_ALIGNED16(o1) && PF8_ALIGNED16(do2_s) && PF8_ALIGNED16(do1) && PF8_ALIGNED16(o2_s), "pointers must be 16-byte aligned");
     dim3 grid((unsigned)((M + 3) / 4)), block(256);
     hipLaunchKernelGGL(k_swiglu_bwd, grid, block, 0, (hipStream_t)stream, o1, do2_s, probs, M, I, do1, probs_grad, o2_s);
+    return pf8_check_launch(__func__);
+}
+
+extern "C" int pf8_swiglu_weighted_bwd_quant(const uint16_t* o1, const uint16_t* do2_s, const float* probs, const int64_t* rows_per_expert,
+                                             int E, int64_t I, uint8_t* do1_q, float* do1_s, int pow2_rows, uint8_t* do1_q_t,
+                                             float* do1_s_t, uint8_t* o2s_q_t, float* o2s_s_t, int pow2_t, float* probs_grad,
+                                             float* pg_partial, pf8_stream_t stream) {
+    PF8_REQUIRE(E >= 0 && I >= 0, "negative shape");
+    PF8_REQUIRE(I % 128 == 0, "I must be a multiple of 128");
+    PF8_REQUIRE(E <= 256, "at most 256 experts per call");
+    if (E == 0) return PF8_OK;
+    PF8_REQUIRE(rows_per_expert, "null pointer");
+    SplitArgs sp = {};
+    int64_t total = 0;
+    for (int e = 0; e < E; ++e) {
+        PF8_REQUIRE(rows_per_expert[e] >= 0 && rows_per_expert[e] % 128 == 0, "rows_per_expert entries must be non-negative multiples of 128");
+        sp.tile_start[e] = (int32_t)(total / 128);
+        total += rows_per_expert[e];
+    }
+    PF8_REQUIRE(total / 128 <= 65535 && (2 * I / 128) * (total / 128) <= 0x7FFFFFF0ll, "too many rows");
+    sp.tile_start[E] = (int32_t)(total / 128);
+    sp.E = E;
+    if (total == 0) return PF8_OK;
+    PF8_REQUIRE(I > 0, "I must be positive");
+    PF8_REQUIRE(o1 && do2_s && probs && do1_q && do1_s && do1_q_t && do1_s_t && o2s_q_t && o2s_s_t && probs_grad && pg_partial, "null pointer");
+    PF8_REQUIRE(PF8_ALIGNED16(o1) && PF8_ALIGNED16(do2_s) && PF8_ALIGNED16(probs) && PF8_ALIGNED16(do1_q) && PF8_ALIGNED16(do1_q_t) &&
+                PF8_ALIGNED16(do1_s_t) && PF8_ALIGNED16(o2s_q_t) && PF8_ALIGNED16(o2s_s_t), "pointers must be 16-byte aligned");
+    // pow2 bits of k_quant_rowcol: 1 = transposed copies, 2 = row-scaled copy, 4 = its scales as UE8M0 bytes [2I/128, M]
+    const int pow2_bits = (pow2_t ? 1 : 0) | (pow2_rows ? 2 : 0) | (pow2_rows == 2 ? 4 : 0);
+    dim3 grid((unsigned)(((I / 128) * (total / 128) + 7) / 8 * 8)), block(256);
+    hipLaunchKernelGGL(k_swiglu_bwd_quant, grid, block, 0, (hipStream_t)stream, o1, do2_s, probs, total, I, do1_q, do1_s, do1_q_t, do1_s_t,
+                       o2s_q_t, o2s_s_t, pg_partial, sp, pow2_bits);
+    int rc = pf8_check_launch(__func__);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_sum_row_partials, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, pg_partial,
+                       (int)(I / 128), total, probs_grad);
     return pf8_check_launch(__func__);
 }
 

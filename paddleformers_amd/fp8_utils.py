@@ -616,6 +616,9 @@ class FP8GroupGemmMlpFunctionNode:
         # backward quantizes out_grad and do1 twice each (row-wise for the dgrad GEMM, transposed per expert
         # for the wgrad GEMM); with this set both come from one read of the gradient, bit-identical
         self.fuse_bwd_quant = True
+        # ... and the SwiGLU backward writes do1 and o2_s in their quantized forms only (one kernel in place of the SwiGLU
+        # backward and the quantizations of its two results): same bytes and scales, probs_grad summed in another order
+        self.fuse_bwd_swiglu_quant = True
         # forward may run the up+gate grouped GEMM with SwiGLU, the probability factor and the 1x128 requantization in
         # its epilogue (one launch, bit-identical to the two calls of fp8_utils.py:949-954 and :981-987).  Measured on
         # config 3 the one launch takes as long as the two (SwiGLU is bound by the vector ALU and the persistent GEMM
@@ -768,8 +771,10 @@ class FP8GroupGemmMlpFunctionNode:
                 self._grouped_gemm(o2_fp8, o2_scale, w2_quant, w2_scale, o3, m_indices if self.fwd_subbatch else self.m_indices, w2_cache)
         return o3
 
-    def bwd_dowm_input(self, expert_w2, unzipped_grad, o1, tokens_per_expert, m_indices=None, unzipped_probs=None):
-        """do2_s [m_sum, I] = do3 . w2^T, then the SwiGLU backward (fp8_utils.py:1011-1052)."""
+    def bwd_dowm_input(self, expert_w2, unzipped_grad, o1, tokens_per_expert, m_indices=None, unzipped_probs=None, quantized=False):
+        """do2_s [m_sum, I] = do3 . w2^T, then the SwiGLU backward (fp8_utils.py:1011-1052).  quantized: do1 comes back as
+        ((fp8, scale), (fp8_t list, scale_t list)), its row-wise and per-expert transposed quantizations, and o2_s as its
+        (fp8_t list, scale_t list), the forms bwd_gate_up_input, bwd_gate_up_weight and bwd_down_weight take."""
         bw_w2_quant, bw_w2_scale, bw_w2_cache = self._stacked(expert_w2, False, len(expert_w2))
         if isinstance(unzipped_grad, F8.GatheredRows):
             # gradient rows that were never copied: quantized per token, read through their source map where the GEMM can
@@ -793,6 +798,10 @@ class FP8GroupGemmMlpFunctionNode:
             else:
                 self._grouped_gemm(unzipped_grad_fp8, unzipped_grad_scale, bw_w2_quant, bw_w2_scale, do2_s,
                                    m_indices if self.bwd_subbatch else self.m_indices, bw_w2_cache)
+        if quantized:
+            d_fp8, d_scale, d_t_fp8, d_t_scale, o_t_fp8, o_t_scale, probs_grad = F8.swiglu_weighted_bwd_quant(
+                o1, do2_s, unzipped_probs, tokens_per_expert, self.use_ue8m0, True, self._scale_bytes)
+            return ((d_fp8, d_scale.T), (d_t_fp8, d_t_scale)), (o_t_fp8, o_t_scale), probs_grad
         do1, probs_grad, o2_s = F8.fused_swiglu_weighted_bwd(o1, do2_s, unzipped_probs)
         return do1, o2_s, probs_grad
 
@@ -1002,12 +1011,16 @@ class FP8GroupGemmMlpFunctionNode:
             g_fp8, g_scale, g_t_fp8, g_t_scale = F8.quant_and_transpose_split(out_grad, tokens_per_expert, self.use_ue8m0, True,
                                                                               ue8m0_scale=self._scale_bytes)
             out_grad, do3_t = (g_fp8, g_scale.T), (g_t_fp8, g_t_scale)
+        fuse_act = (fuse and self.fuse_bwd_swiglu_quant and o1.shape[1] % 256 == 0 and unzipped_probs is not None and
+                    (do3_t is not None or isinstance(out_grad, tuple)))
         do1, o2_s, probs_grad = self.bwd_dowm_input(expert_w2, out_grad, o1, tokens_per_expert, unzipped_probs=unzipped_probs,
-                                                    m_indices=m_indices)
+                                                    m_indices=m_indices, quantized=fuse_act)
         del o1
         self.o1 = None
         do1_rows = do1_t = do1
-        if fuse:
+        if fuse_act:
+            do1_rows, do1_t = do1
+        elif fuse:
             d_fp8, d_scale, d_t_fp8, d_t_scale = F8.quant_and_transpose_split(do1, tokens_per_expert, self.use_ue8m0, True,
                                                                               ue8m0_scale=self._scale_bytes)
             do1_rows, do1_t = (d_fp8, d_scale.T), (d_t_fp8, d_t_scale)

@@ -601,6 +601,60 @@ def fused_swiglu_weighted_bwd(o1: torch.Tensor, do2_s: torch.Tensor, probs: torc
     return do1, pg, o2s
 
 
+def swiglu_weighted_bwd_quant(o1: torch.Tensor, do2_s: torch.Tensor, probs: torch.Tensor, tokens_per_expert: Sequence[int],
+                              using_pow2_scale: bool = False, pow_2_scales: bool = True, ue8m0_scale: bool = False):
+    """fused_swiglu_weighted_bwd(o1, do2_s, probs) followed by quant_and_transpose_split(do1, tokens_per_expert,
+    using_pow2_scale, pow_2_scales, ue8m0_scale) and fused_transpose_split_quant(o2_s, None, tokens_per_expert,
+    pow_2_scales) (transformers/fp8_utils.py:1049-1052, then :1073-1079, :1168 and :1115), from one read of o1 and do2_s:
+    the bf16 do1 and o2_s are never written.  Returns (do1_q [M,2I], do1_s [2I/128,M], do1_q_t list, do1_s_t list,
+    o2s_q_t list, o2s_s_t list, probs_grad [M]); the quantized forms are bit-identical to the separate calls',
+    probs_grad agrees with theirs to the rounding of a sum taken in another order.  At most 256 experts."""
+    for t, n in ((o1, "o1"), (do2_s, "do2_s"), (probs, "probs")):
+        _dev(t, n)
+    if o1.dim() != 2 or do2_s.dim() != 2 or o1.dtype != torch.bfloat16 or do2_s.dtype != torch.bfloat16:
+        raise ValueError("o1 and do2_s must be 2-D bfloat16 tensors")
+    o1 = o1.contiguous()
+    do2_s = do2_s.contiguous()
+    M, I2 = o1.shape
+    I = I2 // 2
+    if I2 % 2 != 0 or tuple(do2_s.shape) != (M, I):
+        raise ValueError(f"do2_s must be [{M}, {I2 // 2}] for o1 [{M}, {I2}]")
+    if I % 128 != 0:
+        raise ValueError(f"I must be divisible by 128, got {I}")
+    rows = [int(t) for t in tokens_per_expert]
+    if sum(rows) != M:
+        raise ValueError(f"tokens_per_expert sums to {sum(rows)} but o1 has {M} rows")
+    if any(r % 128 != 0 or r < 0 for r in rows):
+        raise ValueError("every tokens_per_expert entry must be a non-negative multiple of 128")
+    if len(rows) > 256:
+        raise ValueError("at most 256 experts")
+    if ue8m0_scale and not using_pow2_scale:
+        raise ValueError("ue8m0_scale goes with using_pow2_scale=True")
+    probs = probs.reshape(-1).float().contiguous()
+    if probs.numel() != M:
+        raise ValueError("probs must have one entry per row")
+    if probs.data_ptr() % 16:
+        probs = probs.clone()
+    dev = o1.device
+    q = torch.empty((M, I2), dtype=FP8, device=dev)
+    s = torch.empty((I2 // 128, M), dtype=torch.uint8 if ue8m0_scale else torch.float32, device=dev)
+    q_t = torch.empty((I2 * M,), dtype=FP8, device=dev)
+    s_t = torch.empty(((M // 128) * I2,), dtype=torch.float32, device=dev)
+    oq_t = torch.empty((I * M,), dtype=FP8, device=dev)
+    os_t = torch.empty(((M // 128) * I,), dtype=torch.float32, device=dev)
+    pg = torch.empty((M,), dtype=torch.float32, device=dev)
+    if M and I:
+        part = torch.empty((I // 128, M), dtype=torch.float32, device=dev)
+        arr = (C.c_int64 * len(rows))(*rows)
+        _lib.call("pf8_swiglu_weighted_bwd_quant", _p(o1), _p(do2_s), _p(probs), arr, len(rows), I, _p(q), _p(s),
+                  2 if ue8m0_scale else int(bool(using_pow2_scale)), _p(q_t), _p(s_t), _p(oq_t), _p(os_t), int(bool(pow_2_scales)),
+                  _p(pg), _p(part), _stream())
+    else:
+        pg.zero_()
+    return (q, s, _PackedExperts(q_t, rows, I2, False), _PackedExperts(s_t, rows, I2, True),
+            _PackedExperts(oq_t, rows, I, False), _PackedExperts(os_t, rows, I, True), pg)
+
+
 # ---------------------------------------------------------------------------------------------
 # fp8_gemm_blockwise (weight-gradient GEMM)
 # ---------------------------------------------------------------------------------------------

@@ -42,7 +42,7 @@ class _Recorder:
     """Patches the operator mirrors the node calls so that every call is kept as (name, args, kwargs, result)."""
 
     F8_NAMES = ["fp8_quant_blockwise", "fused_weighted_swiglu_act_quant", "fused_transpose_split_quant",
-                "quant_and_transpose_split", "fused_swiglu_weighted_bwd", "grouped_wgrad"]
+                "quant_and_transpose_split", "fused_swiglu_weighted_bwd", "swiglu_weighted_bwd_quant", "grouped_wgrad"]
 
     def __init__(self):
         self.calls = []
@@ -286,6 +286,9 @@ def test_config5_forward_backward_at_full_size(ue8m0):
     o1 = _check_forward(rec, node, x, probs, rows, ue8m0, tag)
     x_fp8, x_scale = node.input_fp8, node.input_scale      # cached quantised input, scale a [M, K/128] view
 
+    # launch by launch in the reference's sequence (the SwiGLU backward writing bf16 do1 and o2_s); the node's default, one
+    # kernel that writes only their quantized forms, is held against this run at the end
+    node.fuse_bwd_swiglu_quant = False
     with _Recorder() as rec:
         dx, pg = node.backward(dout, probs, rows)
     names = [c[0] for c in rec.calls]
@@ -346,3 +349,19 @@ def test_config5_forward_backward_at_full_size(ue8m0):
     assert outs[(E, H, 2 * I)][1][4].data_ptr() == g1.data_ptr() and outs[(E, I, H)][1][4].data_ptr() == g2.data_ptr()
     _check_grouped_wgrad(outs[(E, H, 2 * I)], rows, f"{tag} dW1")
     _check_grouped_wgrad(outs[(E, I, H)], rows, f"{tag} dW2")
+    # the same backward with the SwiGLU backward fused into the quantizations of its results: dx and both weight gradients
+    # to the bit, probs_grad (summed per column tile, then over the tiles) to 1e-5 of the magnitudes of its terms
+    dw1, dw2 = g1.clone(), g2.clone()
+    g1.zero_()
+    g2.zero_()
+    node.fuse_bwd_swiglu_quant = True
+    node.forward(x, probs, rows)
+    with _Recorder() as rec:
+        dx_f, pg_f = node.backward(dout, probs, rows)
+    names = [c[0] for c in rec.calls]
+    assert names.count("swiglu_weighted_bwd_quant") == 1 and "fused_swiglu_weighted_bwd" not in names, names
+    assert names.count("quant_and_transpose_split") == 1 and names.count("grouped_wgrad") == 2, names
+    assert torch.equal(dx_f.view(torch.int16), dx.view(torch.int16)), f"{tag} dx with the fused SwiGLU backward"
+    assert torch.equal(g1, dw1) and torch.equal(g2, dw2), f"{tag} weight gradients with the fused SwiGLU backward"
+    terms = (do2_s.float().abs() * (o2_s.float().abs() / probs.clamp_min(1e-30))).sum(dim=1)
+    assert bool(((pg_f - pg).abs() <= 1e-5 * terms + 1e-30).all()), f"{tag} probs_grad with the fused SwiGLU backward"
