@@ -420,6 +420,11 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     prb = torch.rand((Mp, 1), device="cuda")
     ms = time_kernel(lambda: F8.fused_swiglu_weighted_bwd(o1b, d2b, prb), [()], 20, 3)
     out["swiglu_bwd_config5"] = dict(ms, bytes=Mp * I * 12 + Mp * 8)
+    # ... and the one kernel that writes do1 row-wise and transposed and o2_s transposed, all e4m3, in place of that launch
+    # and the two quantizations after it (reads 6 bytes per element of the [Mp, I] grid, writes 5, plus scales and probs_grad)
+    ms = time_kernel(lambda: F8.swiglu_weighted_bwd_quant(o1b, d2b, prb, rows, True, True, True), [()], 20, 3)
+    out["swiglu_bwd_quant_config5"] = dict(ms, bytes=Mp * I * 11 + Mp * (2 * I // 128) + (Mp // 128) * 3 * I * 4 + Mp * 8 +
+                                           2 * Mp * (I // 128) * 4)
     del o1b, d2b, prb
     # dense weight gradient of config 2: dW [7168, 4096] = x^T [7168, 8192] . dy^T [4096, 8192]^T, fp32 out
     Mw, Kw, Nw = 8192, 7168, 4096
