@@ -24,7 +24,7 @@ enum { PF8_NOTE_GROUPED_ORDER = 0, PF8_NOTE_MASKED_TABLE = 1 };
 // bytes (implemented next to that kernel; used by the UE8M0 entry point when a skewed expert load
 // makes 256-row tiles wasteful).  pair_list: DEVICE work-item list of the paired-tile kernel; this kernel
 // returns at once when that one takes the call (e8_paired_tiles_win).  cus: the compute-unit budget, read ONCE by
-// the caller for both launches so that they reach the same verdict.
+// the caller for both launches so that they reach the same decision.
 int pf8_launch_deep_ue8m0(const uint8_t* p, const uint8_t* q, const uint8_t* sp8, const uint8_t* sq8, int64_t ldsq, void* out,
                           int64_t Prows, int64_t Qrows, int64_t red, int E, const int32_t* m_indices, const int32_t* pair_list,
                           int cus, hipStream_t stream, const char* where);

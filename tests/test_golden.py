@@ -82,6 +82,16 @@ def test_quantizers_match_the_fixtures(gold):
     # a row sum of 256 fp32 products: the summation order is the kernel's own
     assert np.allclose(pg.cpu().numpy(), gold["swiglu_bwd_pg"], rtol=1e-5, atol=1e-7)
     _same(G.from_torch_bf16(o2s), gold["swiglu_bwd_o2s"], "swiglu backward o2_s")
+    # the backward that writes quantized forms only: the quantizations of the golden do1 and o2_s
+    fq, fs, fqt, fst, foqt, fost, fpg = F.swiglu_weighted_bwd_quant(o1, G.to_torch_bf16(gold["swiglu_bwd_do2"]), probs, [128], False, True)
+    eq, es = O.quant_1x128(gold["swiglu_bwd_do1"], 1)
+    _same(G.from_torch_fp8(fq), eq, "fused swiglu backward: do1 bytes")
+    _same(fs.cpu().numpy(), es, "fused swiglu backward: do1 scales")
+    for got_q, got_s, key in ((fqt, fst, "swiglu_bwd_do1"), (foqt, fost, "swiglu_bwd_o2s")):
+        etq, ets = O.transpose_split_quant(gold[key], None, [128], True)
+        _same(G.from_torch_fp8(got_q[0]), etq[0], f"fused swiglu backward: {key} transposed bytes")
+        _same(got_s[0].cpu().numpy(), ets[0], f"fused swiglu backward: {key} transposed scales")
+    assert np.allclose(fpg.cpu().numpy(), gold["swiglu_bwd_pg"], rtol=1e-5, atol=1e-7)
     rows = [int(r) for r in gold["split_rows"]]
     xs3 = G.to_torch_bf16(gold["split_x"])
     qs, ss = F.fused_transpose_split_quant(xs3, None, rows, True)
