@@ -327,6 +327,17 @@ def bench_other_gemms(iters=50, warmup=10, gemm_only=False):
     out["stack_quant_both_config3_w1"] = dict(ms, bytes=Ew * Hw * 2 * Iw * 4 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4)
     ms = time_kernel(lambda: (F8.fused_stack_transpose_quant(ws, False), F8.fused_stack_transpose_quant(ws, True)), [()], 20, 3)
     out["stack_quant_two_calls_config3_w1"] = dict(ms, bytes=Ew * Hw * 2 * Iw * 6 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4)
+    # ... with the fragment-major copies of both orientations (what the node's GEMMs read): written by the quantizer's own
+    # pass, and as the two re-ordering passes over its plain outputs that this replaces
+    ms = time_kernel(lambda: F8.fused_stack_quant_both(ws, fragment_major=True), [()], 20, 3)
+    out["stack_quant_both_fragment_major_config3_w1"] = dict(ms, bytes=Ew * Hw * 2 * Iw * 6 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4)
+
+    def quant_then_reorder():
+        q, s, qt, st = F8.fused_stack_quant_both(ws)
+        return deep_gemm.to_fragment_major(q.view(Ew, Hw, 2 * Iw)), deep_gemm.to_fragment_major(qt.view(Ew, 2 * Iw, Hw))
+
+    ms = time_kernel(quant_then_reorder, [()], 20, 3)
+    out["stack_quant_both_then_two_reorders_config3_w1"] = dict(ms, bytes=Ew * Hw * 2 * Iw * 8 + 2 * Ew * (Hw // 128) * (2 * Iw // 128) * 4)
     del ws
     torch.cuda.empty_cache()
     # checkpoint load: block-FP8 [32, 4096, 7168] (128x128 blocks, UE8M0 scales) -> bf16

@@ -88,6 +88,14 @@ int pf8_stack_transpose_quant(const uint16_t* const* w_list, int E, int64_t R, i
 int pf8_stack_quant_both(const uint16_t* const* w_list, int E, int64_t R, int64_t C, uint8_t* q,
                          float* s, uint8_t* q_t, float* s_t, int pow2, pf8_stream_t stream);
 
+/* pf8_stack_quant_both with the fragment-major copies of its two outputs made in the same pass (no counterpart in the
+ * reference, whose FP8 weight cache is read by deep_gemm only): q_fm / q_t_fm receive the bytes of q / q_t in the order
+ * pf8_weight_to_fragment_major gives them, what the *_fm GEMMs read.  Either may be NULL (an orientation whose shape those
+ * GEMMs do not take), not both.  Saves the two re-ordering passes per cached weight and optimizer step. */
+int pf8_stack_quant_both_fm(const uint16_t* const* w_list, int E, int64_t R, int64_t C, uint8_t* q, float* s,
+                            uint8_t* q_t, float* s_t, uint8_t* q_fm, uint8_t* q_t_fm, int pow2,
+                            pf8_stream_t stream);
+
 /* fused_weighted_swiglu_act_quant(o1, probs, using_pow2_scaling) -- transformers/fp8_utils.py:981-987;
  * un-fused definition ernie token_dispatcher/fp8_utils.py:996-1004.  o1 bf16 [M,2I] (gate first),
  * probs fp32 [M] or NULL -> q [M,I], s per scale_layout.  o2 (bf16 [M,I]) optionally receives the

@@ -26,6 +26,7 @@ SIGNATURES = {
     "pf8_quant_transpose": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _vp],
     "pf8_stack_transpose_quant": [_vp, _i32, _i64, _i64, _i32, _vp, _vp, _i32, _vp],
     "pf8_stack_quant_both": [_vp, _i32, _i64, _i64, _vp, _vp, _vp, _vp, _i32, _vp],
+    "pf8_stack_quant_both_fm": [_vp, _i32, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp],
     "pf8_swiglu_weighted_quant": [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i32, _i32, _vp],
     "pf8_transpose_split_quant": [_vp, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _vp, _i32, _vp],
     "pf8_transpose_split_quant_gather": [_vp, _vp, _i32, _i32, _i64, _vp, _vp, _i32, _i64, _vp, _vp, _i32, _vp],

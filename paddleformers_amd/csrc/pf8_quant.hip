@@ -274,13 +274,30 @@ struct StackArgs {
     const uint16_t* w[256];
 };
 
+// One staged 128x128 byte tile (row n of the LDS tile = weight row n0 + n, its 128 bytes = K block kb) written as the two
+// 8 KB fragment-major blocks it fills (the order pf8_gemm_fm.hip describes and k_weight_to_fm produces from the plain
+// bytes): chunk t = pf<<8 | kh<<7 | h<<6 | hh<<5 | x of a block is bytes 64 kh + 32 hh + 16 h .. + 15 of row 32 pf + x of its
+// 64-row panel.  wf: the expert's fragment-major matrix, KB its K blocks per row.  A workgroup writes 4 KB per pass.
+__device__ __forceinline__ void store_tile_fragment_major(const uint32_t* lds, uint8_t* __restrict__ wf, int64_t n0, int64_t KB, int64_t kb) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int ch = it * 256 + threadIdx.x;
+        const int panel = ch >> 9, pf = (ch >> 8) & 1, kh = (ch >> 7) & 1, h = (ch >> 6) & 1, hh = (ch >> 5) & 1, x = ch & 31;
+        const uint4 o = lds_get_row(lds, panel * 64 + pf * 32 + x, kh * 4 + hh * 2 + h);
+        st16(wf + ((n0 / 64 + panel) * KB + kb) * 8192 + (ch & 511) * 16, o);
+    }
+}
+
 // 128x128 block-scaled quantizer.  Source tile (tr, tc) of expert e; writes q (same orientation)
 // and/or qt (transposed).  STACK: sources come from a pointer table, outputs are stacked per expert.
-template <bool STACK>
+// FM: also the fragment-major copies of q and / or qt (q_fm, qt_fm; either may be null), made from the same registers.
+template <bool STACK, bool FM = false>
 __global__ __launch_bounds__(256) void k_quant_128x128(const uint16_t* __restrict__ w, StackArgs ptrs, int64_t R, int64_t C,
                                                        uint8_t* __restrict__ q, float* __restrict__ s, uint8_t* __restrict__ qt,
-                                                       float* __restrict__ st, int pow2) {
+                                                       float* __restrict__ st, int pow2, uint8_t* __restrict__ q_fm,
+                                                       uint8_t* __restrict__ qt_fm) {
     __shared__ uint32_t lds_t[128 * LDT];
+    __shared__ uint32_t lds_r[FM ? 128 * LDT : 1];
     __shared__ uint32_t lds4[4];
     const int tid = threadIdx.x, g = tid >> 4, l = tid & 15;
     const int64_t CB = C / 128, RB = R / 128;
@@ -304,6 +321,10 @@ __global__ __launch_bounds__(256) void k_quant_128x128(const uint16_t* __restric
         for (int i = 0; i < 8; ++i) {
             uint2 o = quant8(v[i], t);
             st8(q + ebase + (row0 + 8 * g + i) * C + col0 + 8 * l, o);
+            if (FM && q_fm) {
+                lds_r[(8 * g + i) * LDT + 2 * l] = o.x;
+                lds_r[(8 * g + i) * LDT + 2 * l + 1] = o.y;
+            }
         }
         if (tid == 0) s[e * RB * CB + tr * CB + tc] = t.s;
     }
@@ -323,6 +344,11 @@ __global__ __launch_bounds__(256) void k_quant_128x128(const uint16_t* __restric
             st16(qt + ebase + (col0 + c) * R + row0 + 16 * seg, o);
         }
         if (tid == 0) st[e * RB * CB + tc * RB + tr] = t.s;
+        if (FM && qt_fm) store_tile_fragment_major(lds_t, qt_fm + ebase, col0, RB, tr);     // [C, R]: weight rows = columns here
+    }
+    if (FM && q && q_fm) {
+        if (!qt) __syncthreads();              // with qt the barrier above has covered the row tile's writes as well
+        store_tile_fragment_major(lds_r, q_fm + ebase, row0, CB, tc);
     }
 }
 
@@ -839,7 +865,8 @@ extern "C" int pf8_quant_128x128(const uint16_t* w, int64_t R, int64_t C, uint8_
     PF8_REQUIRE(R / 128 <= 65535 && C / 128 <= 0x7FFFFFFF, "shape too large");
     dim3 grid((unsigned)(C / 128), (unsigned)(R / 128), 1), block(256);
     StackArgs none = {};
-    hipLaunchKernelGGL(k_quant_128x128<false>, grid, block, 0, (hipStream_t)stream, w, none, R, C, q, s, q_t, s_t, pow2);
+    hipLaunchKernelGGL(k_quant_128x128<false>, grid, block, 0, (hipStream_t)stream, w, none, R, C, q, s, q_t, s_t, pow2, (uint8_t*)nullptr,
+                       (uint8_t*)nullptr);
     return pf8_check_launch(__func__);
 }
 
@@ -862,10 +889,10 @@ extern "C" int pf8_stack_transpose_quant(const uint16_t* const* w_list, int E, i
         float* se = s + (int64_t)e0 * per_s;
         if (transpose)
             hipLaunchKernelGGL(k_quant_128x128<true>, grid, block, 0, (hipStream_t)stream, nullptr, a, R, C, (uint8_t*)nullptr,
-                               (float*)nullptr, qe, se, pow2);
+                               (float*)nullptr, qe, se, pow2, (uint8_t*)nullptr, (uint8_t*)nullptr);
         else
             hipLaunchKernelGGL(k_quant_128x128<true>, grid, block, 0, (hipStream_t)stream, nullptr, a, R, C, qe, se,
-                               (uint8_t*)nullptr, (float*)nullptr, pow2);
+                               (uint8_t*)nullptr, (float*)nullptr, pow2, (uint8_t*)nullptr, (uint8_t*)nullptr);
         int rc = pf8_check_launch(__func__);
         if (rc) return rc;
     }
@@ -888,7 +915,33 @@ extern "C" int pf8_stack_quant_both(const uint16_t* const* w_list, int E, int64_
         for (int i = 0; i < n; ++i) a.w[i] = w_list[e0 + i];
         dim3 grid((unsigned)(C / 128), (unsigned)(R / 128), (unsigned)n), block(256);
         hipLaunchKernelGGL(k_quant_128x128<true>, grid, block, 0, (hipStream_t)stream, nullptr, a, R, C,
-                           q + (int64_t)e0 * per_q, s + (int64_t)e0 * per_s, q_t + (int64_t)e0 * per_q, s_t + (int64_t)e0 * per_s, pow2);
+                           q + (int64_t)e0 * per_q, s + (int64_t)e0 * per_s, q_t + (int64_t)e0 * per_q, s_t + (int64_t)e0 * per_s, pow2,
+                           (uint8_t*)nullptr, (uint8_t*)nullptr);
+        int rc = pf8_check_launch(__func__);
+        if (rc) return rc;
+    }
+    return PF8_OK;
+}
+
+extern "C" int pf8_stack_quant_both_fm(const uint16_t* const* w_list, int E, int64_t R, int64_t C, uint8_t* q, float* s,
+                                       uint8_t* q_t, float* s_t, uint8_t* q_fm, uint8_t* q_t_fm, int pow2, pf8_stream_t stream) {
+    PF8_REQUIRE(E >= 0 && R >= 0 && C >= 0, "negative shape");
+    PF8_REQUIRE(R % 128 == 0 && C % 128 == 0, "R and C must be multiples of 128");
+    if (E == 0 || R == 0 || C == 0) return PF8_OK;
+    PF8_REQUIRE(w_list && q && s && q_t && s_t, "null pointer");
+    PF8_REQUIRE(q_fm || q_t_fm, "no fragment-major output asked for (pf8_stack_quant_both makes the plain copies)");
+    PF8_REQUIRE(PF8_ALIGNED16(q) && PF8_ALIGNED16(q_t) && PF8_ALIGNED16(q_fm) && PF8_ALIGNED16(q_t_fm), "pointers must be 16-byte aligned");
+    PF8_REQUIRE(R / 128 <= 65535, "shape too large");
+    for (int e = 0; e < E; ++e) PF8_REQUIRE(w_list[e] && PF8_ALIGNED16(w_list[e]), "null or misaligned weight pointer");
+    const int64_t per_q = R * C, per_s = (R / 128) * (C / 128);
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        const int n = E - e0 < 256 ? E - e0 : 256;
+        StackArgs a = {};
+        for (int i = 0; i < n; ++i) a.w[i] = w_list[e0 + i];
+        dim3 grid((unsigned)(C / 128), (unsigned)(R / 128), (unsigned)n), block(256);
+        hipLaunchKernelGGL((k_quant_128x128<true, true>), grid, block, 0, (hipStream_t)stream, nullptr, a, R, C,
+                           q + (int64_t)e0 * per_q, s + (int64_t)e0 * per_s, q_t + (int64_t)e0 * per_q, s_t + (int64_t)e0 * per_s, pow2,
+                           q_fm ? q_fm + (int64_t)e0 * per_q : nullptr, q_t_fm ? q_t_fm + (int64_t)e0 * per_q : nullptr);
         int rc = pf8_check_launch(__func__);
         if (rc) return rc;
     }

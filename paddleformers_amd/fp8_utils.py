@@ -154,7 +154,25 @@ def cache_fp8_weight(weight, quant_transpose=None):
         raise ValueError("quant_transpose must be either True, False or None.")
 
 
-def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_transpose=None, using_pow2_scale=False):
+def _fm_wanted(fragment_major, using_pow2_scale, R, C):
+    """Which of the two orientations of a [R, C] weight (q: rows = R, q_t: rows = C) get a fragment-major copy next to
+    the cache: those whose shape the fragment-major GEMMs take.  None = wherever the node would make one on first use
+    (fp32 scales; with power-of-two scales its GEMMs read the plain bytes)."""
+    if fragment_major is None:
+        fragment_major = not using_pow2_scale
+    if not fragment_major:
+        return (False, False)
+    return (deep_gemm.fragment_major_supported(128, R, C), deep_gemm.fragment_major_supported(128, C, R))
+
+
+def _attach_fragment_major(weight_obj, name, source, fm_bytes, E):
+    """Files a fragment-major copy made by the quantizer where `_cache_derived` looks for it."""
+    if fm_bytes is not None:
+        shape = (E, source.shape[0] // E, source.shape[1])
+        setattr(weight_obj, name + "_fragment_major", (source, source._version, deep_gemm.FragmentMajor(fm_bytes.view(shape), shape)))
+
+
+def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_transpose=None, using_pow2_scale=False, fragment_major=None):
     """DeepseekV2MoE.fp8_quant_weight (cli/train/deepseek_v3_pretrain/modeling.py:506-567), the body
     FP8QuantWeightCallback.on_step_begin runs once per optimizer step: attach the stacked FP8 copies
     of the expert weights to the first weight of each list (batch mode) or to every weight.
@@ -162,7 +180,9 @@ def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_tra
     quant_transpose None caches both orientations; here they come from one read of the weights
     (`fused_stack_quant_both`) instead of two passes.  Weights that already carry a cache are left
     alone, as in the reference.  using_pow2_scale (for `use_ue8m0`, transformers/configuration_utils.py:454-459)
-    rounds every scale up to a power of two and marks the cache so."""
+    rounds every scale up to a power of two and marks the cache so.  fragment_major (with quant_transpose None): the
+    same pass writes the fragment-major copies the node's GEMMs read (None = exactly where the node would otherwise
+    make them on first use, one more pass over each cached weight)."""
 
     def quantize_weights(weight_list, weight_obj=None):
         if weight_obj is None:
@@ -170,9 +190,12 @@ def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_tra
         if hasattr(weight_obj, "fp8_weight_stacked") or hasattr(weight_obj, "fp8_weight_stacked_transpose"):
             return
         if quant_transpose is None:
-            q, s, qt, st = F8.fused_stack_quant_both(weight_list, using_pow2_scale=using_pow2_scale)
+            q, s, qt, st, q_fm, qt_fm = F8.fused_stack_quant_both(
+                weight_list, using_pow2_scale=using_pow2_scale, fragment_major=_fm_wanted(fragment_major, using_pow2_scale, *weight_list[0].shape))
             weight_obj.fp8_weight_stacked, weight_obj.fp8_scale_stacked = q, s
             weight_obj.fp8_weight_stacked_transpose, weight_obj.fp8_scale_stacked_transpose = qt, st
+            _attach_fragment_major(weight_obj, "fp8_weight_stacked", q, q_fm, len(weight_list))
+            _attach_fragment_major(weight_obj, "fp8_weight_stacked_transpose", qt, qt_fm, len(weight_list))
         elif quant_transpose is False:
             weight_obj.fp8_weight_stacked, weight_obj.fp8_scale_stacked = F8.fused_stack_transpose_quant(
                 weight_list, transpose=False, using_pow2_scale=using_pow2_scale)
@@ -196,7 +219,7 @@ def fp8_quant_weight(expert_w1_list, expert_w2_list, batch_mode=False, quant_tra
             quantize_weights([w2])
 
 
-def fp8_quant_weight_all_layers(layers, quant_transpose=None, using_pow2_scale=False):
+def fp8_quant_weight_all_layers(layers, quant_transpose=None, using_pow2_scale=False, fragment_major=None):
     """What FP8QuantWeightCallback.on_step_begin (trainer/trainer_callback.py:725-765) asks for through
     model.fp8_quant_weight(True, ...): the batch-mode caches of every MoE layer, here built by ONE launch
     per weight shape instead of one (or two) per layer and list.  `layers` is a sequence of
@@ -214,9 +237,10 @@ def fp8_quant_weight_all_layers(layers, quant_transpose=None, using_pow2_scale=F
             groups.setdefault((tuple(ws[0].shape), len(ws)), []).append(ws)
     for ((R, Cc), E), lists in groups.items():
         flat = [w for ws in lists for w in ws]
-        q = s = qt = st = None
+        q = s = qt = st = q_fm = qt_fm = None
         if quant_transpose is None:
-            q, s, qt, st = F8.fused_stack_quant_both(flat, using_pow2_scale=using_pow2_scale)
+            q, s, qt, st, q_fm, qt_fm = F8.fused_stack_quant_both(flat, using_pow2_scale=using_pow2_scale,
+                                                                  fragment_major=_fm_wanted(fragment_major, using_pow2_scale, R, Cc))
         elif quant_transpose is False:
             q, s = F8.fused_stack_transpose_quant(flat, transpose=False, using_pow2_scale=using_pow2_scale)
         else:
@@ -226,9 +250,14 @@ def fp8_quant_weight_all_layers(layers, quant_transpose=None, using_pow2_scale=F
             if q is not None:
                 w0.fp8_weight_stacked = q[i * E * R:(i + 1) * E * R]
                 w0.fp8_scale_stacked = s[i * E * R // 128:(i + 1) * E * R // 128]
+                if q_fm is not None:      # 64-row panels are contiguous in the fragment-major order: a layer's rows are a slice of it
+                    _attach_fragment_major(w0, "fp8_weight_stacked", w0.fp8_weight_stacked, q_fm[i * E * R:(i + 1) * E * R], E)
             if qt is not None:
                 w0.fp8_weight_stacked_transpose = qt[i * E * Cc:(i + 1) * E * Cc]
                 w0.fp8_scale_stacked_transpose = st[i * E * Cc // 128:(i + 1) * E * Cc // 128]
+                if qt_fm is not None:
+                    _attach_fragment_major(w0, "fp8_weight_stacked_transpose", w0.fp8_weight_stacked_transpose,
+                                           qt_fm[i * E * Cc:(i + 1) * E * Cc], E)
             w0.fp8_scale_is_pow2 = bool(using_pow2_scale)
 
 

@@ -261,12 +261,15 @@ def fused_stack_transpose_quant(weight_list: Sequence[torch.Tensor], transpose: 
     return q, s
 
 
-def fused_stack_quant_both(weight_list: Sequence[torch.Tensor], using_pow2_scale: bool = False):
+def fused_stack_quant_both(weight_list: Sequence[torch.Tensor], using_pow2_scale: bool = False, fragment_major=False):
     """Both orientations of `fused_stack_transpose_quant` from one read of the weights.
 
     Returns (q, s, q_t, s_t) equal to `fused_stack_transpose_quant(ws, False)` +
     `fused_stack_transpose_quant(ws, True)`: the pair DeepseekV2MoE.fp8_quant_weight builds with two
     calls when quant_transpose is None (cli/train/deepseek_v3_pretrain/modeling.py:521-534).
+    fragment_major: True, or a pair of flags for (q, q_t): the same pass also writes the fragment-major copies
+    the `*_fm` GEMMs read, and the result is (q, s, q_t, s_t, q_fm, q_t_fm) with None where none was asked for;
+    each equals `pf8_weight_to_fragment_major` of its plain tensor to the byte.
     """
     if len(weight_list) == 0:
         raise ValueError("weight_list is empty")
@@ -286,8 +289,15 @@ def fused_stack_quant_both(weight_list: Sequence[torch.Tensor], using_pow2_scale
     qt = torch.empty((E * Cc, R), dtype=FP8, device=dev)
     st = torch.empty((E * Cc // 128, R // 128), dtype=torch.float32, device=dev)
     ptrs = (C.c_void_p * E)(*[w.data_ptr() for w in ws])
+    want_fm = (bool(fragment_major),) * 2 if isinstance(fragment_major, bool) else tuple(bool(f) for f in fragment_major)
+    if any(want_fm):
+        q_fm = torch.empty_like(q) if want_fm[0] else None
+        qt_fm = torch.empty_like(qt) if want_fm[1] else None
+        _lib.call("pf8_stack_quant_both_fm", ptrs, E, R, Cc, _p(q), _p(s), _p(qt), _p(st), _p(q_fm), _p(qt_fm),
+                  int(bool(using_pow2_scale)), _stream())
+        return q, s, qt, st, q_fm, qt_fm
     _lib.call("pf8_stack_quant_both", ptrs, E, R, Cc, _p(q), _p(s), _p(qt), _p(st), int(bool(using_pow2_scale)), _stream())
-    return q, s, qt, st
+    return (q, s, qt, st, None, None) if not isinstance(fragment_major, bool) else (q, s, qt, st)
 
 
 # ---------------------------------------------------------------------------------------------

@@ -564,7 +564,7 @@ def test_moe_node_reads_fragment_major_copies_of_the_cached_weights():
     dout = G.bf16_normal((sum(rows), H), seed=42, std=1e-3)
     tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
     tx, tdo = G.to_torch_bf16(x), G.to_torch_bf16(dout)
-    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True)
+    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True, fragment_major=False)
 
     def run(fragment_major):
         for e in experts:
@@ -594,8 +594,69 @@ def test_moe_node_reads_fragment_major_copies_of_the_cached_weights():
             e.w1.mul_(2.0)
     for name in ("fp8_weight_stacked", "fp8_scale_stacked", "fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose"):
         delattr(w0, name)
-    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True)
+    U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True, fragment_major=False)
     fresh_plain, fresh_fm = run(False), run(True)
     assert torch.equal(fresh_plain[0].view(torch.int16), fresh_fm[0].view(torch.int16))
     assert not torch.equal(fresh_fm[0].view(torch.int16), fm[0].view(torch.int16))
     assert w0.fp8_weight_stacked_transpose_fragment_major is not kept
+
+
+@pytest.mark.parametrize("all_layers", [False, True])
+def test_weight_requantization_writes_the_fragment_major_copies_the_node_reads(monkeypatch, all_layers):
+    """fp8_quant_weight (the per-optimizer-step caller, modeling.py:506-567) makes the fragment-major copies in the pass that
+    quantizes the weights: the node's GEMMs then run no re-ordering pass, the copies are the bytes that pass would have
+    written, and the results are those of a cache without them."""
+    from paddleformers_amd import deep_gemm as dg
+    from paddleformers_amd import fp8_utils as U
+
+    E, H, I = 3, 512, 384
+    rows = [256, 0, 384]
+    _, _, experts, x, probs = _make(E, H, I, rows, seed=47)
+    dout = G.bf16_normal((sum(rows), H), seed=48, std=1e-3)
+    tp = torch.from_numpy(probs).cuda().unsqueeze(-1)
+    tx, tdo = G.to_torch_bf16(x), G.to_torch_bf16(dout)
+    names = ("fp8_weight_stacked", "fp8_scale_stacked", "fp8_weight_stacked_transpose", "fp8_scale_stacked_transpose")
+
+    def quantize(**kw):
+        for w in (experts[0].w1, experts[0].w2):
+            for name in names + tuple(n + "_fragment_major" for n in names):
+                if hasattr(w, name):
+                    delattr(w, name)
+        if all_layers:
+            U.fp8_quant_weight_all_layers([([e.w1 for e in experts], [e.w2 for e in experts])], **kw)
+        else:
+            U.fp8_quant_weight([e.w1 for e in experts], [e.w2 for e in experts], batch_mode=True, **kw)
+
+    def run():
+        for e in experts:
+            e.w1.main_grad = None
+            e.w2.main_grad = None
+        node = U.FP8GroupGemmMlpFunctionNode(_Map(experts))
+        o3 = node.forward(tx, tp, rows).clone()
+        dx, pg = node.backward(tdo, tp, rows)
+        return o3, dx.clone(), pg.clone()
+
+    quantize(fragment_major=False)
+    lazy = run()
+    made_lazily = {n: getattr(experts[0].w1, n + "_fragment_major")[2].data.clone() for n in ("fp8_weight_stacked", "fp8_weight_stacked_transpose")}
+    quantize()                                        # default: fp32 scales -> the copies come with the cache
+    calls = []
+    real = dg.to_fragment_major
+    monkeypatch.setattr(dg, "to_fragment_major", lambda w: calls.append(tuple(w.shape)) or real(w))
+    w0, v0 = experts[0].w1, experts[0].w2
+    for w in (w0, v0):
+        for n in ("fp8_weight_stacked", "fp8_weight_stacked_transpose"):
+            slot = getattr(w, n + "_fragment_major")
+            assert slot[0] is getattr(w, n) and isinstance(slot[2], dg.FragmentMajor)
+            assert torch.equal(slot[2].data.view(torch.uint8), real(getattr(w, n).view(slot[2].shape)).data.view(torch.uint8))
+    for n, t in made_lazily.items():
+        assert torch.equal(getattr(w0, n + "_fragment_major")[2].data.view(torch.uint8), t.view(torch.uint8))
+    eager = run()
+    assert calls == []
+    for a, b in zip(lazy, eager):
+        assert torch.equal(a.view(torch.int16) if a.dtype == torch.bfloat16 else a, b.view(torch.int16) if b.dtype == torch.bfloat16 else b)
+    # power-of-two scales (use_ue8m0): the node's GEMMs read the plain bytes, no copy is made unless asked for
+    quantize(using_pow2_scale=True)
+    assert not hasattr(w0, "fp8_weight_stacked_fragment_major")
+    quantize(using_pow2_scale=True, fragment_major=True)
+    assert hasattr(w0, "fp8_weight_stacked_fragment_major")

@@ -254,6 +254,26 @@ def test_fused_stack_quant_both_equals_two_calls(F):
     _scales_same(st.cpu().numpy(), est, "stacked transposed scales")
 
 
+@pytest.mark.parametrize("want", [(True, True), (True, False), (False, True)])
+def test_fused_stack_quant_both_writes_fragment_major_copies(F, want):
+    """The copies made in the quantizer's pass are the bytes the re-ordering pass makes of its plain outputs."""
+    from paddleformers_amd import deep_gemm as dg
+
+    E, R, C = 3, 256, 384
+    ws = [G.to_torch_bf16(G.bf16_normal((R, C), seed=320 + e, std=0.02, outlier_frac=1e-3, outlier_scale=50.0)) for e in range(E)]
+    q0, s0, qt0, st0 = F.fused_stack_quant_both(ws)
+    q, s, qt, st, q_fm, qt_fm = F.fused_stack_quant_both(ws, fragment_major=want)
+    for a, b in ((q, q0), (qt, qt0)):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    assert torch.equal(s, s0) and torch.equal(st, st0)
+    assert (q_fm is not None, qt_fm is not None) == want
+    if q_fm is not None:
+        assert torch.equal(q_fm.view(torch.uint8).view(E, R, C), dg.to_fragment_major(q.view(E, R, C)).data.view(torch.uint8))
+    if qt_fm is not None:
+        assert torch.equal(qt_fm.view(torch.uint8).view(E, C, R), dg.to_fragment_major(qt.view(E, C, R)).data.view(torch.uint8))
+    assert F.fused_stack_quant_both(ws, fragment_major=(False, False))[4:] == (None, None)
+
+
 def test_fp8_quant_weight_caches_what_fused_stack_quant_reads():
     """The per-step requantization caller (modeling.py:506-567): batch mode attaches both
     orientations to expert 0's weights, and fused_stack_quant then serves them from the cache."""
