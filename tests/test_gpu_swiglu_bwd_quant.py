@@ -30,19 +30,21 @@ def _u8(t):
     return t.view(torch.uint8) if t.dtype == torch.float8_e4m3fn else t
 
 
-@pytest.mark.parametrize("I,rows,pow2_rows,ue8m0", [
-    (128, [128], False, False),
-    (256, [256, 0, 128, 384], True, False),
-    (384, [128] * 5 + [0, 640], True, True),
-    (1408, [512, 0, 1024, 128], True, True),
+@pytest.mark.parametrize("I,rows,pow2_rows,ue8m0,pow2_t", [
+    (128, [128], False, False, True),
+    (256, [256, 0, 128, 384], True, False, True),
+    (384, [128] * 5 + [0, 640], True, True, True),
+    (1408, [512, 0, 1024, 128], True, True, True),
+    (256, [384, 128], False, False, False),          # exact scales (amax / 448) in both directions
+    (384, [256, 256], True, False, False),
 ])
-def test_quantized_forms_equal_the_chain_of_separate_operators(I, rows, pow2_rows, ue8m0):
+def test_quantized_forms_equal_the_chain_of_separate_operators(I, rows, pow2_rows, ue8m0, pow2_t):
     from paddleformers_amd import functional as F8
 
     o1, do2, probs = _inputs(I, rows, seed=7 * I + len(rows))
     M = sum(rows)
     to1, tdo2, tp = G.to_torch_bf16(o1), G.to_torch_bf16(do2), torch.from_numpy(probs).cuda()
-    q, s, qt, st, oqt, ost, pg = F8.swiglu_weighted_bwd_quant(to1, tdo2, tp, rows, pow2_rows, True, ue8m0)
+    q, s, qt, st, oqt, ost, pg = F8.swiglu_weighted_bwd_quant(to1, tdo2, tp, rows, pow2_rows, pow2_t, ue8m0)
     # the oracle's chain
     edo1, epg, eo2s = O.swiglu_weighted_bwd(o1, do2, probs)
     eq, es = O.quant_1x128(edo1, 1, pow2=pow2_rows)
@@ -52,7 +54,7 @@ def test_quantized_forms_equal_the_chain_of_separate_operators(I, rows, pow2_row
     else:
         assert np.array_equal(s.cpu().numpy().view(np.uint32), es.view(np.uint32))
     for name, got_q, got_s, src, K in (("do1", qt, st, edo1, 2 * I), ("o2_s", oqt, ost, eo2s, I)):
-        eqs, ess = O.transpose_split_quant(src, None, rows, True)
+        eqs, ess = O.transpose_split_quant(src, None, rows, pow2_t)
         for e, r in enumerate(rows):
             assert tuple(got_q[e].shape) == (K, r) and tuple(got_s[e].shape) == (r // 128, K)
             if r:
@@ -63,8 +65,8 @@ def test_quantized_forms_equal_the_chain_of_separate_operators(I, rows, pow2_row
     assert np.all(np.abs(pg.cpu().numpy() - epg) <= PG_TOL * terms + 1e-30)
     # the library's own chain
     do1, pg0, o2s = F8.fused_swiglu_weighted_bwd(to1, tdo2, tp)
-    q0, s0, qt0, st0 = F8.quant_and_transpose_split(do1, rows, pow2_rows, True, ue8m0_scale=ue8m0)
-    oqt0, ost0 = F8.fused_transpose_split_quant(o2s, None, rows, True)
+    q0, s0, qt0, st0 = F8.quant_and_transpose_split(do1, rows, pow2_rows, pow2_t, ue8m0_scale=ue8m0)
+    oqt0, ost0 = F8.fused_transpose_split_quant(o2s, None, rows, pow2_t)
     assert torch.equal(_u8(q), _u8(q0)) and torch.equal(s, s0)
     for a, b in ((qt, qt0), (st, st0), (oqt, oqt0), (ost, ost0)):
         assert torch.equal(_u8(a.buf), _u8(b.buf))
