@@ -310,6 +310,11 @@ class ExpertsGroupGemmContiguousNode:
         self.is_split_group_gemm = has_config(self.fp8_fused_ops_configs, "split_group_gemm")
         self.group = group
         self.name = name
+        # backward quantizes out_grad twice (row-wise for the dgrad GEMM, transposed per expert for the weight gradient)
+        # and do1 and o2_s right after the SwiGLU backward has written them; with this set the first pair comes from
+        # one read of out_grad and the SwiGLU backward writes only the quantized forms (same bytes and scales as the
+        # reference's sequence; probs_grad summed per 128-column tile).  False = the reference's sequence of calls.
+        self.fuse_bwd_quant = True
 
     def reset_status(self):
         self.tokens_per_expert = None
@@ -374,12 +379,22 @@ class ExpertsGroupGemmContiguousNode:
         self._grouped(o2_fp8, o2_scale, w2_quant, w2_scale, o3)
         return o3, unzipped_probs
 
-    def bwd_down_input(self, expert_w2, unzipped_grad, o1):
-        """fp8_utils.py:1019-1094: (do1 [M, 2I], o2_s [M, I], probs_grad [M])."""
+    def bwd_down_input(self, expert_w2, unzipped_grad, o1, quantized=False):
+        """fp8_utils.py:1019-1094: (do1 [M, 2I], o2_s [M, I], probs_grad [M]).  unzipped_grad: bf16, or its row-wise
+        (fp8, scale [H/128, M]) pair.  quantized: do1 comes back as ((fp8, scale [2I/128, M]), (fp8_t list, scale_t list))
+        and o2_s as (fp8_t list, scale_t list), the forms bwd_gate_up_input and the weight gradients take."""
         bw_w2_quant, bw_w2_scale = _quant_weights(expert_w2, False, self._stack_quant())
-        g_fp8, g_scale = F8.fp8_quant_blockwise(unzipped_grad, quant_method="1x128", input_transpose=False, output_scale_transpose=True)
-        do2_s = torch.empty((g_fp8.shape[0], bw_w2_quant.shape[1]), dtype=unzipped_grad.dtype, device=unzipped_grad.device)
+        if isinstance(unzipped_grad, tuple):
+            g_fp8, g_scale = unzipped_grad
+        else:
+            g_fp8, g_scale = F8.fp8_quant_blockwise(unzipped_grad, quant_method="1x128", input_transpose=False, output_scale_transpose=True)
+        do2_s = torch.empty((g_fp8.shape[0], bw_w2_quant.shape[1]), dtype=o1.dtype, device=o1.device)
         self._grouped(g_fp8, g_scale.T, bw_w2_quant, bw_w2_scale, do2_s)
+        if quantized:
+            pow2 = has_config(self.fp8_fused_ops_configs, "transpose_split_quant")
+            d_fp8, d_scale, d_t, d_ts, o_t, o_ts, probs_grad = F8.swiglu_weighted_bwd_quant(
+                o1, do2_s, self.unzipped_probs.squeeze(-1), self.tokens_per_expert, False, pow2)
+            return ((d_fp8, d_scale), (d_t, d_ts)), (o_t, o_ts), probs_grad
         do1, probs_grad, o2_s = F8.fused_swiglu_weighted_bwd(o1, do2_s, self.unzipped_probs.squeeze(-1))
         return do1, o2_s, probs_grad
 
@@ -390,8 +405,11 @@ class ExpertsGroupGemmContiguousNode:
     def bwd_gate_up_input(self, do1, expert_w1):
         """fp8_utils.py:1100-1155: dx [M, H]."""
         bw_w1_quant, bw_w1_scale = _quant_weights(expert_w1, False, self._stack_quant())
-        do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, quant_method="1x128", input_transpose=False, output_scale_transpose=True)
-        dx = torch.empty((do1_fp8.shape[0], bw_w1_quant.shape[1]), dtype=torch.bfloat16, device=do1.device)
+        if isinstance(do1, tuple):              # already quantized row-wise: (fp8, scale [2I/128, M])
+            do1_fp8, do1_scale = do1
+        else:
+            do1_fp8, do1_scale = F8.fp8_quant_blockwise(do1, quant_method="1x128", input_transpose=False, output_scale_transpose=True)
+        dx = torch.empty((do1_fp8.shape[0], bw_w1_quant.shape[1]), dtype=torch.bfloat16, device=do1_fp8.device)
         self._grouped(do1_fp8, do1_scale.T, bw_w1_quant, bw_w1_scale, dx)
         return dx
 
@@ -405,8 +423,9 @@ class ExpertsGroupGemmContiguousNode:
         plain scales and splits the scales per expert: the same values as the per-expert kernel without
         power-of-two scales, since every segment is a multiple of 128 rows."""
         pow2 = has_config(self.fp8_fused_ops_configs, "transpose_split_quant")
-        a_t, sa_t = self.fused_transpose_split_quant(a, self.tokens_per_expert, pow2)
-        b_t, sb_t = self.fused_transpose_split_quant(b, self.tokens_per_expert, pow2)
+        # an operand handed in as (fp8_t list, scale_t list) was transposed and quantized (with this switch's scales) already
+        a_t, sa_t = a if isinstance(a, tuple) else self.fused_transpose_split_quant(a, self.tokens_per_expert, pow2)
+        b_t, sb_t = b if isinstance(b, tuple) else self.fused_transpose_split_quant(b, self.tokens_per_expert, pow2)
         FP8GroupGemmMlpFunctionNode._expert_wgrads(a_t, sa_t, b_t, sb_t, expert_w, pow2)
 
     def bwd_down_weight(self, do3, o2, expert_w2):
@@ -457,7 +476,19 @@ class ExpertsGroupGemmContiguousNode:
             o1 = self.fwd_gate_up(None if self.dequant_input else self.input, expert_w1, len(expert_w1), self.tokens_per_expert)
         else:
             o1 = self.o1
-        do1, o2_s, probs_grad = self.bwd_down_input(expert_w2, out_grad, o1)
+        rows = [int(t) for t in self.tokens_per_expert]
+        fuse = (self.fuse_bwd_quant and not self.is_split_group_gemm and len(rows) <= 256 and all(r % 128 == 0 for r in rows)
+                and o1.shape[1] % 256 == 0 and out_grad.dtype == torch.bfloat16 and out_grad.shape[1] % 128 == 0)
+        do1_rows = do1_t = None
+        if fuse:
+            pow2 = has_config(self.fp8_fused_ops_configs, "transpose_split_quant")
+            g_fp8, g_scale, g_t, g_ts = F8.quant_and_transpose_split(out_grad, rows, False, pow2)
+            (do1_rows, do1_t), o2_s, probs_grad = self.bwd_down_input(expert_w2, (g_fp8, g_scale), o1, quantized=True)
+            out_grad = (g_t, g_ts)
+        else:
+            do1, o2_s, probs_grad = self.bwd_down_input(expert_w2, out_grad, o1)
+            do1_rows = do1_t = do1
+            del do1
         del o1
         if not self.recompute_fwd_gate_up:
             self.o1 = None
@@ -468,21 +499,21 @@ class ExpertsGroupGemmContiguousNode:
             input_x = self.input
         task = None
         if a2a_async_fn is None:
-            self.bwd_gate_up_weight(do1, input_x, expert_w1)
+            self.bwd_gate_up_weight(do1_t, input_x, expert_w1)
             del input_x
             if not self.dequant_input:
                 self.input = None
-            dx = self.bwd_gate_up_input(do1, expert_w1)
-            del do1
+            dx = self.bwd_gate_up_input(do1_rows, expert_w1)
+            del do1_rows, do1_t
             self.bwd_down_weight(out_grad, o2_s, expert_w2)
         else:
-            dx = self.bwd_gate_up_input(do1, expert_w1)
+            dx = self.bwd_gate_up_input(do1_rows, expert_w1)
             dx, task = a2a_async_fn(dx)
-            self.bwd_gate_up_weight(do1, input_x, expert_w1)
+            self.bwd_gate_up_weight(do1_t, input_x, expert_w1)
             del input_x
             if not self.dequant_input:
                 self.input = None
-            del do1
+            del do1_rows, do1_t
             self.bwd_down_weight(out_grad, o2_s, expert_w2)
             task.wait()
         self.reset_status()

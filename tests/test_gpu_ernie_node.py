@@ -238,11 +238,13 @@ def _ernie_experts(w1, w2):
     return ex
 
 
+@pytest.mark.parametrize("fuse_bwd", [True, False])
 @pytest.mark.parametrize("dequant_input", [False, True])
 @pytest.mark.parametrize("recompute", [False, True])
-def test_ernie_contiguous_node_equals_the_transformers_node_when_every_switch_is_on(dequant_input, recompute):
+def test_ernie_contiguous_node_equals_the_transformers_node_when_every_switch_is_on(dequant_input, recompute, fuse_bwd):
     """With stack_quant, spaq, swiglu_probs_bwd and transpose_split_quant the two classes ask for the same
-    operators with the same arguments: identical outputs and gradients."""
+    operators with the same arguments: identical outputs and gradients, with the backward's quantizations fused into
+    their producers (both classes' default) and as the reference's sequence of calls."""
     from paddleformers_amd.ernie_fp8_utils import ExpertsGroupGemmContiguousNode
     from paddleformers_amd.fp8_utils import FP8GroupGemmMlpFunctionNode
 
@@ -251,6 +253,7 @@ def test_ernie_contiguous_node_equals_the_transformers_node_when_every_switch_is
     w1, w2, x, probs, dout = _contig_case(E, H, I, rows, seed=71)
     ex = _ernie_experts(w1, w2)
     node = ExpertsGroupGemmContiguousNode(_Map(ex, dict(_ALL_FUSED)), recompute_fwd_gate_up=recompute, dequant_input=dequant_input)
+    node.fuse_bwd_quant = fuse_bwd
     tp = torch.from_numpy(probs).cuda()
     o3 = node.forward(G.to_torch_bf16(x), tp, rows, rows)
     assert tuple(node.unzipped_probs.shape) == (sum(rows), 1)
@@ -264,7 +267,7 @@ def test_ernie_contiguous_node_equals_the_transformers_node_when_every_switch_is
         t2.main_grad = None
         tex.append(_W(t1, t2))
     ref = FP8GroupGemmMlpFunctionNode(_TMap(tex), recompute_fwd_gate_up=recompute)
-    ref.fuse_bwd_swiglu_quant = False       # the SwiGLU backward as the operator both classes name (probs_grad summed per row)
+    ref.fuse_bwd_quant = ref.fuse_bwd_swiglu_quant = fuse_bwd
     r3 = ref.forward(G.to_torch_bf16(x), tp.unsqueeze(-1), rows)
     rdx, rpg = ref.backward(G.to_torch_bf16(dout), tp.unsqueeze(-1), rows)
     assert torch.equal(o3, r3) and torch.equal(dx, rdx) and torch.equal(pg, rpg)
@@ -329,6 +332,33 @@ def test_ernie_contiguous_node_against_fp32_moe(cfg):
         if r:
             assert G.rel_fro(ex[e].up_gate_proj.weight.main_grad.cpu().numpy(), w1t[e].grad.numpy()) < 0.08
             assert G.rel_fro(ex[e].down_proj.weight.main_grad.cpu().numpy(), w2t[e].grad.numpy()) < 0.08
+
+
+@pytest.mark.parametrize("cfg", [{}, dict(_ALL_FUSED)])
+@pytest.mark.parametrize("dequant_input", [False, True])
+def test_ernie_contiguous_node_backward_with_fused_quantizations_is_the_reference_sequence(cfg, dequant_input):
+    """One read of out_grad for its two quantizations and a SwiGLU backward that writes quantized forms only, against the
+    reference's sequence of calls (fp8_utils.py:1345-1436): dx and the weight gradients to the bit, probs_grad (summed in
+    another order) to 1e-5 of its largest entry."""
+    from paddleformers_amd.ernie_fp8_utils import ExpertsGroupGemmContiguousNode
+
+    E, H, I = 3, 512, 384
+    rows = [256, 0, 384]
+    w1, w2, x, probs, dout = _contig_case(E, H, I, rows, seed=91)
+    tp = torch.from_numpy(probs).cuda()
+    res = []
+    for fuse in (False, True):
+        ex = _ernie_experts(w1, w2)
+        node = ExpertsGroupGemmContiguousNode(_Map(ex, dict(cfg)), dequant_input=dequant_input)
+        node.fuse_bwd_quant = fuse
+        node.forward(G.to_torch_bf16(x), tp, rows, rows)
+        dx, pg = node.backward(G.to_torch_bf16(dout))
+        res.append((dx, pg, [e.up_gate_proj.weight.main_grad for e in ex], [e.down_proj.weight.main_grad for e in ex]))
+    a, b = res
+    assert torch.equal(a[0].view(torch.int16), b[0].view(torch.int16))
+    for ga, gb in zip(a[2] + a[3], b[2] + b[3]):
+        assert (ga is None) == (gb is None) and (ga is None or torch.equal(ga, gb))
+    assert float(a[1].abs().max()) > 0 and float((a[1] - b[1]).abs().max()) <= 1e-5 * float(a[1].abs().max())
 
 
 def test_ernie_contiguous_node_zero_rows_and_prequantized_input():
