@@ -215,7 +215,8 @@ int pf8_swiglu_weighted_bwd(const uint16_t* o1, const uint16_t* do2_s, const flo
  * output_scale_transpose, :1073-1079) and transposed per expert for the weight gradient (fused_transpose_split_quant,
  * :1168), o2_s [M,I] transposed per expert (:1115).  One kernel reads o1 [M,2I], do2_s [M,I] (bf16) and probs fp32 [M]
  * and writes only the quantized forms; M = sum of rows_per_expert (HOST array of E multiples of 128, E <= 256).
- * do1_q e4m3 [M,2I]; do1_s fp32 [2I/128,M] (pow2_rows = 0 or 1) or UE8M0 bytes of that shape (pow2_rows = 2);
+ * do1_q e4m3 [M,2I]; do1_s fp32 [M,2I/128] (scale_layout 0) or [2I/128,M] (scale_layout 1), exact (pow2_rows = 0) or
+ * powers of two (1), or UE8M0 bytes [2I/128,M] (pow2_rows = 2, scale_layout 1);
  * do1_q_t / do1_s_t and o2s_q_t / o2s_s_t: the experts' [2I,Me] / [I,Me] blocks and [Me/128,2I] / [Me/128,I] scales
  * packed back to back, as pf8_transpose_split_quant lays them out.  All of these equal, byte for byte, what
  * pf8_quant_and_transpose_split and pf8_transpose_split_quant make of pf8_swiglu_weighted_bwd's outputs.  probs_grad
@@ -223,8 +224,8 @@ int pf8_swiglu_weighted_bwd(const uint16_t* o1, const uint16_t* do2_s, const flo
  * rounding only.  pg_partial: DEVICE scratch of (I/128) x M floats. */
 int pf8_swiglu_weighted_bwd_quant(const uint16_t* o1, const uint16_t* do2_s, const float* probs,
                                   const int64_t* rows_per_expert, int E, int64_t I, uint8_t* do1_q, float* do1_s,
-                                  int pow2_rows, uint8_t* do1_q_t, float* do1_s_t, uint8_t* o2s_q_t, float* o2s_s_t,
-                                  int pow2_t, float* probs_grad, float* pg_partial, pf8_stream_t stream);
+                                  int scale_layout, int pow2_rows, uint8_t* do1_q_t, float* do1_s_t, uint8_t* o2s_q_t,
+                                  float* o2s_s_t, int pow2_t, float* probs_grad, float* pg_partial, pf8_stream_t stream);
 
 /* deep_gemm.fp8_gemm_nt((a, sa), (b, sb), out) -- transformers/fp8_utils.py:278, 368;
  * cli/train/deepseek_v3_pretrain/kernel.py:129-220.  a e4m3 [M,K], sa per sa_layout, b e4m3 [N,K],

@@ -40,7 +40,7 @@ SIGNATURES = {
     "pf8_rms_norm_fwd": [_vp, _vp, C.c_float, _i64, _i64, _vp, _vp, _vp],
     "pf8_rms_norm_bwd": [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _vp],
     "pf8_swiglu_weighted_bwd": [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp],
-    "pf8_swiglu_weighted_bwd_quant": [_vp, _vp, _vp, _vp, _i32, _i64, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp],
+    "pf8_swiglu_weighted_bwd_quant": [_vp, _vp, _vp, _vp, _i32, _i64, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp],
     "pf8_gemm_nt": [_vp, _vp, _i32, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
     "pf8_gemm_nt_1d1d_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp],
     "pf8_gemm_nt_1d1d_f32_pow2": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp],

@@ -596,8 +596,11 @@ __device__ __forceinline__ void pin_words(uint4& w) {
 // column-scaled, transposed per expert (oqt, ost).  Every value takes the arithmetic of k_swiglu_bwd and is rounded to
 // bf16 before it is quantized, so the bytes and scales are those of k_quant_rowcol<true, 1> on the tensors k_swiglu_bwd
 // writes; neither tensor exists in memory here.  probs_grad leaves as one partial sum per row and column tile
-// (pg_part [I/128, M]) that k_sum_row_partials adds up in the order of the tiles.
-__global__ __launch_bounds__(256, 3) void k_swiglu_bwd_quant(const uint16_t* __restrict__ o1, const uint16_t* __restrict__ do2_s,
+// (pg_part [I/128, M]) that k_sum_row_partials adds up in the order of the tiles.  LAYOUT: do1's row scales as [M, 2I/128]
+// (0) or [2I/128, M] (1).
+// (three workgroups per compute unit; the row-major scale stores of LAYOUT 0 need a few registers more than that leaves)
+template <int LAYOUT>
+__global__ __launch_bounds__(256, LAYOUT == 1 ? 3 : 2) void k_swiglu_bwd_quant(const uint16_t* __restrict__ o1, const uint16_t* __restrict__ do2_s,
                                                           const float* __restrict__ probs, int64_t M, int64_t I,
                                                           uint8_t* __restrict__ q, float* __restrict__ s, uint8_t* __restrict__ qt,
                                                           float* __restrict__ st, uint8_t* __restrict__ oqt, float* __restrict__ ost,
@@ -670,8 +673,8 @@ __global__ __launch_bounds__(256, 3) void k_swiglu_bwd_quant(const uint16_t* __r
         // one row at a time: interleaved, the eight rows' temporaries do not fit the register file next to the patches
         __builtin_amdgcn_sched_barrier(0);
     }
-    quant_rowcol_tile<true, 1>(a, tr, tc, M, 2 * I, q, s, qt, st, sp, pow2, true, L, e);
-    quant_rowcol_tile<true, 1>(b, tr, tc + IB, M, 2 * I, q, s, qt, st, sp, pow2, true, L, e);
+    quant_rowcol_tile<true, LAYOUT>(a, tr, tc, M, 2 * I, q, s, qt, st, sp, pow2, true, L, e);
+    quant_rowcol_tile<true, LAYOUT>(b, tr, tc + IB, M, 2 * I, q, s, qt, st, sp, pow2, true, L, e);
     quant_rowcol_tile<true, 1>(o, tr, tc, M, I, nullptr, nullptr, oqt, ost, sp, pow2 & 1, false, L, e);
 }
 
@@ -1073,12 +1076,14 @@ extern "C" int pf8_swiglu_weighted_bwd(const uint16_t* o1, const uint16_t* do2_s
 }
 
 extern "C" int pf8_swiglu_weighted_bwd_quant(const uint16_t* o1, const uint16_t* do2_s, const float* probs, const int64_t* rows_per_expert,
-                                             int E, int64_t I, uint8_t* do1_q, float* do1_s, int pow2_rows, uint8_t* do1_q_t,
+                                             int E, int64_t I, uint8_t* do1_q, float* do1_s, int scale_layout, int pow2_rows, uint8_t* do1_q_t,
                                              float* do1_s_t, uint8_t* o2s_q_t, float* o2s_s_t, int pow2_t, float* probs_grad,
                                              float* pg_partial, pf8_stream_t stream) {
     PF8_REQUIRE(E >= 0 && I >= 0, "negative shape");
     PF8_REQUIRE(I % 128 == 0, "I must be a multiple of 128");
     PF8_REQUIRE(E <= 256, "at most 256 experts per call");
+    PF8_REQUIRE(scale_layout == 0 || scale_layout == 1, "scale_layout must be 0 ([M, 2I/128]) or 1 ([2I/128, M])");
+    PF8_REQUIRE(pow2_rows != 2 || scale_layout == 1, "UE8M0 row scales (pow2_rows 2) are written [2I/128, M] (scale_layout 1)");
     if (E == 0) return PF8_OK;
     PF8_REQUIRE(rows_per_expert, "null pointer");
     SplitArgs sp = {};
@@ -1099,8 +1104,12 @@ extern "C" int pf8_swiglu_weighted_bwd_quant(const uint16_t* o1, const uint16_t*
     // pow2 bits of k_quant_rowcol: 1 = transposed copies, 2 = row-scaled copy, 4 = its scales as UE8M0 bytes [2I/128, M]
     const int pow2_bits = (pow2_t ? 1 : 0) | (pow2_rows ? 2 : 0) | (pow2_rows == 2 ? 4 : 0);
     dim3 grid((unsigned)(((I / 128) * (total / 128) + 7) / 8 * 8)), block(256);
-    hipLaunchKernelGGL(k_swiglu_bwd_quant, grid, block, 0, (hipStream_t)stream, o1, do2_s, probs, total, I, do1_q, do1_s, do1_q_t, do1_s_t,
-                       o2s_q_t, o2s_s_t, pg_partial, sp, pow2_bits);
+    if (scale_layout == 0)
+        hipLaunchKernelGGL(k_swiglu_bwd_quant<0>, grid, block, 0, (hipStream_t)stream, o1, do2_s, probs, total, I, do1_q, do1_s, do1_q_t,
+                           do1_s_t, o2s_q_t, o2s_s_t, pg_partial, sp, pow2_bits);
+    else
+        hipLaunchKernelGGL(k_swiglu_bwd_quant<1>, grid, block, 0, (hipStream_t)stream, o1, do2_s, probs, total, I, do1_q, do1_s, do1_q_t,
+                           do1_s_t, o2s_q_t, o2s_s_t, pg_partial, sp, pow2_bits);
     int rc = pf8_check_launch(__func__);
     if (rc) return rc;
     hipLaunchKernelGGL(k_sum_row_partials, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, pg_partial,

@@ -98,6 +98,9 @@ class ExpertsGroupGemmNode:
         self.tokens_per_expert = None
         self.fp8_fused_ops_configs = custom_map.config.fp8_fused_ops_configs
         self.name = name
+        # backward (with probs): the SwiGLU backward writes do1 and o2_s in the quantized forms their consumers read (one
+        # kernel instead of four, same bytes and scales; probs_grad summed per 128-column tile).  False = the reference's calls.
+        self.fuse_bwd_quant = True
 
     def reset_status(self):
         self.o1 = None
@@ -177,11 +180,18 @@ class ExpertsGroupGemmNode:
         masked_m = self._masked(tokens_per_expert, E, unzipped_grad.device)
         return self._masked_gemm(g_fp8, g_scale, bw_w2_quant, bw_w2_scale, masked_m, expected_m, unzipped_grad.dtype)
 
-    def bwd_down_input(self, expert_w2, unzipped_grad, tokens_per_expert, expected_m):
+    def bwd_down_input(self, expert_w2, unzipped_grad, tokens_per_expert, expected_m, quantized=False):
         """fp8_utils.py:371-439: do2_s = out_grad . w2^T, then the weighted SwiGLU backward.
-        Returns (do1 [E, Mmax, 2I], o2_s [E, Mmax, I], probs_grad [E, Mmax])."""
+        Returns (do1 [E, Mmax, 2I], o2_s [E, Mmax, I], probs_grad [E, Mmax]).  quantized: do1 as ((fp8 [E, Mmax, 2I],
+        scale [E, Mmax, 2I/128]), (fp8_t list, scale_t list)) and o2_s as (fp8_t list, scale_t list), the forms
+        bwd_gate_up_input and the weight gradients take."""
         do2_s = self._dgrad_down(expert_w2, unzipped_grad, tokens_per_expert, expected_m)
         E, Mmax, I = do2_s.shape
+        if quantized:
+            d_fp8, d_scale, d_t, d_ts, o_t, o_ts, probs_grad = F8.swiglu_weighted_bwd_quant(
+                self.o1.reshape(E * Mmax, 2 * I), do2_s.reshape(E * Mmax, I), self.unzipped_probs, [Mmax] * E, False, False,
+                output_scale_transpose=False)
+            return ((d_fp8.reshape(E, Mmax, 2 * I), d_scale.reshape(E, Mmax, -1)), (d_t, d_ts)), (o_t, o_ts), probs_grad.reshape(E, Mmax)
         do1, probs_grad, o2_s = F8.fused_swiglu_weighted_bwd(self.o1.reshape(E * Mmax, 2 * I), do2_s.reshape(E * Mmax, I),
                                                              self.unzipped_probs)
         return do1.reshape(E, Mmax, 2 * I), o2_s.reshape(E, Mmax, I), probs_grad.reshape(E, Mmax)
@@ -201,8 +211,11 @@ class ExpertsGroupGemmNode:
         """fp8_utils.py:498-554: dx [E, Mmax, H] = do1 . w1^T."""
         E = len(expert_w1)
         bw_w1_quant, bw_w1_scale = _quant_weights(expert_w1, False, self._stack_quant())
-        do1_fp8, do1_scale = self._quant_rows(do1.reshape(-1, do1.shape[-1]), E)
-        masked_m = self._masked(tokens_per_expert, E, do1.device)
+        if isinstance(do1, tuple):              # already quantized row-wise: (fp8 [E, Mmax, 2I], scale [E, Mmax, 2I/128])
+            do1_fp8, do1_scale = do1
+        else:
+            do1_fp8, do1_scale = self._quant_rows(do1.reshape(-1, do1.shape[-1]), E)
+        masked_m = self._masked(tokens_per_expert, E, do1_fp8.device)
         return self._masked_gemm(do1_fp8, do1_scale, bw_w1_quant, bw_w1_scale, masked_m, expected_m)
 
     @staticmethod
@@ -211,13 +224,18 @@ class ExpertsGroupGemmNode:
         count are zero in both operands): both operands transposed per expert and 1x128-quantized along
         the rows, then the fp32 weight-gradient GEMM (fp8_utils.py:556-716)."""
         E = len(expert_w)
-        a2, b2 = a.reshape(-1, a.shape[-1]), b.reshape(-1, b.shape[-1])
-        Mmax = a2.shape[0] // E
-        if Mmax % 128 != 0:
-            raise ValueError("the capacity per expert must be a multiple of 128 for the weight-gradient GEMM")
-        rows = [Mmax] * E
-        a_t, sa_t = F8.fused_transpose_split_quant(a2, None, rows, False)
-        b_t, sb_t = F8.fused_transpose_split_quant(b2, None, rows, False)
+
+        def transposed(t):
+            if isinstance(t, tuple):            # (fp8_t list, scale_t list): transposed and quantized per expert already
+                return t
+            t2 = t.reshape(-1, t.shape[-1])
+            Mmax = t2.shape[0] // E
+            if Mmax % 128 != 0:
+                raise ValueError("the capacity per expert must be a multiple of 128 for the weight-gradient GEMM")
+            return F8.fused_transpose_split_quant(t2, None, [Mmax] * E, False)
+
+        a_t, sa_t = transposed(a)
+        b_t, sb_t = transposed(b)
         FP8GroupGemmMlpFunctionNode._expert_wgrads(a_t, sa_t, b_t, sb_t, expert_w, False)
 
     def bwd_down_weight(self, out_grad, o2, expert_w2):
@@ -248,11 +266,15 @@ class ExpertsGroupGemmNode:
         weight gradients go to each weight's main_grad (or grad)."""
         expert_w2 = [x.down_proj.weight for x in self.custom_map.experts if x is not None]
         expert_w1 = [x.up_gate_proj.weight for x in self.custom_map.experts if x is not None]
-        do1, o2_s, probs_grad = self.bwd_down_input(expert_w2, out_grad, tokens_per_expert, expected_m)
-        dx = self.bwd_gate_up_input(do1, expert_w1, tokens_per_expert, expected_m)
+        E, Mmax = len(expert_w2), int(numpy.prod(out_grad.shape[:-1])) // max(len(expert_w2), 1)
+        fuse = self.fuse_bwd_quant and 0 < E <= 256 and Mmax > 0 and Mmax % 128 == 0 and self.o1.shape[-1] % 256 == 0
+        do1, o2_s, probs_grad = self.bwd_down_input(expert_w2, out_grad, tokens_per_expert, expected_m, quantized=fuse)
+        do1_rows, do1_t = do1 if fuse else (do1, do1)
+        del do1
+        dx = self.bwd_gate_up_input(do1_rows, expert_w1, tokens_per_expert, expected_m)
         dx = dx.reshape(-1, dx.shape[-1])
         self.bwd_down_weight(out_grad, o2_s, expert_w2)
-        self.bwd_gate_up_weight(do1, self.unzipped_tokens, expert_w1)
+        self.bwd_gate_up_weight(do1_t, self.unzipped_tokens, expert_w1)
         self.reset_status()
         return dx, probs_grad
 

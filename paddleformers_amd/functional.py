@@ -612,13 +612,16 @@ def fused_swiglu_weighted_bwd(o1: torch.Tensor, do2_s: torch.Tensor, probs: torc
 
 
 def swiglu_weighted_bwd_quant(o1: torch.Tensor, do2_s: torch.Tensor, probs: torch.Tensor, tokens_per_expert: Sequence[int],
-                              using_pow2_scale: bool = False, pow_2_scales: bool = True, ue8m0_scale: bool = False):
+                              using_pow2_scale: bool = False, pow_2_scales: bool = True, ue8m0_scale: bool = False,
+                              output_scale_transpose: bool = True):
     """fused_swiglu_weighted_bwd(o1, do2_s, probs) followed by quant_and_transpose_split(do1, tokens_per_expert,
     using_pow2_scale, pow_2_scales, ue8m0_scale) and fused_transpose_split_quant(o2_s, None, tokens_per_expert,
     pow_2_scales) (transformers/fp8_utils.py:1049-1052, then :1073-1079, :1168 and :1115), from one read of o1 and do2_s:
     the bf16 do1 and o2_s are never written.  Returns (do1_q [M,2I], do1_s [2I/128,M], do1_q_t list, do1_s_t list,
     o2s_q_t list, o2s_s_t list, probs_grad [M]); the quantized forms are bit-identical to the separate calls',
-    probs_grad agrees with theirs to the rounding of a sum taken in another order.  At most 256 experts."""
+    probs_grad agrees with theirs to the rounding of a sum taken in another order.  At most 256 experts.
+    output_scale_transpose=False: do1_s comes back [M, 2I/128], as fp8_quant_blockwise(..., output_scale_transpose=False)
+    stores it (not with ue8m0_scale)."""
     for t, n in ((o1, "o1"), (do2_s, "do2_s"), (probs, "probs")):
         _dev(t, n)
     if o1.dim() != 2 or do2_s.dim() != 2 or o1.dtype != torch.bfloat16 or do2_s.dtype != torch.bfloat16:
@@ -640,6 +643,8 @@ def swiglu_weighted_bwd_quant(o1: torch.Tensor, do2_s: torch.Tensor, probs: torc
         raise ValueError("at most 256 experts")
     if ue8m0_scale and not using_pow2_scale:
         raise ValueError("ue8m0_scale goes with using_pow2_scale=True")
+    if ue8m0_scale and not output_scale_transpose:
+        raise ValueError("ue8m0_scale bytes are stored [2I/128, M] (output_scale_transpose=True)")
     probs = probs.reshape(-1).float().contiguous()
     if probs.numel() != M:
         raise ValueError("probs must have one entry per row")
@@ -647,7 +652,7 @@ def swiglu_weighted_bwd_quant(o1: torch.Tensor, do2_s: torch.Tensor, probs: torc
         probs = probs.clone()
     dev = o1.device
     q = torch.empty((M, I2), dtype=FP8, device=dev)
-    s = torch.empty((I2 // 128, M), dtype=torch.uint8 if ue8m0_scale else torch.float32, device=dev)
+    s = torch.empty((I2 // 128, M) if output_scale_transpose else (M, I2 // 128), dtype=torch.uint8 if ue8m0_scale else torch.float32, device=dev)
     q_t = torch.empty((I2 * M,), dtype=FP8, device=dev)
     s_t = torch.empty(((M // 128) * I2,), dtype=torch.float32, device=dev)
     oq_t = torch.empty((I * M,), dtype=FP8, device=dev)
@@ -657,7 +662,7 @@ def swiglu_weighted_bwd_quant(o1: torch.Tensor, do2_s: torch.Tensor, probs: torc
         part = torch.empty((I // 128, M), dtype=torch.float32, device=dev)
         arr = (C.c_int64 * len(rows))(*rows)
         _lib.call("pf8_swiglu_weighted_bwd_quant", _p(o1), _p(do2_s), _p(probs), arr, len(rows), I, _p(q), _p(s),
-                  2 if ue8m0_scale else int(bool(using_pow2_scale)), _p(q_t), _p(s_t), _p(oq_t), _p(os_t), int(bool(pow_2_scales)),
+                  int(bool(output_scale_transpose)), 2 if ue8m0_scale else int(bool(using_pow2_scale)), _p(q_t), _p(s_t), _p(oq_t), _p(os_t), int(bool(pow_2_scales)),
                   _p(pg), _p(part), _stream())
     else:
         pg.zero_()

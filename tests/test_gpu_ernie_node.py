@@ -146,6 +146,32 @@ def test_ernie_node_forward_backward_against_fp32_moe(cfg):
     assert G.rel_fro(g1.cpu().numpy(), 2 * ref_dw1[0].numpy()) < 0.08
 
 
+@pytest.mark.parametrize("cfg", [{"stack_quant": True, "swiglu_probs_bwd": True}, {}])
+def test_ernie_node_backward_with_the_fused_swiglu_backward_is_the_reference_sequence(cfg):
+    """The SwiGLU backward that writes do1 and o2_s in quantized form only (row scales [E, Mmax, 2I/128], exact scales in
+    both directions) against the reference's calls (fp8_utils.py:371-439, 498-716): dx and the weight gradients to the bit,
+    probs_grad to 1e-5 of its largest entry."""
+    from paddleformers_amd.ernie_fp8_utils import ExpertsGroupGemmNode
+
+    E, H, I, Mmax = 3, 512, 384, 256
+    valid = [256, 130, 0]
+    res = []
+    for fuse in (False, True):
+        w1, w2, experts, x, probs, dout = _make(E, H, I, Mmax, valid, seed=49)
+        node = ExpertsGroupGemmNode(experts, _Map(experts, dict(cfg)))
+        node.fuse_bwd_quant = fuse
+        tm = torch.tensor(valid, dtype=torch.int32, device="cuda")
+        node.forward(G.to_torch_bf16(x), torch.from_numpy(probs).cuda(), tm)
+        dx, pg = node.backward(G.to_torch_bf16(dout), tm, None, Mmax)
+        res.append((dx, pg, [e.up_gate_proj.weight.main_grad for e in experts] + [e.down_proj.weight.main_grad for e in experts]))
+    a, b = res
+    assert torch.equal(a[0].view(torch.int16), b[0].view(torch.int16))
+    for ga, gb in zip(a[2], b[2]):
+        assert torch.equal(ga, gb)
+    assert tuple(b[1].shape) == (E, Mmax) and float(a[1].abs().max()) > 0
+    assert float((a[1] - b[1]).abs().max()) <= 1e-5 * float(a[1].abs().max())
+
+
 def test_ernie_node_no_prob_path():
     from paddleformers_amd.ernie_fp8_utils import ExpertsGroupGemmNode
 

@@ -74,6 +74,23 @@ def test_quantized_forms_equal_the_chain_of_separate_operators(I, rows, pow2_row
     assert M == 0 or float(pg.abs().max()) > 0
 
 
+def test_row_scales_in_either_layout():
+    from paddleformers_amd import functional as F8
+
+    I, rows = 256, [128, 0, 384]
+    o1, do2, probs = _inputs(I, rows, seed=9)
+    args = (G.to_torch_bf16(o1), G.to_torch_bf16(do2), torch.from_numpy(probs).cuda(), rows)
+    for pow2 in (False, True):
+        a = F8.swiglu_weighted_bwd_quant(*args, pow2, True)
+        b = F8.swiglu_weighted_bwd_quant(*args, pow2, True, output_scale_transpose=False)
+        assert tuple(b[1].shape) == (sum(rows), 2 * I // 128) and torch.equal(b[1], a[1].t().contiguous())
+        for x, y in zip(a[:1] + a[2:6], b[:1] + b[2:6]):
+            assert torch.equal(_u8(getattr(x, "buf", x)), _u8(getattr(y, "buf", y)))
+        assert torch.equal(a[6], b[6])
+    with pytest.raises(ValueError):
+        F8.swiglu_weighted_bwd_quant(*args, True, True, True, output_scale_transpose=False)
+
+
 def test_probs_grad_does_not_depend_on_how_rows_are_grouped_into_experts():
     """A row's sum is taken over its own 128-column tiles in their order, whatever tile the row sits in."""
     from paddleformers_amd import functional as F8
@@ -117,10 +134,10 @@ def test_c_abi_argument_checks():
     L = _lib.lib()
     rows = (C.c_int64 * 1)(100)
     z = C.c_void_p(0)
-    rc = L.pf8_swiglu_weighted_bwd_quant(z, z, z, rows, 1, 128, z, z, 0, z, z, z, z, 1, z, z, z)
+    rc = L.pf8_swiglu_weighted_bwd_quant(z, z, z, rows, 1, 128, z, z, 1, 0, z, z, z, z, 1, z, z, z)
     assert rc != 0 and b"multiples of 128" in L.pf8_last_error()
     rows = (C.c_int64 * 1)(128)
-    rc = L.pf8_swiglu_weighted_bwd_quant(z, z, z, rows, 1, 128, z, z, 0, z, z, z, z, 1, z, z, z)
+    rc = L.pf8_swiglu_weighted_bwd_quant(z, z, z, rows, 1, 128, z, z, 1, 0, z, z, z, z, 1, z, z, z)
     assert rc != 0 and b"null pointer" in L.pf8_last_error()
-    rc = L.pf8_swiglu_weighted_bwd_quant(z, z, z, rows, 1, 100, z, z, 0, z, z, z, z, 1, z, z, z)
+    rc = L.pf8_swiglu_weighted_bwd_quant(z, z, z, rows, 1, 100, z, z, 1, 0, z, z, z, z, 1, z, z, z)
     assert rc != 0 and b"multiple of 128" in L.pf8_last_error()
